@@ -1,0 +1,193 @@
+/*
+ * kermac_amd.h -- C ABI of libkermac_amd.so, the MI355X (gfx950) implementation
+ * of kermac's fused distance hot path.
+ *
+ * Everything here is plain C: device pointers travel as `const float *`, the
+ * HIP stream as `void *` (a hipStream_t; NULL = the default stream).  All
+ * tensors are fp32 and already resident in device memory.  Launches are
+ * asynchronous on the given stream; no entry point synchronises or allocates.
+ *
+ * Every entry point returns 0 on success.  A non-zero return is one of the
+ * KMC_ERR_* codes below or (values >= 1000) 1000 + a hipError_t /
+ * 2000 + a hiprtcResult; kmc_last_error() then holds a readable message for
+ * the calling thread.
+ *
+ * The citations name the interface in the reference checkout that each entry
+ * point stands in for.
+ */
+#ifndef KERMAC_AMD_H
+#define KERMAC_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KMC_ABI_VERSION 1
+
+enum kmc_status {
+    KMC_OK = 0,
+    KMC_ERR_INVALID_ARGUMENT = 1,   /* bad shape, stride, enum or null pointer */
+    KMC_ERR_UNSUPPORTED_VARIANT = 2,/* descriptor not compiled into the library: JIT it */
+    KMC_ERR_WRONG_DEVICE = 3,       /* the current device is not a gfx950 */
+    KMC_ERR_JIT = 4,                /* hiprtc compilation failed; log in kmc_last_error() */
+    KMC_ERR_HIP_BASE = 1000,
+    KMC_ERR_HIPRTC_BASE = 2000
+};
+
+/* Template-parameter enums of the reference kernels
+ * (include/kermac_internal_common.cuh:41-74).  The numeric values are ABI. */
+enum kmc_inner_operator { KMC_OP_DIFF = 0, KMC_OP_DOT = 1 };
+enum kmc_power_type { KMC_POW_NOOP = 0, KMC_POW_ABS = 1, KMC_POW_SQUARE = 2, KMC_POW_SQRT = 3, KMC_POW_POW = 4 };
+enum kmc_kernel_type { KMC_KERNEL_NONE = 0, KMC_KERNEL_LAPLACE = 1, KMC_KERNEL_GAUSSIAN = 2 };
+enum kmc_norm_type { KMC_NORM_L1 = 0, KMC_NORM_L2 = 1, KMC_NORM_P = 2 };
+/* COL_MAJOR: the row index (m / n) has stride 1, k has stride ld ("K-major
+ * panel", storage a[K,M]).  ROW_MAJOR: k has stride 1, rows have stride ld. */
+enum kmc_majorness { KMC_COL_MAJOR = 0, KMC_ROW_MAJOR = 1 };
+
+enum kmc_flags {
+    /* Use the 32-bit loaders/stores even when the operands are 16-byte aligned
+     * (what the reference does without try_to_align). */
+    KMC_FLAG_FORCE_SCALAR_ACCESS = 1,
+    /* Compute A(m,k) - B(n,k) instead of B(n,k) - A(m,k).  Set by callers that
+     * swapped the operands to obtain a row-major result; only matters for the
+     * sign-sensitive inner powers (NOOP, SQRT). */
+    KMC_FLAG_NEGATE_DIFF = 2
+};
+
+/*
+ * Arguments of the fused pairwise-reduction kernel.  Mirrors, field for field,
+ * the 21 launch arguments of cute_build_kernel
+ * (include/build_a_kernel.cuh:554-566, marshalled at
+ * src/kermac/build_a_kernel.py:378-390) plus the 8 template parameters that the
+ * reference passes in the kernel name (src/kermac/build_a_kernel.py:52-71).
+ *
+ *   C[m + n*c_ld + l*c_bs] =
+ *       kernel_fn( outer( sum_k inner( B(n,k,l) (-|*) A(m,k,l) ) ) )
+ *
+ * A(m,k,l) = a[m*1 + k*a_ld + l*a_bs] when a_majorness == KMC_COL_MAJOR,
+ *            a[m*a_ld + k*1 + l*a_bs] when KMC_ROW_MAJOR; likewise B.
+ * C is always written with m contiguous.  A batch stride of 0 broadcasts.
+ *
+ * Hyper-parameters (inner power, outer power, bandwidth, regularisation) are
+ * either a device pointer read at [l * stride] or, when the pointer is NULL,
+ * the by-value field next to it.
+ */
+typedef struct kmc_build_kernel_params {
+    int32_t inner_operator;     /* enum kmc_inner_operator */
+    int32_t inner_power;        /* enum kmc_power_type */
+    int32_t outer_power;        /* enum kmc_power_type */
+    int32_t kernel_type;        /* enum kmc_kernel_type */
+    int32_t a_majorness;        /* enum kmc_majorness */
+    int32_t b_majorness;
+    int32_t flags;              /* enum kmc_flags */
+    int32_t m, n, k, l;
+    const float *a; int64_t a_ld; int64_t a_bs;
+    const float *b; int64_t b_ld; int64_t b_bs;
+    float *c;       int64_t c_ld; int64_t c_bs;
+    const float *p_inner;        int64_t p_inner_bs;        float p_inner_value;
+    const float *p_outer;        int64_t p_outer_bs;        float p_outer_value;
+    const float *bandwidth;      int64_t bandwidth_bs;      float bandwidth_value;
+    const float *regularization; int64_t regularization_bs; float regularization_value;
+    int32_t regularization_offset_x;
+    int32_t regularization_offset_y;
+    float epsilon;
+} kmc_build_kernel_params;
+
+/* Stands in for launch(stream, config, cute_build_kernel<...>, *args)
+ * (src/kermac/build_a_kernel.py:339-392).  Returns
+ * KMC_ERR_UNSUPPORTED_VARIANT when the (inner_operator, inner_power) pair is
+ * not among the ahead-of-time compiled ones. */
+int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream);
+
+/*
+ * Arguments of the fused kernel-gradient contraction; mirrors the 24 launch
+ * arguments of cute_norm_kernel_gradient (include/p_norm_gradient.cuh:413-422,
+ * marshalled at src/kermac/cdist_grad.py:226-235).
+ *
+ *   E[m + n*e_ld_n + o*e_ld_o + l*e_bs] =
+ *       sum_k C[o*c_ld + k + l*c_bs] * A[m + k*a_ld + l*a_bs]
+ *             * g( D[m + n*d_ld + l*d_bs] - B[n*b_ld + k + l*b_bs] )
+ *   g(x) = copysign(1,x) (L1), x (L2), copysign(1,x)*|x|^(p-1) (P)
+ *
+ * p is a device pointer read at [l * p_bs], or by value when NULL.
+ */
+typedef struct kmc_norm_gradient_params {
+    int32_t norm_type;          /* enum kmc_norm_type */
+    int32_t flags;
+    int32_t m, n, o, k, l;
+    const float *a; int64_t a_ld; int64_t a_bs;   /* [k, m], m contiguous */
+    const float *b; int64_t b_ld; int64_t b_bs;   /* [n, k], k contiguous */
+    const float *c; int64_t c_ld; int64_t c_bs;   /* [o, k], k contiguous */
+    const float *d; int64_t d_ld; int64_t d_bs;   /* [n, m], m contiguous */
+    float *e; int64_t e_ld_n; int64_t e_ld_o; int64_t e_bs; /* [o, n, m], m contiguous */
+    const float *p; int64_t p_bs; float p_value;
+} kmc_norm_gradient_params;
+
+/* Stands in for launch(stream, config, cute_norm_kernel_gradient<NormType>, *args)
+ * (src/kermac/cdist_grad.py:192-237). */
+int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *params, void *stream);
+
+/*
+ * Fused kernel matrix x coefficients:
+ *   out[m*out_ld + o + l*out_bs] = sum_n Kmat(m,n,l) * coef[n*coef_ld + o + l*coef_bs]
+ * where Kmat(m,n,l) is exactly the value kmc_build_kernel would have stored at
+ * C(m,n,l) for `kernel` (its c, c_ld, c_bs fields are ignored).  The m x n
+ * matrix is never written to memory.  The reference has no such kernel
+ * (its run_kernel always materialises out[L,M,N],
+ * src/kermac/build_a_kernel.py:259,378-392); the semantics are those of
+ * run_kernel(...) followed by a matmul with the coefficients.
+ */
+typedef struct kmc_kernel_coefficients_params {
+    kmc_build_kernel_params kernel;
+    int32_t o;                                    /* coefficient columns, 1..64 */
+    const float *coef; int64_t coef_ld; int64_t coef_bs;  /* [n, o], o contiguous */
+    float *out; int64_t out_ld; int64_t out_bs;           /* [m, o], o contiguous */
+} kmc_kernel_coefficients_params;
+
+int kmc_kernel_times_coefficients(const kmc_kernel_coefficients_params *params, void *stream);
+
+/* ---- run-time compilation (stands in for cuda.core Program / ObjectCode:
+ *      src/kermac/module_cache/module_cache.py:13-51, 219-239) ---- */
+
+/* Compile `source` for the current device's architecture with hiprtc.
+ * `headers`/`header_names` are in-memory include files.  On success *code is a
+ * malloc'ed code object of *code_size bytes and lowered_names[i] (malloc'ed
+ * strings) is the mangled symbol of name_expressions[i].  Free with
+ * kmc_jit_free. */
+int kmc_jit_compile(const char *source, const char *source_name,
+                    int n_headers, const char *const *headers, const char *const *header_names,
+                    int n_options, const char *const *options,
+                    int n_names, const char *const *name_expressions,
+                    void **code, size_t *code_size, char **lowered_names);
+void kmc_jit_free(void *ptr);
+
+/* hipModuleLoadData / hipModuleGetFunction / hipModuleUnload. */
+int kmc_module_load(const void *code, size_t code_size, void **module);
+int kmc_module_get_function(void *module, const char *lowered_name, void **function);
+int kmc_module_unload(void *module);
+
+/* Launch a run-time compiled instance of the kernels above.  `function` must be
+ * an instantiation of kmc::build_kernel / kmc::norm_kernel_gradient from the
+ * kernel headers shipped with this library, compiled for load modes
+ * (load_a, load_b) as reported by kmc_build_kernel_load_modes. */
+int kmc_build_kernel_jit(void *function, const kmc_build_kernel_params *params, void *stream);
+/* The loader variants (0..3: col-vec, col-scalar, row-vec, row-scalar) that
+ * kmc_build_kernel would pick for these operands. */
+int kmc_build_kernel_load_modes(const kmc_build_kernel_params *params, int32_t *load_a, int32_t *load_b);
+
+/* ---- misc ---- */
+int kmc_abi_version(void);
+/* Message of the last failing call on this thread ("" if none). */
+const char *kmc_last_error(void);
+/* gcnArchName of `device` (e.g. "gfx950:sramecc+:xnack-") into buf. */
+int kmc_device_arch(int device, char *buf, size_t buf_len);
+/* 1 when (inner_operator, inner_power) is compiled ahead of time. */
+int kmc_build_kernel_has_variant(int32_t inner_operator, int32_t inner_power);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KERMAC_AMD_H */

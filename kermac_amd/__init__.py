@@ -1,0 +1,26 @@
+"""kermac_amd: kermac's fused distance hot path on MI355X (gfx950).
+
+``import kermac_amd as kermac`` gives the reference's names:
+``cdist``, ``cdist_grad``, ``run_kernel``, ``pre_compile_descriptors``,
+``KernelDescriptor``, the enums, the predefined descriptors, ``ModuleCache``
+and the helpers of ``common``.
+"""
+from .common import (Alignment, CudaTimer, FillMode, Majorness, PyTorchStreamWrapper, TensorStats, ceil_div,
+                     merge_batch_size, tensor_stats)
+from .module_cache.module_cache import ModuleCache
+from .build_a_kernel import (InnerOperator, KernelDescriptor, KernelType, PowerType, Symmetry,
+                             kernel_descriptor_l1_norm, kernel_descriptor_l2_norm, kernel_descriptor_laplace_l1,
+                             kernel_descriptor_laplace_l2, kernel_descriptor_mma, kernel_descriptor_p_norm,
+                             pre_compile_descriptors, run_kernel)
+from .cdist import cdist
+from .cdist_grad import cdist_grad
+
+__version__ = "0.1.0"
+
+__all__ = [
+    "cdist", "cdist_grad", "KernelDescriptor", "run_kernel", "PowerType", "InnerOperator", "KernelType",
+    "Symmetry", "kernel_descriptor_laplace_l1", "kernel_descriptor_laplace_l2", "kernel_descriptor_p_norm",
+    "kernel_descriptor_l1_norm", "kernel_descriptor_l2_norm", "kernel_descriptor_mma",
+    "pre_compile_descriptors", "ModuleCache", "CudaTimer", "PyTorchStreamWrapper", "TensorStats",
+    "tensor_stats", "Majorness", "Alignment", "FillMode", "ceil_div", "merge_batch_size",
+]

@@ -1,0 +1,122 @@
+"""Ahead-of-time build of libkermac_amd.so (hipcc, gfx950 only).
+
+Run as ``python -m kermac_amd._build`` or through ``__graft_entry__.build()``.
+The object files and the library stay inside the package directory so that the
+library travels with the source tree; nothing is installed elsewhere.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PACKAGE_DIR = Path(__file__).resolve().parent
+CSRC = PACKAGE_DIR / "csrc"
+OBJ_DIR = PACKAGE_DIR / "_obj"
+LIB_DIR = PACKAGE_DIR / "_lib"
+LIB_PATH = LIB_DIR / "libkermac_amd.so"
+
+ARCH = "gfx950"
+
+# Compiler flags for every translation unit.  Packed-fp32 code generation is
+# switched off on purpose (the last three words are one clang target feature).
+HIPCC_FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-x", "hip",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+# (inner operator, inner power) pairs compiled ahead of time; must match
+# csrc/host/launcher_table.cpp.
+AOT_BUILD_KERNEL_VARIANTS = [(0, 0), (0, 1), (0, 2), (0, 4), (1, 0)]
+
+HOST_SOURCES = [
+    "host/runtime.cpp",
+    "host/build_kernel_launch.cpp",
+    "host/launcher_table.cpp",
+    "host/norm_gradient_launch.cpp",
+    "host/kernel_coefficients_launch.cpp",
+]
+
+
+# Device translation units without per-variant defines.
+EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip"]
+
+
+def _hipcc() -> str:
+    found = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(found):
+        raise RuntimeError("hipcc not found; the library can only be built in a ROCm image")
+    return found
+
+
+def _jobs():
+    jobs = []
+    for rel in HOST_SOURCES:
+        src = CSRC / rel
+        jobs.append((src, OBJ_DIR / (src.stem + ".o"), []))
+    inst = CSRC / "kernels" / "build_kernel_inst.hip"
+    for op, pw in AOT_BUILD_KERNEL_VARIANTS:
+        jobs.append((inst, OBJ_DIR / f"build_kernel_inst_{op}_{pw}.o", [f"-DKMC_INNER_OP={op}", f"-DKMC_INNER_POW={pw}"]))
+    for rel in EXTRA_DEVICE_SOURCES:
+        src = CSRC / rel
+        jobs.append((src, OBJ_DIR / (src.stem + ".o"), []))
+    return jobs
+
+
+def _newest_source_mtime() -> float:
+    newest = 0.0
+    for path in list(CSRC.rglob("*")) + [Path(__file__), PACKAGE_DIR.parent / "include" / "kermac_amd.h"]:
+        if path.is_file():
+            newest = max(newest, path.stat().st_mtime)
+    return newest
+
+
+def build(force: bool = True, verbose: bool = False, workers: int | None = None) -> Path:
+    """Compile every translation unit and link the shared library.
+
+    force=False skips objects that are newer than every source file (used while
+    developing); the default always recompiles.
+    """
+    hipcc = _hipcc()
+    OBJ_DIR.mkdir(exist_ok=True)
+    LIB_DIR.mkdir(exist_ok=True)
+    newest = _newest_source_mtime()
+
+    def compile_one(job):
+        src, obj, defines = job
+        if not force and obj.exists() and obj.stat().st_mtime > newest:
+            return obj
+        cmd = [hipcc, *HIPCC_FLAGS, *defines, "-c", str(src), "-o", str(obj)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {src.name} {defines}:\n{proc.stdout}\n{proc.stderr}")
+        return obj
+
+    workers = workers or min(8, os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        objects = list(pool.map(compile_one, _jobs()))
+
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objects), "-lhiprtc"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build(force="--incremental" not in sys.argv, verbose="-v" in sys.argv)
+    print(path)

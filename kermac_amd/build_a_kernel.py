@@ -1,0 +1,403 @@
+"""Kernel descriptors and the fused kernel-matrix builder ``run_kernel``.
+
+Same public surface as the reference's ``src/kermac/build_a_kernel.py``:
+``InnerOperator``, ``PowerType``, ``KernelType``, ``Symmetry``,
+``KernelDescriptor``, the six predefined descriptors,
+``pre_compile_descriptors`` and ``run_kernel`` with the same positional order,
+defaults, return value and exception types.  The work is done by the gfx950
+kernels in ``csrc/kernels/build_kernel.hpp`` through the C ABI.
+
+View convention (torch.cdist's): ``a`` is ``[L?, M, K]``, ``b`` is ``[L?, N, K]``,
+``out`` is ``[L?, M, N]``.  The fast path is the "K-major panel" storage
+``a_store[K, M]``, ``b_store[K, N]``, ``out_store[N, M]`` passed as ``.T`` views.
+"""
+from __future__ import annotations
+
+from enum import Enum, auto
+from itertools import product
+from typing import Any, List, Optional, Union
+
+import numpy as np
+import torch
+
+from . import _backend
+from .common import (Alignment, Majorness, PyTorchStreamWrapper, TensorStats, ceil_div, merge_batch_size,
+                     tensor_stats)
+from .module_cache.module_cache import ModuleCache, build_kernel_function_name
+
+
+class InnerOperator(Enum):
+    DIFF = auto()
+    DOT = auto()
+
+
+class PowerType(Enum):
+    NOOP = auto()
+    ABS = auto()
+    SQUARE = auto()
+    SQRT = auto()
+    POW = auto()
+
+
+class KernelType(Enum):
+    NONE = auto()
+    LAPLACE = auto()
+    GAUSSIAN = auto()
+
+
+class Symmetry(Enum):
+    NonSymmetric = auto()
+    Symmetric = auto()
+
+
+# Enum member -> C-ABI value (include/kermac_amd.h).
+_INNER_OPERATOR_ABI = {InnerOperator.DIFF: 0, InnerOperator.DOT: 1}
+_POWER_TYPE_ABI = {PowerType.NOOP: 0, PowerType.ABS: 1, PowerType.SQUARE: 2, PowerType.SQRT: 3, PowerType.POW: 4}
+_KERNEL_TYPE_ABI = {KernelType.NONE: 0, KernelType.LAPLACE: 1, KernelType.GAUSSIAN: 2}
+_MAJORNESS_ABI = {Majorness.COL_MAJOR: _backend.COL_MAJOR, Majorness.ROW_MAJOR: _backend.ROW_MAJOR}
+# (majorness, alignment) -> device loader variant (csrc/kernels/device_common.hpp LoadMode).
+_LOAD_MODE = {
+    (Majorness.COL_MAJOR, Alignment.ALIGN_4): 0,
+    (Majorness.COL_MAJOR, Alignment.ALIGN_1): 1,
+    (Majorness.ROW_MAJOR, Alignment.ALIGN_4): 2,
+    (Majorness.ROW_MAJOR, Alignment.ALIGN_1): 3,
+}
+
+
+class KernelDescriptor:
+    """What the fused kernel computes per output element
+    (reference: build_a_kernel.py:39-71):
+
+    ``kernel_type( outer_power( sum_k inner_power( b[n,k] (-|*) a[m,k] ) ) )``
+    """
+
+    def __init__(self, inner_operator, inner_power, outer_power, kernel_type):
+        self._inner_operator = inner_operator
+        self._inner_power = inner_power
+        self._outer_power = outer_power
+        self._kernel_type = kernel_type
+
+    def _replace(self, **fields) -> "KernelDescriptor":
+        current = dict(inner_operator=self._inner_operator, inner_power=self._inner_power,
+                       outer_power=self._outer_power, kernel_type=self._kernel_type)
+        current.update(fields)
+        return KernelDescriptor(**current)
+
+    def _render_function_name(self, majorness_A, majorness_B, align_A, align_B):
+        """Template-id of the device function for this descriptor and operand
+        layout.  Outer power and kernel type are run-time arguments of the gfx950
+        kernel, so they are not part of the name (one binary serves them all)."""
+        return build_kernel_function_name(
+            _INNER_OPERATOR_ABI[self._inner_operator],
+            _POWER_TYPE_ABI[self._inner_power],
+            _LOAD_MODE[(majorness_A, align_A)],
+            _LOAD_MODE[(majorness_B, align_B)],
+        )
+
+    def __repr__(self):
+        return (f"KernelDescriptor({self._inner_operator.name}, {self._inner_power.name}, "
+                f"{self._outer_power.name}, {self._kernel_type.name})")
+
+
+kernel_descriptor_laplace_l1 = KernelDescriptor(
+    inner_operator=InnerOperator.DIFF, inner_power=PowerType.ABS,
+    outer_power=PowerType.NOOP, kernel_type=KernelType.LAPLACE)
+
+kernel_descriptor_laplace_l2 = KernelDescriptor(
+    inner_operator=InnerOperator.DIFF, inner_power=PowerType.SQUARE,
+    outer_power=PowerType.SQRT, kernel_type=KernelType.LAPLACE)
+
+kernel_descriptor_p_norm = KernelDescriptor(
+    inner_operator=InnerOperator.DIFF, inner_power=PowerType.POW,
+    outer_power=PowerType.POW, kernel_type=KernelType.NONE)
+
+kernel_descriptor_l1_norm = KernelDescriptor(
+    inner_operator=InnerOperator.DIFF, inner_power=PowerType.ABS,
+    outer_power=PowerType.NOOP, kernel_type=KernelType.NONE)
+
+kernel_descriptor_l2_norm = KernelDescriptor(
+    inner_operator=InnerOperator.DIFF, inner_power=PowerType.SQUARE,
+    outer_power=PowerType.SQRT, kernel_type=KernelType.NONE)
+
+kernel_descriptor_mma = KernelDescriptor(
+    inner_operator=InnerOperator.DOT, inner_power=PowerType.NOOP,
+    outer_power=PowerType.NOOP, kernel_type=KernelType.NONE)
+
+
+def pre_compile_descriptors(device, descriptors: List[Any], try_to_align=False, debug=False):
+    """Make every operand-layout variant of ``descriptors`` ready before the
+    first call (reference: build_a_kernel.py:121-156).
+
+    Variants that ship ahead-of-time compiled in the library need nothing; the
+    others are compiled with hiprtc in one program and stored in the on-disk
+    kernel cache.  ``try_to_align`` adds the 16-byte-aligned loader variants,
+    as in the reference.
+    """
+    layouts = [(Majorness.ROW_MAJOR, Alignment.ALIGN_1), (Majorness.COL_MAJOR, Alignment.ALIGN_1)]
+    if try_to_align:
+        if debug:
+            print("(Kermac Debug) Because `try_to_align` is set, generating full matrix of alignment conditions")
+        layouts += [(Majorness.COL_MAJOR, Alignment.ALIGN_4), (Majorness.ROW_MAJOR, Alignment.ALIGN_4)]
+
+    function_names = []
+    for descriptor in descriptors:
+        op = _INNER_OPERATOR_ABI[descriptor._inner_operator]
+        power = _POWER_TYPE_ABI[descriptor._inner_power]
+        if _backend.build_kernel_has_variant(op, power):
+            if debug:
+                print(f"(Kermac Debug) {descriptor!r} is compiled ahead of time")
+            continue
+        for (majorness_A, align_A), (majorness_B, align_B) in product(layouts, layouts):
+            name = descriptor._render_function_name(majorness_A, majorness_B, align_A, align_B)
+            if name not in function_names:
+                function_names.append(name)
+    if function_names:
+        ModuleCache(debug).compile_and_cache_functions(device=device, function_names=function_names, debug=debug)
+
+
+def _hyper_parameter(name, value, L, device, require_device):
+    """Normalise a scalar hyper-parameter to (pointer, batch stride, by-value, keepalive).
+
+    A Python number is passed by value in the parameter block (no device
+    allocation, no host-to-device copy).  A tensor must be fp32 on ``device``
+    with 0 dimensions, or 1 dimension of length 1 or L; it is read in place.
+    """
+    if value is None:
+        return 0, 0, 0.0, None
+    if isinstance(value, (float, int)) and not isinstance(value, bool):
+        return 0, 0, float(np.float32(value)), None
+    if not isinstance(value, torch.Tensor):
+        raise TypeError(f"`{name}` must be a float or a torch.Tensor")
+    if value.dtype != torch.float32:
+        raise TypeError(f"`{name}` tensor must have dtype torch.float32")
+    if require_device and (not value.is_cuda or value.device != device):
+        raise ValueError(f"`{name}` tensor must be on the same CUDA device as inputs")
+    if value.dim() > 1:
+        raise ValueError(f"`{name}` tensor must have 0 or 1 dimensions, got {value.dim()}")
+    if value.numel() == 1:
+        return value.data_ptr(), 0, 0.0, value
+    if value.numel() != L:
+        raise ValueError(f"`{name}` tensor has {value.numel()} elements but the batch size is {L}")
+    return value.data_ptr(), value.stride(0), 0.0, value
+
+
+class _LaunchPlan:
+    """Everything needed to launch: the C parameter block, the tensor that will
+    be returned, and references that keep device memory alive until launch."""
+
+    __slots__ = ("params", "out", "keepalive", "swapped", "L", "M", "N", "K")
+
+
+def _plan_run_kernel(
+    kernel_descriptor, a, b, out, p, inner_p, outer_p, bandwidth, epsilon, regularization,
+    regularization_offset_x, regularization_offset_y, try_to_align, require_device=True, allocate_out=True,
+) -> _LaunchPlan:
+    """Validation, batch merge, layout analysis and parameter marshalling of
+    ``run_kernel`` (reference: build_a_kernel.py:174-390), without the launch."""
+    d = kernel_descriptor
+    # Descriptor / hyper-parameter consistency (reference: :174-199).
+    if d._inner_power is PowerType.POW:
+        if p is None and inner_p is None:
+            raise ValueError("'inner_power' 'PowerType' is 'Pow' but 'p' and 'inner_p' is not set")
+    elif p is not None or inner_p is not None:
+        raise ValueError("'inner_power' 'PowerType' is not 'Pow' but 'p' or 'inner_p' is set")
+    if d._outer_power is PowerType.POW:
+        if p is None and outer_p is None:
+            raise ValueError("'outer_power' 'PowerType' is 'Pow' but 'p' and 'outer_p' is not set")
+    elif p is not None or outer_p is not None:
+        raise ValueError("'outer_power' 'PowerType' is not 'Pow' but 'p' or 'outer_p' is set")
+    if d._kernel_type is KernelType.NONE:
+        if bandwidth is not None or epsilon is not None or regularization is not None:
+            raise ValueError("'KernelType' is 'None' but 'bandwidth' or 'epsilon' or 'regularization' is set")
+    elif bandwidth is None:
+        raise ValueError("'KernelType' is not 'None' but 'bandwidth' is not set")
+    if p is not None and inner_p is not None:
+        raise ValueError("'p' is not 'None' but 'inner_p' is also not 'None")
+    if p is not None and outer_p is not None:
+        raise ValueError("'p' is not 'None' but 'outer_p' is also not 'None")
+
+    def as_float(x):
+        return float(x) if isinstance(x, int) and not isinstance(x, bool) else x
+
+    p, inner_p, outer_p = as_float(p), as_float(inner_p), as_float(outer_p)
+    bandwidth, regularization = as_float(bandwidth), as_float(regularization)
+
+    # Batch size: every operand's batch is 1 or the common L (reference: :203-211).
+    L = 1
+    L = merge_batch_size("p", L, p, expected_dims=0, can_be_none=True)
+    L = merge_batch_size("inner_p", L, inner_p, expected_dims=0, can_be_none=True)
+    L = merge_batch_size("outer_p", L, outer_p, expected_dims=0, can_be_none=True)
+    L = merge_batch_size("bandwidth", L, bandwidth, expected_dims=0, can_be_none=True)
+    L = merge_batch_size("regularization", L, regularization, expected_dims=0, can_be_none=True)
+    if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor):
+        raise TypeError("a and b must be PyTorch tensors")
+    if out is not None and not isinstance(out, torch.Tensor):
+        raise TypeError("out must be a PyTorch tensor if provided")
+    L = merge_batch_size("a", L, a, expected_dims=2, can_be_none=False)
+    L = merge_batch_size("b", L, b, expected_dims=2, can_be_none=False)
+    L = merge_batch_size("out", L, out, expected_dims=2, can_be_none=True)
+
+    if a.dtype != torch.float32 or b.dtype != torch.float32:
+        raise TypeError("a and b must have dtype torch.float32")
+    if out is not None and out.dtype != torch.float32:
+        raise TypeError("out must have dtype torch.float32")
+    if require_device:
+        if not a.is_cuda or not b.is_cuda:
+            raise ValueError("a and b must be on a CUDA device")
+        if out is not None and not out.is_cuda:
+            raise ValueError("out must be on a CUDA device")
+    device = a.device
+    if b.device != device:
+        raise ValueError(f"All inputs must be on the same CUDA device: got {[x.device for x in (a, b)]}")
+    if out is not None and out.device != device:
+        raise ValueError(f"out must be on the same CUDA device as inputs: got {out.device}, expected {device}")
+
+    stats_a, stats_b = tensor_stats(a), tensor_stats(b)
+    _, M, K_a = stats_a.shape
+    _, N, K_b = stats_b.shape
+    if K_a != K_b:
+        raise ValueError(f"K dimensions must match: got {K_a} for a and {K_b} for b")
+    K = K_a
+
+    if out is not None:
+        stats_c = tensor_stats(out)
+        L_c, M_c, N_c = stats_c.shape
+        if (M_c, N_c) != (M, N):
+            raise ValueError(f"out must have shape (M={M}, N={N}), got {(M_c, N_c)}")
+        if L_c != L and L != 1:
+            raise ValueError(f"out must have batch dimension (L={L}), got {(L_c)}")
+    elif allocate_out:
+        out = torch.zeros((L, M, N), dtype=torch.float32, device=device)
+        stats_c = tensor_stats(out)
+    else:
+        stats_c = None
+
+    keepalive = [a, b, out]
+
+    # Hyper-parameters.  `p` sets inner = p and outer = 1/p, both rounded to fp32
+    # the way the reference's device-side division does (reference: :281-290).
+    if p is not None:
+        if isinstance(p, float):
+            inner_p = float(np.float32(p))
+            outer_p = float(np.float32(1.0) / np.float32(p)) if p != 0.0 else float("inf")
+        else:
+            if not isinstance(p, torch.Tensor):
+                raise TypeError("`p` must be a float or a torch.Tensor")
+            if p.dtype != torch.float32:
+                raise TypeError("`p` tensor must have dtype torch.float32")
+            if require_device and (not p.is_cuda or p.device != device):
+                raise ValueError("`p` tensor must be on the same CUDA device as inputs")
+            inner_p = p.contiguous()
+            outer_p = 1.0 / inner_p
+    pi_ptr, pi_bs, pi_val, pi_keep = _hyper_parameter("inner_p", inner_p, L, device, require_device)
+    po_ptr, po_bs, po_val, po_keep = _hyper_parameter("outer_p", outer_p, L, device, require_device)
+    bw_ptr, bw_bs, bw_val, bw_keep = _hyper_parameter("bandwidth", bandwidth, L, device, require_device)
+    rg_ptr, rg_bs, rg_val, rg_keep = _hyper_parameter("regularization", regularization, L, device, require_device)
+    keepalive += [pi_keep, po_keep, bw_keep, rg_keep]
+
+    # The kernel writes C with m contiguous.  A row-major out is the transpose of
+    # that, so swap the operands (reference: :323-336).  Unlike the reference the
+    # swap also exchanges the regularisation offsets and keeps the sign of b - a,
+    # so the result does not depend on the layout of `out`.
+    swapped = stats_c is not None and stats_c.majorness is Majorness.ROW_MAJOR
+    off_x, off_y = int(regularization_offset_x), int(regularization_offset_y)
+    if swapped:
+        M, N = N, M
+        a, b = b, a
+        stats_a, stats_b = stats_b, stats_a
+        off_x, off_y = off_y, off_x
+
+    params = _backend.BuildKernelParams()
+    params.inner_operator = _INNER_OPERATOR_ABI[d._inner_operator]
+    params.inner_power = _POWER_TYPE_ABI[d._inner_power]
+    params.outer_power = _POWER_TYPE_ABI[d._outer_power]
+    params.kernel_type = _KERNEL_TYPE_ABI[d._kernel_type]
+    params.a_majorness = _MAJORNESS_ABI[stats_a.majorness]
+    params.b_majorness = _MAJORNESS_ABI[stats_b.majorness]
+    params.flags = _backend.FLAG_NEGATE_DIFF if swapped else 0
+    params.m, params.n, params.k, params.l = M, N, K, L
+    params.a, params.a_ld, params.a_bs = a.data_ptr(), stats_a.leading_dimension_stride, stats_a.batch_stride
+    params.b, params.b_ld, params.b_bs = b.data_ptr(), stats_b.leading_dimension_stride, stats_b.batch_stride
+    if stats_c is not None:
+        params.c, params.c_ld, params.c_bs = out.data_ptr(), stats_c.leading_dimension_stride, stats_c.batch_stride
+    params.p_inner, params.p_inner_bs, params.p_inner_value = pi_ptr, pi_bs, pi_val
+    params.p_outer, params.p_outer_bs, params.p_outer_value = po_ptr, po_bs, po_val
+    params.bandwidth, params.bandwidth_bs, params.bandwidth_value = bw_ptr, bw_bs, bw_val
+    params.regularization, params.regularization_bs, params.regularization_value = rg_ptr, rg_bs, rg_val
+    params.regularization_offset_x, params.regularization_offset_y = off_x, off_y
+    params.epsilon = 1e-5 if epsilon is None else float(epsilon)
+
+    plan = _LaunchPlan()
+    plan.params, plan.out, plan.keepalive, plan.swapped = params, out, keepalive, swapped
+    plan.L, plan.M, plan.N, plan.K = L, M, N, K
+    return plan
+
+
+def _current_stream_for(device: torch.device) -> int:
+    stream = torch.cuda.current_stream()
+    if stream.device != device:
+        raise ValueError(f"cuda stream must be on the same device as the tensors: got {stream.device}, expected {device}")
+    return PyTorchStreamWrapper(stream).handle
+
+
+def run_kernel(
+    kernel_descriptor: KernelDescriptor,
+    a: torch.Tensor,
+    b: torch.Tensor,
+    out: torch.Tensor = None,
+    p: Optional[Union[float, torch.Tensor]] = None,
+    inner_p: Optional[Union[float, torch.Tensor]] = None,
+    outer_p: Optional[Union[float, torch.Tensor]] = None,
+    bandwidth: Optional[Union[float, torch.Tensor]] = None,
+    epsilon: Optional[float] = None,
+    regularization: Optional[Union[float, torch.Tensor]] = None,
+    regularization_offset_x: int = 0,
+    regularization_offset_y: int = 0,
+    try_to_align: bool = False,
+    debug=False,
+    coefficients: Optional[torch.Tensor] = None,
+):
+    """Fused pairwise kernel matrix (reference: build_a_kernel.py:158-394).
+
+    ``out[l, m, n] = kernel_type(outer_power(sum_k inner_power(b[l,n,k] (-|*) a[l,m,k])))``
+    followed, for Laplace/Gaussian kernels with a non-zero ``regularization``,
+    by replacing every element with ``offset_x + m == offset_y + n`` by
+    ``1 + regularization``.  ``a``, ``b``, ``out`` and the hyper-parameter
+    tensors may each carry a leading batch dimension of 1 or L; a missing batch
+    broadcasts.  Returns ``out`` (allocated as zeros ``[L, M, N]`` when None).
+
+    ``try_to_align`` is accepted for signature compatibility: 128-bit accesses
+    are used whenever pointer, leading dimension and batch stride allow them.
+
+    ``coefficients`` (an addition to the reference's signature): a ``[L?, N, O]``
+    tensor with ``O <= 64`` contiguous columns.  When given, the kernel matrix is
+    contracted with it on the fly and ``out`` is ``[L?, M, O]``:
+    ``out[l, m, o] = sum_n kernelmatrix[l, m, n] * coefficients[l, n, o]``; the
+    M x N matrix is never written to memory.
+    """
+    if coefficients is not None:
+        from .kernel_coefficients import run_kernel_coefficients
+        return run_kernel_coefficients(
+            kernel_descriptor, a, b, coefficients, out=out, p=p, inner_p=inner_p, outer_p=outer_p,
+            bandwidth=bandwidth, epsilon=epsilon, regularization=regularization,
+            regularization_offset_x=regularization_offset_x, regularization_offset_y=regularization_offset_y,
+            debug=debug)
+
+    plan = _plan_run_kernel(
+        kernel_descriptor, a, b, out, p, inner_p, outer_p, bandwidth, epsilon, regularization,
+        regularization_offset_x, regularization_offset_y, try_to_align)
+    stream = _current_stream_for(a.device)
+    params = plan.params
+    with torch.cuda.device(a.device):
+        if _backend.build_kernel_has_variant(params.inner_operator, params.inner_power):
+            if debug:
+                print(f"(Kermac Debug) Launching ahead-of-time kernel for {kernel_descriptor!r}")
+            _backend.build_kernel(params, stream)
+        else:
+            load_a, load_b = _backend.build_kernel_load_modes(params)
+            function_name = build_kernel_function_name(params.inner_operator, params.inner_power, load_a, load_b)
+            function = ModuleCache(debug).get_function(a.device, function_name, debug=debug)
+            if debug:
+                print(f"(Kermac Debug) Launching kernel: {function_name}")
+            _backend.build_kernel_jit(function, params, stream)
+    return plan.out

@@ -1,0 +1,168 @@
+// C-ABI entry points for the fused pairwise-reduction kernel: argument checks,
+// loader selection, and dispatch to the ahead-of-time instantiations (or to a
+// run-time compiled function).
+#include "host_common.hpp"
+#include "../kernels/build_kernel.hpp"
+#include "launchers.hpp"
+
+#include <climits>
+
+using namespace kmc_host;
+
+namespace {
+
+int check_operand(const char *name, const float *ptr, int rows, int k, int64_t ld, int64_t bs, int majorness, int l)
+{
+    if (majorness != KMC_COL_MAJOR && majorness != KMC_ROW_MAJOR)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "%s: majorness %d is not a kmc_majorness", name, majorness);
+    if (rows > 0 && k > 0 && !ptr) return fail(KMC_ERR_INVALID_ARGUMENT, "%s: null pointer", name);
+    const int contiguous_extent = majorness == KMC_COL_MAJOR ? rows : k;
+    const int strided_extent = majorness == KMC_COL_MAJOR ? k : rows;
+    if (strided_extent > 1 && ld < contiguous_extent)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "%s: leading dimension %lld is smaller than the contiguous extent %d",
+                    name, static_cast<long long>(ld), contiguous_extent);
+    if (ld < 0 || bs < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "%s: negative stride", name);
+    (void)l;
+    return KMC_OK;
+}
+
+int pick_load_mode(const float *ptr, int64_t ld, int64_t bs, int majorness, int flags)
+{
+    const bool vec = !(flags & KMC_FLAG_FORCE_SCALAR_ACCESS) && aligned16(ptr) && ld % 4 == 0 && bs % 4 == 0;
+    if (majorness == KMC_COL_MAJOR) return vec ? kmc::LOAD_COL_VEC : kmc::LOAD_COL_SCALAR;
+    return vec ? kmc::LOAD_ROW_VEC : kmc::LOAD_ROW_SCALAR;
+}
+
+// Validates `p` and fills the device argument block.  `need_c` is false for the
+// fused coefficient kernel, which never stores the m x n matrix.
+int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs *args, int *load_a, int *load_b)
+{
+    if (!p) return fail(KMC_ERR_INVALID_ARGUMENT, "null parameter block");
+    if (p->inner_operator != KMC_OP_DIFF && p->inner_operator != KMC_OP_DOT)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "inner_operator %d is not a kmc_inner_operator", p->inner_operator);
+    if (p->inner_power < KMC_POW_NOOP || p->inner_power > KMC_POW_POW)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "inner_power %d is not a kmc_power_type", p->inner_power);
+    if (p->outer_power < KMC_POW_NOOP || p->outer_power > KMC_POW_POW)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "outer_power %d is not a kmc_power_type", p->outer_power);
+    if (p->kernel_type < KMC_KERNEL_NONE || p->kernel_type > KMC_KERNEL_GAUSSIAN)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "kernel_type %d is not a kmc_kernel_type", p->kernel_type);
+    if (p->m < 0 || p->n < 0 || p->k < 0 || p->l < 0)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "negative extent (m=%d n=%d k=%d l=%d)", p->m, p->n, p->k, p->l);
+    if (p->l > 65535) return fail(KMC_ERR_INVALID_ARGUMENT, "batch count %d exceeds 65535", p->l);
+    int status = check_operand("a", p->a, p->m, p->k, p->a_ld, p->a_bs, p->a_majorness, p->l);
+    if (status != KMC_OK) return status;
+    status = check_operand("b", p->b, p->n, p->k, p->b_ld, p->b_bs, p->b_majorness, p->l);
+    if (status != KMC_OK) return status;
+    if (need_c) {
+        if (p->m > 0 && p->n > 0 && !p->c) return fail(KMC_ERR_INVALID_ARGUMENT, "c: null pointer");
+        if (p->n > 1 && p->c_ld < p->m)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "c: leading dimension %lld is smaller than m=%d",
+                        static_cast<long long>(p->c_ld), p->m);
+        if (p->c_ld < 0 || p->c_bs < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "c: negative stride");
+    }
+    const int64_t tiles_m = ceil_div(p->m, kmc::BK_TILE_M);
+    const int64_t tiles_n = ceil_div(p->n, kmc::BK_TILE_N);
+    if (tiles_m * tiles_n > INT_MAX) return fail(KMC_ERR_INVALID_ARGUMENT, "m x n needs more than 2^31 tiles");
+
+    args->m = p->m; args->n = p->n; args->k = p->k; args->l = p->l;
+    args->a = p->a; args->a_ld = p->a_ld; args->a_bs = p->a_bs;
+    args->b = p->b; args->b_ld = p->b_ld; args->b_bs = p->b_bs;
+    args->c = p->c; args->c_ld = p->c_ld; args->c_bs = p->c_bs;
+    args->p_inner = p->p_inner; args->p_inner_bs = p->p_inner_bs; args->p_inner_value = p->p_inner_value;
+    args->p_outer = p->p_outer; args->p_outer_bs = p->p_outer_bs; args->p_outer_value = p->p_outer_value;
+    args->bandwidth = p->bandwidth; args->bandwidth_bs = p->bandwidth_bs; args->bandwidth_value = p->bandwidth_value;
+    args->regularization = p->regularization; args->regularization_bs = p->regularization_bs;
+    args->regularization_value = p->regularization_value;
+    args->reg_off_x = p->regularization_offset_x;
+    args->reg_off_y = p->regularization_offset_y;
+    args->epsilon = p->epsilon;
+    args->diff_sign = (p->flags & KMC_FLAG_NEGATE_DIFF) ? -1.0f : 1.0f;
+    args->outer_power = p->outer_power;
+    args->kernel_type = p->kernel_type;
+    args->c_vec = need_c && !(p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) && aligned16(p->c) && p->c_ld % 4 == 0 &&
+                  p->c_bs % 4 == 0;
+    args->tiles_m = static_cast<int>(tiles_m);
+    args->tiles_n = static_cast<int>(tiles_n);
+    *load_a = pick_load_mode(p->a, p->a_ld, p->a_bs, p->a_majorness, p->flags);
+    *load_b = pick_load_mode(p->b, p->b_ld, p->b_bs, p->b_majorness, p->flags);
+    return KMC_OK;
+}
+
+kmc_host::build_launcher_fn find_launcher(int inner_operator, int inner_power)
+{
+    for (int i = 0; i < kmc_host::build_launcher_count; i++) {
+        const kmc_host::BuildLauncher &entry = kmc_host::build_launchers[i];
+        if (entry.inner_operator == inner_operator && entry.inner_power == inner_power) return entry.launch;
+    }
+    return nullptr;
+}
+
+}  // namespace
+
+namespace kmc_host {
+int prepare_build_kernel(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs *args, int *load_a, int *load_b)
+{
+    return prepare(p, need_c, args, load_a, load_b);
+}
+}  // namespace kmc_host
+
+extern "C" {
+
+int kmc_build_kernel_has_variant(int32_t inner_operator, int32_t inner_power)
+{
+    return find_launcher(inner_operator, inner_power) != nullptr;
+}
+
+int kmc_build_kernel_load_modes(const kmc_build_kernel_params *params, int32_t *load_a, int32_t *load_b)
+{
+    kmc::BuildKernelArgs args;
+    int la = 0, lb = 0;
+    int status = prepare(params, true, &args, &la, &lb);
+    if (status != KMC_OK) return status;
+    if (load_a) *load_a = la;
+    if (load_b) *load_b = lb;
+    return KMC_OK;
+}
+
+int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
+{
+    kmc::BuildKernelArgs args;
+    int load_a = 0, load_b = 0;
+    int status = prepare(params, true, &args, &load_a, &load_b);
+    if (status != KMC_OK) return status;
+    kmc_host::build_launcher_fn launch = find_launcher(params->inner_operator, params->inner_power);
+    if (!launch) {
+        return fail(KMC_ERR_UNSUPPORTED_VARIANT,
+                    "inner_operator=%d inner_power=%d is not compiled ahead of time; compile it at run time",
+                    params->inner_operator, params->inner_power);
+    }
+    if (args.m == 0 || args.n == 0 || args.l == 0) return KMC_OK;
+    status = require_gfx950();
+    if (status != KMC_OK) return status;
+    const dim3 grid(static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n), args.l, 1);
+    hipError_t e = launch(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail_hip(e, "build_kernel launch");
+    return KMC_OK;
+}
+
+int kmc_build_kernel_jit(void *function, const kmc_build_kernel_params *params, void *stream)
+{
+    if (!function) return fail(KMC_ERR_INVALID_ARGUMENT, "kmc_build_kernel_jit: null function");
+    kmc::BuildKernelArgs args;
+    int load_a = 0, load_b = 0;
+    int status = prepare(params, true, &args, &load_a, &load_b);
+    if (status != KMC_OK) return status;
+    if (args.m == 0 || args.n == 0 || args.l == 0) return KMC_OK;
+    status = require_gfx950();
+    if (status != KMC_OK) return status;
+    size_t size = sizeof(args);
+    void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+    hipError_t e = hipModuleLaunchKernel(static_cast<hipFunction_t>(function),
+                                         static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n),
+                                         args.l, 1, kmc::BK_THREADS, 1, 1, 0, static_cast<hipStream_t>(stream), nullptr,
+                                         config);
+    if (e != hipSuccess) return fail_hip(e, "build_kernel (run-time compiled) launch");
+    return KMC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,24 @@
+// Table of the ahead-of-time compiled kernel instantiations.  Each entry is
+// defined in its own device translation unit (kernels/build_kernel_inst.hip
+// compiled once per (inner operator, inner power) pair).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "../kernels/build_kernel.hpp"
+
+namespace kmc_host {
+
+typedef hipError_t (*build_launcher_fn)(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid,
+                                        hipStream_t stream);
+
+struct BuildLauncher {
+    int inner_operator;
+    int inner_power;
+    build_launcher_fn launch;
+};
+
+extern const BuildLauncher build_launchers[];
+extern const int build_launcher_count;
+
+}  // namespace kmc_host

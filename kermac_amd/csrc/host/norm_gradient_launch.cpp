@@ -1,0 +1,67 @@
+// C-ABI entry point for the fused kernel-gradient contraction.
+#include "host_common.hpp"
+#include "../kernels/norm_gradient.hpp"
+
+using namespace kmc_host;
+
+namespace kmc_host {
+hipError_t launch_norm_gradient(int norm_type, int o_tile, const kmc::NormGradientArgs &args, dim3 grid,
+                                hipStream_t stream);
+}
+
+namespace {
+
+bool vec_ok(const void *ptr, int64_t s0, int64_t s1, int64_t s2, int flags)
+{
+    return !(flags & KMC_FLAG_FORCE_SCALAR_ACCESS) && aligned16(ptr) && s0 % 4 == 0 && s1 % 4 == 0 && s2 % 4 == 0;
+}
+
+}  // namespace
+
+extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void *stream)
+{
+    if (!p) return fail(KMC_ERR_INVALID_ARGUMENT, "null parameter block");
+    if (p->norm_type < KMC_NORM_L1 || p->norm_type > KMC_NORM_P)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "norm_type %d is not a kmc_norm_type", p->norm_type);
+    if (p->m < 0 || p->n < 0 || p->o < 0 || p->k < 0 || p->l < 0)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "negative extent (m=%d n=%d o=%d k=%d l=%d)", p->m, p->n, p->o, p->k, p->l);
+    if (p->m == 0 || p->n == 0 || p->o == 0 || p->l == 0) return KMC_OK;
+    if (!p->e || !p->d || (p->k > 0 && (!p->a || !p->b || !p->c)))
+        return fail(KMC_ERR_INVALID_ARGUMENT, "null tensor pointer");
+    if ((p->k > 1 && p->a_ld < p->m) || (p->n > 1 && p->b_ld < p->k) || (p->o > 1 && p->c_ld < p->k) ||
+        (p->n > 1 && p->d_ld < p->m) || (p->n > 1 && p->e_ld_n < p->m))
+        return fail(KMC_ERR_INVALID_ARGUMENT, "a leading dimension is smaller than the contiguous extent it spans");
+    if (p->a_ld < 0 || p->b_ld < 0 || p->c_ld < 0 || p->d_ld < 0 || p->e_ld_n < 0 || p->e_ld_o < 0 || p->a_bs < 0 ||
+        p->b_bs < 0 || p->c_bs < 0 || p->d_bs < 0 || p->e_bs < 0 || p->p_bs < 0)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "negative stride");
+
+    const int o_tile = p->o <= 4 ? 4 : (p->o <= 8 ? 8 : 16);
+    const int o_chunks = ceil_div(p->o, o_tile);
+    const int64_t grid_z = static_cast<int64_t>(p->l) * o_chunks;
+    const int tiles_m = ceil_div(p->m, kmc::NG_TILE_M);
+    const int tiles_n = ceil_div(p->n, kmc::NG_TILE_N);
+    if (grid_z > 65535 || tiles_n > 65535)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "grid too large (n tiles %d, batch x o chunks %lld; limit 65535)", tiles_n,
+                    static_cast<long long>(grid_z));
+
+    kmc::NormGradientArgs args;
+    args.m = p->m; args.n = p->n; args.o = p->o; args.k = p->k; args.l = p->l;
+    args.a = p->a; args.a_ld = p->a_ld; args.a_bs = p->a_bs;
+    args.b = p->b; args.b_ld = p->b_ld; args.b_bs = p->b_bs;
+    args.c = p->c; args.c_ld = p->c_ld; args.c_bs = p->c_bs;
+    args.d = p->d; args.d_ld = p->d_ld; args.d_bs = p->d_bs;
+    args.e = p->e; args.e_ld_n = p->e_ld_n; args.e_ld_o = p->e_ld_o; args.e_bs = p->e_bs;
+    args.p = p->p; args.p_bs = p->p_bs; args.p_value = p->p_value;
+    args.o_chunks = o_chunks;
+    args.a_vec = vec_ok(p->a, p->a_ld, p->a_bs, 0, p->flags);
+    args.b_vec = vec_ok(p->b, p->b_ld, p->b_bs, 0, p->flags);
+    args.c_vec = vec_ok(p->c, p->c_ld, p->c_bs, 0, p->flags);
+    args.e_vec = vec_ok(p->e, p->e_ld_n, p->e_ld_o, p->e_bs, p->flags);
+
+    int status = require_gfx950();
+    if (status != KMC_OK) return status;
+    const dim3 grid(tiles_m, tiles_n, static_cast<unsigned>(grid_z));
+    hipError_t e = launch_norm_gradient(p->norm_type, o_tile, args, grid, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail_hip(e, "norm_kernel_gradient launch");
+    return KMC_OK;
+}

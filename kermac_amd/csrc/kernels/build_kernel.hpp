@@ -1,0 +1,346 @@
+// Fused pairwise-reduction kernel for gfx950:
+//
+//   C[m, n, l] = kernel_fn( outer( sum_k inner( B[n,k,l] (- or *) A[m,k,l] ) ) )
+//
+// Replaces the reference's cute_build_kernel (include/build_a_kernel.cuh:541-623)
+// with a design written for CDNA4 wave64 hardware:
+//
+//   * one workgroup of 256 lanes (4 waves) owns a 128 x 128 output tile and walks
+//     K in slices of 16;
+//   * each lane owns an 8 x 8 register tile made of 4-wide contiguous pieces, so
+//     every LDS fragment read is one ds_read_b128 and every output store is one
+//     128-bit store along the contiguous M direction;
+//   * HBM -> register -> LDS staging is double buffered: the loads for slice
+//     t+1 are in flight while slice t is consumed, with one barrier per slice;
+//   * the inner loop is nothing but subtract + accumulate on the fp32 VALU
+//     (|x| and negation ride on source modifiers), 2 issue slots per (m,n,k);
+//   * outer power, epsilon mask, Laplace/Gaussian function and the diagonal
+//     regularisation are applied to the registers right before the store.
+//
+// Output is always written "column major": C[m + n * c_ld + l * c_bs].  The host
+// swaps the operands when the caller's out tensor is row major, exactly as the
+// reference does (src/kermac/build_a_kernel.py:323-336).
+#pragma once
+
+#include "device_common.hpp"
+
+namespace kmc {
+
+struct BuildKernelArgs {
+    int m, n, k, l;
+    const float *a; i64 a_ld, a_bs;  // A: m x k panel
+    const float *b; i64 b_ld, b_bs;  // B: n x k panel
+    float *c; i64 c_ld, c_bs;        // C: m x n, m contiguous
+    // Hyper-parameters: a device pointer indexed [l * stride], or (pointer null) the value.
+    const float *p_inner; i64 p_inner_bs;
+    const float *p_outer; i64 p_outer_bs;
+    const float *bandwidth; i64 bandwidth_bs;
+    const float *regularization; i64 regularization_bs;
+    float p_inner_value, p_outer_value, bandwidth_value, regularization_value;
+    int reg_off_x, reg_off_y;
+    float epsilon;
+    float diff_sign;   // +1, or -1 when the host swapped the operands
+    int outer_power, kernel_type;
+    int c_vec;     // c, c_ld and c_bs are multiples of 16 bytes: 128-bit stores allowed
+    int tiles_m, tiles_n;
+};
+
+constexpr int BK_TILE_M = 128;
+constexpr int BK_TILE_N = 128;
+constexpr int BK_TILE_K = 16;
+constexpr int BK_THREADS = 256;
+// Row pitch of an LDS slice in floats.  +4 keeps rows 16-byte aligned and skews
+// the banks so that the transposing (k-contiguous) loaders write conflict-free.
+constexpr int BK_LDS_PITCH = BK_TILE_M + 4;
+constexpr int BK_LDS_SLICE = BK_TILE_K * BK_LDS_PITCH;
+
+// One operand's share of a 128 x 16 slice: 8 floats per lane.  `row` is the m (or
+// n) index inside the tile, `kk` the k index inside the slice.
+template <int MODE>
+struct TileLoader {
+    const float *ptr;   // this lane's first element of the current slice
+    i64 step;           // pointer advance per slice
+    i64 ld;
+    int lane_row, lane_k;
+
+    __device__ __forceinline__ void init(const float *base, i64 ld_, int row0, int tid)
+    {
+        ld = ld_;
+        if (MODE == LOAD_COL_VEC) {
+            lane_row = (tid & 31) * 4; lane_k = tid >> 5;          // rows +0..3, k +0 / +8
+            ptr = base + (i64)lane_k * ld + row0 + lane_row; step = (i64)BK_TILE_K * ld;
+        } else if (MODE == LOAD_COL_SCALAR) {
+            lane_row = tid & 127; lane_k = tid >> 7;               // k + 2 i
+            ptr = base + (i64)lane_k * ld + row0 + lane_row; step = (i64)BK_TILE_K * ld;
+        } else if (MODE == LOAD_ROW_VEC) {
+            lane_row = tid >> 2; lane_k = (tid & 3) * 4;           // rows +0 / +64, k +0..3
+            ptr = base + (i64)(row0 + lane_row) * ld + lane_k; step = BK_TILE_K;
+        } else {
+            lane_row = tid >> 4; lane_k = tid & 15;                // rows + 16 i
+            ptr = base + (i64)(row0 + lane_row) * ld + lane_k; step = BK_TILE_K;
+        }
+    }
+
+    // (row, k) of register i inside the tile / slice, and its offset from ptr.
+    __device__ __forceinline__ int row_of(int i) const
+    {
+        if (MODE == LOAD_COL_VEC) return lane_row + (i & 3);
+        if (MODE == LOAD_COL_SCALAR) return lane_row;
+        if (MODE == LOAD_ROW_VEC) return lane_row + (i >> 2) * 64;
+        return lane_row + 16 * i;
+    }
+    __device__ __forceinline__ int k_of(int i) const
+    {
+        if (MODE == LOAD_COL_VEC) return lane_k + (i >> 2) * 8;
+        if (MODE == LOAD_COL_SCALAR) return lane_k + 2 * i;
+        if (MODE == LOAD_ROW_VEC) return lane_k + (i & 3);
+        return lane_k;
+    }
+    __device__ __forceinline__ i64 offset_of(int i) const
+    {
+        if (MODE == LOAD_COL_VEC) return (i64)(i >> 2) * 8 * ld + (i & 3);
+        if (MODE == LOAD_COL_SCALAR) return (i64)(2 * i) * ld;
+        if (MODE == LOAD_ROW_VEC) return (i64)(i >> 2) * 64 * ld + (i & 3);
+        return (i64)(16 * i) * ld;
+    }
+
+    // Whole slice inside the matrix: no predicates.
+    __device__ __forceinline__ void load_full(float (&r)[8]) const
+    {
+        if (MODE == LOAD_COL_VEC || MODE == LOAD_ROW_VEC) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const float4 v = *reinterpret_cast<const float4 *>(ptr + offset_of(4 * h));
+                r[4 * h + 0] = v.x; r[4 * h + 1] = v.y; r[4 * h + 2] = v.z; r[4 * h + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) r[i] = ptr[offset_of(i)];
+        }
+    }
+
+    // Edge slice: rows >= rows_valid or k >= k_valid read as 0.  A zero in both
+    // operands contributes inner(0) = 0 for every inner power the kernel offers
+    // (the reference zero-fills its shared-memory tiles the same way,
+    // include/build_a_kernel.cuh:203-252).
+    __device__ __forceinline__ void load_edge(float (&r)[8], int rows_valid, int k_valid) const
+    {
+        if (MODE == LOAD_COL_VEC || MODE == LOAD_ROW_VEC) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const bool all_in = row_of(4 * h + 3) < rows_valid && k_of(4 * h + 3) < k_valid;
+                if (all_in) {
+                    const float4 v = *reinterpret_cast<const float4 *>(ptr + offset_of(4 * h));
+                    r[4 * h + 0] = v.x; r[4 * h + 1] = v.y; r[4 * h + 2] = v.z; r[4 * h + 3] = v.w;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int i = 4 * h + j;
+                        r[i] = (row_of(i) < rows_valid && k_of(i) < k_valid) ? ptr[offset_of(i)] : 0.0f;
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                r[i] = (row_of(i) < rows_valid && k_of(i) < k_valid) ? ptr[offset_of(i)] : 0.0f;
+            }
+        }
+    }
+
+    __device__ __forceinline__ void advance() { ptr += step; }
+
+    // Write the 8 registers into one LDS slice laid out [k][row] with pitch BK_LDS_PITCH.
+    __device__ __forceinline__ void store(float *slice, const float (&r)[8]) const
+    {
+        if (MODE == LOAD_COL_VEC) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                *reinterpret_cast<float4 *>(slice + (lane_k + 8 * h) * BK_LDS_PITCH + lane_row) =
+                    make_float4(r[4 * h], r[4 * h + 1], r[4 * h + 2], r[4 * h + 3]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) slice[k_of(i) * BK_LDS_PITCH + row_of(i)] = r[i];
+        }
+    }
+};
+
+// 8 floats of one LDS row: columns [0,4) and [64,68) relative to p.
+__device__ __forceinline__ void read_fragment(float (&f)[8], const float *p)
+{
+    const float4 lo = *reinterpret_cast<const float4 *>(p);
+    const float4 hi = *reinterpret_cast<const float4 *>(p + 64);
+    f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w;
+    f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+}
+
+// The K walk for one output tile.  FULL = the tile is interior and K is a
+// multiple of the slice depth, so no load needs a predicate; the compiler then
+// produces a branch-free steady-state loop.
+template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B, bool FULL>
+__device__ __forceinline__ void accumulate_tile(
+    float (&acc)[8][8], TileLoader<LOAD_A> &load_a, TileLoader<LOAD_B> &load_b,
+    float *lds_a, float *lds_b, int k_total, int m_valid, int n_valid, float p_inner, float diff_sign, int tx, int ty)
+{
+    const int k_slices = (k_total + BK_TILE_K - 1) / BK_TILE_K;
+    const int k_tail = k_total - (k_slices - 1) * BK_TILE_K;   // valid k in the last slice
+    float stage_a[8], stage_b[8];
+
+    if (k_slices == 0) return;
+    if (FULL) {
+        load_a.load_full(stage_a);
+        load_b.load_full(stage_b);
+    } else {
+        const int kv = k_slices > 1 ? BK_TILE_K : k_tail;
+        load_a.load_edge(stage_a, m_valid, kv);
+        load_b.load_edge(stage_b, n_valid, kv);
+    }
+    load_a.store(lds_a, stage_a);
+    load_b.store(lds_b, stage_b);
+    __syncthreads();
+
+    for (int slice = 0; slice < k_slices; slice++) {
+        const int cur = slice & 1;
+        const bool has_next = slice + 1 < k_slices;
+        if (has_next) {
+            load_a.advance();
+            load_b.advance();
+            if (FULL) {
+                load_a.load_full(stage_a);
+                load_b.load_full(stage_b);
+            } else {
+                const int kv = slice + 2 == k_slices ? k_tail : BK_TILE_K;
+                load_a.load_edge(stage_a, m_valid, kv);
+                load_b.load_edge(stage_b, n_valid, kv);
+            }
+        }
+
+        const float *sa = lds_a + cur * BK_LDS_SLICE + tx * 4;
+        const float *sb = lds_b + cur * BK_LDS_SLICE + ty * 4;
+        // Register double buffer over the 16 k-steps: the fragments of the next
+        // step are requested before the 128 VALU operations of the current one
+        // are issued.  The loop is kept rolled (two k-steps per trip) on purpose:
+        // fully unrolled, the compiler hoists all 64 LDS reads of a slice to the
+        // top and needs > 300 registers; rolled, it needs ~128 and four waves
+        // fit on each SIMD.
+        float fa0[8], fb0[8], fa1[8], fb1[8];
+        read_fragment(fa0, sa);
+        read_fragment(fb0, sb);
+#pragma unroll 1
+        for (int kk = 0; kk < BK_TILE_K; kk += 2) {
+            read_fragment(fa1, sa + (kk + 1) * BK_LDS_PITCH);
+            read_fragment(fb1, sb + (kk + 1) * BK_LDS_PITCH);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[j][i] += inner_term<INNER_OP, INNER_POW>(fa0[i], fb0[j], p_inner, diff_sign);
+            // On the last trip this reads row 16: the first row of the other
+            // buffer or the pad row.  The values are never used; reading them
+            // unconditionally keeps the loop free of register copies.
+            read_fragment(fa0, sa + (kk + 2) * BK_LDS_PITCH);
+            read_fragment(fb0, sb + (kk + 2) * BK_LDS_PITCH);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[j][i] += inner_term<INNER_OP, INNER_POW>(fa1[i], fb1[j], p_inner, diff_sign);
+        }
+
+        if (has_next) {
+            load_a.store(lds_a + (cur ^ 1) * BK_LDS_SLICE, stage_a);
+            load_b.store(lds_b + (cur ^ 1) * BK_LDS_SLICE, stage_b);
+        }
+        __syncthreads();
+    }
+}
+
+template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
+__global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs args)
+{
+    // Two slices per operand plus one pad row (see the fragment prefetch).
+    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+
+    const int tid = threadIdx.x;
+    const int batch = blockIdx.y;
+    const int tile_m = blockIdx.x % args.tiles_m;
+    const int tile_n = blockIdx.x / args.tiles_m;
+    const int m0 = tile_m * BK_TILE_M;
+    const int n0 = tile_n * BK_TILE_N;
+    const int m_valid = args.m - m0;   // rows of A that exist from m0 on (may exceed 128)
+    const int n_valid = args.n - n0;
+    const int tx = tid & 15;
+    const int ty = tid >> 4;
+
+    float p_inner = 0.0f;
+    if (INNER_POW == POW_POW) {
+        p_inner = args.p_inner ? args.p_inner[batch * args.p_inner_bs] : args.p_inner_value;
+    }
+
+    TileLoader<LOAD_A> load_a;
+    TileLoader<LOAD_B> load_b;
+    load_a.init(args.a + batch * args.a_bs, args.a_ld, m0, tid);
+    load_b.init(args.b + batch * args.b_bs, args.b_ld, n0, tid);
+
+    float acc[8][8];
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[j][i] = 0.0f;
+
+    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
+        accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, true>(
+            acc, load_a, load_b, lds_a, lds_b, args.k, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
+    } else {
+        accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, false>(
+            acc, load_a, load_b, lds_a, lds_b, args.k, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
+    }
+
+    // Epilogue on registers.
+    const int outer_power = args.outer_power;
+    const int kernel_type = args.kernel_type;
+    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
+    if (outer_power == POW_POW) {
+        p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
+    }
+    if (kernel_type != KERNEL_NONE) {
+        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
+        neg_gamma = kernel_neg_gamma(kernel_type, bw);
+        regularization = args.regularization ? args.regularization[batch * args.regularization_bs]
+                                             : args.regularization_value;
+    }
+    const float epsilon = args.epsilon;
+    const bool regularize = kernel_type != KERNEL_NONE && regularization != 0.0f;
+    const float diagonal_value = 1.0f + regularization;
+
+    float *c_tile = args.c + batch * args.c_bs;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int n_local = ty * 4 + (j & 3) + (j >> 2) * 64;
+        const int n_global = n0 + n_local;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int m_local = tx * 4 + h * 64;
+            const int m_global = m0 + m_local;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                v[i] = epilogue_value(acc[j][4 * h + i], outer_power, kernel_type, p_outer, neg_gamma, epsilon);
+                // include/build_a_kernel.cuh:429-447: the diagonal is replaced, not incremented.
+                if (regularize && args.reg_off_x + m_global + i == args.reg_off_y + n_global) v[i] = diagonal_value;
+            }
+            if (n_local < n_valid) {
+                float *dst = c_tile + (i64)n_global * args.c_ld + m_global;
+                if (args.c_vec && m_local + 3 < m_valid) {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (m_local + i < m_valid) dst[i] = v[i];
+                }
+            }
+        }
+    }
+}
+
+}  // namespace kmc

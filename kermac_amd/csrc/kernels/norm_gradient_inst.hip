@@ -1,0 +1,33 @@
+// Ahead-of-time instantiations of the kernel-gradient contraction:
+// 3 norm types x 3 output-tile widths.
+#include <hip/hip_runtime.h>
+
+#include "norm_gradient.hpp"
+
+namespace kmc_host {
+
+template <int NORM>
+static hipError_t launch_norm(int o_tile, const kmc::NormGradientArgs &args, dim3 grid, hipStream_t stream)
+{
+    const dim3 block(kmc::NG_THREADS);
+    switch (o_tile) {
+    case 4: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 4>), grid, block, 0, stream, args); break;
+    case 8: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 8>), grid, block, 0, stream, args); break;
+    case 16: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 16>), grid, block, 0, stream, args); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_norm_gradient(int norm_type, int o_tile, const kmc::NormGradientArgs &args, dim3 grid,
+                                hipStream_t stream)
+{
+    switch (norm_type) {
+    case kmc::NORM_L1: return launch_norm<kmc::NORM_L1>(o_tile, args, grid, stream);
+    case kmc::NORM_L2: return launch_norm<kmc::NORM_L2>(o_tile, args, grid, stream);
+    case kmc::NORM_P: return launch_norm<kmc::NORM_P>(o_tile, args, grid, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace kmc_host

@@ -1,0 +1,30 @@
+"""Shared helpers for the parity tests."""
+import torch
+
+
+def assert_close_to_truth(got: torch.Tensor, truth: torch.Tensor, rtol: float, atol: float = 0.0, what: str = ""):
+    """|got - truth| <= rtol * |truth| + atol element-wise, with a useful message."""
+    got = got.detach().to("cpu", torch.float64)
+    truth = truth.detach().to("cpu", torch.float64)
+    assert got.shape == truth.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(truth.shape)}"
+    err = (got - truth).abs()
+    bound = rtol * truth.abs() + atol
+    bad = err > bound
+    if bad.any() or torch.isnan(got).any() != torch.isnan(truth).any():
+        idx = torch.nonzero(bad)[0].tolist() if bad.any() else None
+        rel = (err / truth.abs().clamp_min(1e-300)).max().item()
+        raise AssertionError(
+            f"{what}: {int(bad.sum())} of {bad.numel()} elements outside rtol={rtol} atol={atol}; "
+            f"max abs err {err.max().item():.3e}, max rel err {rel:.3e}, first bad index {idx}")
+
+
+def make_operand(L, rows, K, col_major, device, generator, batch=True, dist="randn"):
+    """A [L, rows, K] (or [rows, K]) fp32 view that is row- or column-major."""
+    shape = (L, K, rows) if col_major else (L, rows, K)
+    if not batch:
+        shape = shape[1:]
+    fn = torch.randn if dist == "randn" else torch.rand
+    t = fn(shape, generator=generator, dtype=torch.float32).to(device)
+    if col_major:
+        t = t.transpose(-1, -2)
+    return t
