@@ -1,0 +1,343 @@
+"""CPU tests of the host side: layout analysis, batch merging, validation,
+parameter marshalling, the C-ABI surface and the kernel cache.
+
+No kernel is launched here.  The marshalling tests take the parameter block that
+``run_kernel`` / ``cdist_grad`` would hand to the GPU library and interpret it with
+the CPU oracle on the same host memory, so a wrong stride, a missing operand swap
+or a wrong enum value shows up without a GPU.
+"""
+import ctypes
+import re
+from ctypes import POINTER, c_float, c_int, c_int64
+from itertools import product
+from pathlib import Path
+
+import pytest
+import torch
+
+import kermac_amd as kermac
+from kermac_amd import _backend
+from kermac_amd.build_a_kernel import _plan_run_kernel
+from kermac_amd.cdist_grad import _plan_cdist_grad
+from oracle import oracle
+from tests.helpers import assert_close_to_truth, make_operand
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+# ------------------------------------------------------------------ TensorStats
+
+def test_tensor_stats_majorness_alignment_and_batch():
+    t = torch.zeros(3, 8, 12)
+    s = kermac.tensor_stats(t)
+    assert s.shape == (3, 8, 12) and s.majorness is kermac.Majorness.ROW_MAJOR
+    assert s.alignment is kermac.Alignment.ALIGN_1          # row major is never ALIGN_4
+    assert s.batch_stride == 96 and s.leading_dimension_stride == 12 and s.num_batches == 3
+
+    s = kermac.tensor_stats(t.transpose(1, 2))              # [3, 12, 8] view, rows contiguous
+    assert s.shape == (3, 12, 8) and s.majorness is kermac.Majorness.COL_MAJOR
+    assert s.alignment is kermac.Alignment.ALIGN_4 and s.leading_dimension_stride == 12
+
+    s = kermac.tensor_stats(torch.zeros(7, 5).t())          # ld = 5: not a multiple of 4
+    assert s.majorness is kermac.Majorness.COL_MAJOR and s.alignment is kermac.Alignment.ALIGN_1
+    assert s.batch_stride == 0 and s.num_batches == 1
+
+    base = torch.zeros(8 * 12 + 1)
+    off = base[1:].view(8, 12).t()                          # pointer 4 bytes off a 16-byte boundary
+    assert kermac.tensor_stats(off).alignment is kermac.Alignment.ALIGN_1
+
+    assert kermac.tensor_stats(torch.zeros(1, 4, 4)).batch_stride == 0   # batch of 1 broadcasts
+
+    with pytest.raises(ValueError):
+        kermac.tensor_stats(torch.zeros(4, 8)[:, ::2])      # neither dimension contiguous
+    with pytest.raises(ValueError):
+        kermac.tensor_stats(torch.zeros(4))
+    with pytest.raises(TypeError):
+        kermac.tensor_stats(torch.zeros(4, 4, dtype=torch.float64))
+
+
+def test_merge_batch_size_rules():
+    m = kermac.merge_batch_size
+    assert m("x", 1, None, 2, can_be_none=True) == 1
+    with pytest.raises(ValueError):
+        m("x", 1, None, 2)
+    assert m("p", 4, 1.5, 0) == 4
+    with pytest.raises(ValueError):
+        m("a", 1, 1.5, 2)
+    assert m("a", 1, torch.zeros(3, 3), 2) == 1
+    assert m("a", 1, torch.zeros(5, 3, 3), 2) == 5
+    assert m("a", 5, torch.zeros(1, 3, 3), 2) == 5
+    assert m("a", 5, torch.zeros(5, 3, 3), 2) == 5
+    with pytest.raises(ValueError):
+        m("a", 5, torch.zeros(4, 3, 3), 2)
+    with pytest.raises(ValueError):
+        m("a", 1, torch.zeros(2, 2, 3, 3), 2)
+    assert m("p", 1, torch.zeros(6), 0) == 6
+    assert kermac.ceil_div(1000, 128) == 8 and kermac.ceil_div(1024, 128) == 8 and kermac.ceil_div(0, 32) == 0
+
+
+# ------------------------------------------------------------------- validation
+
+def test_run_kernel_validation_errors():
+    a, b = torch.zeros(4, 3), torch.zeros(5, 3)
+    plan = lambda d, *args, **kw: _plan_run_kernel(
+        d, kw.pop("a", a), kw.pop("b", b), kw.pop("out", None), kw.pop("p", None), kw.pop("inner_p", None),
+        kw.pop("outer_p", None), kw.pop("bandwidth", None), kw.pop("epsilon", None), kw.pop("regularization", None),
+        0, 0, False, require_device=False)
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_p_norm)                          # POW without p
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_l1_norm, p=1.3)                  # p without POW
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_l1_norm, bandwidth=1.0)          # bandwidth without kernel
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_laplace_l1)                      # kernel without bandwidth
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_p_norm, p=1.3, inner_p=1.3)
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_p_norm, p=1.3, outer_p=1.3)
+    with pytest.raises(TypeError):
+        plan(kermac.kernel_descriptor_l1_norm, a=[[1.0]])
+    with pytest.raises(TypeError):
+        plan(kermac.kernel_descriptor_l1_norm, a=torch.zeros(4, 3, dtype=torch.float64))
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_l1_norm, b=torch.zeros(5, 4))    # K mismatch
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_l1_norm, out=torch.zeros(5, 4))  # out is [M, N], not [N, M]
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_l1_norm, a=torch.zeros(2, 4, 3), b=torch.zeros(3, 5, 3))  # batch 2 vs 3
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_l1_norm, a=torch.zeros(2, 4, 3), out=torch.zeros(1, 4, 5))
+    with pytest.raises(TypeError):
+        plan(kermac.kernel_descriptor_laplace_l1, bandwidth=torch.zeros((), dtype=torch.float64))
+    with pytest.raises(ValueError):
+        plan(kermac.kernel_descriptor_laplace_l1, a=torch.zeros(2, 4, 3), bandwidth=torch.ones(3))
+    # the real entry points refuse CPU tensors, as the reference does
+    with pytest.raises(ValueError):
+        kermac.run_kernel(kermac.kernel_descriptor_l1_norm, a, b)
+    with pytest.raises(ValueError):
+        kermac.cdist(a, b)
+    with pytest.raises(ValueError):
+        kermac.cdist_grad(torch.zeros(3, 4), torch.zeros(5, 3), torch.zeros(2, 3), torch.zeros(5, 4))
+
+
+def test_cdist_grad_validation_errors():
+    a, b, c, d = torch.zeros(6, 4), torch.zeros(5, 6), torch.zeros(2, 6), torch.zeros(5, 4)
+    plan = lambda *t, **kw: _plan_cdist_grad(*t, kw.get("out"), kw.get("p", 2.0), require_device=False)
+    assert plan(a, b, c, d).out.shape == (1, 2, 5, 4)
+    with pytest.raises(TypeError):
+        plan(a, b, c, [1.0])
+    with pytest.raises(TypeError):
+        plan(a.double(), b, c, d)
+    with pytest.raises(ValueError):
+        plan(a, torch.zeros(5, 7), c, d)                    # K mismatch
+    with pytest.raises(ValueError):
+        plan(a, b, torch.zeros(2, 7), d)
+    with pytest.raises(ValueError):
+        plan(a, b, c, torch.zeros(4, 5))                    # d must be [N, M]
+    with pytest.raises(ValueError):
+        plan(a, b, c, d, out=torch.zeros(2, 4, 5))          # out must be [O, N, M]
+    with pytest.raises(ValueError):
+        plan(a.t().contiguous().t(), b, c, d)               # a not contiguous in M
+    with pytest.raises(ValueError):
+        plan(torch.zeros(6), b, c, d)
+    with pytest.raises(ValueError):
+        plan(torch.zeros(2, 6, 4), torch.zeros(3, 5, 6), c, d)
+
+
+def test_skip_epilogue_does_not_modify_shared_descriptors():
+    # The reference mutates its module-level descriptor (cdist.py:65,75); here the
+    # predefined descriptors must be untouched by any call.
+    before = (kermac.kernel_descriptor_l2_norm._outer_power, kermac.kernel_descriptor_p_norm._outer_power)
+    for p in (2.0, 1.3):
+        with pytest.raises(ValueError):                     # CPU tensors: rejected after descriptor handling
+            kermac.cdist(torch.zeros(2, 2), torch.zeros(2, 2), p=p, skip_epilogue=True)
+    assert before == (kermac.PowerType.SQRT, kermac.PowerType.POW)
+    assert (kermac.kernel_descriptor_l2_norm._outer_power, kermac.kernel_descriptor_p_norm._outer_power) == before
+
+
+# ---------------------------------------------- marshalling, interpreted on the CPU
+
+_lib = ctypes.CDLL(str(oracle.build()))
+_OP = ["DIFF", "DOT"]
+_POWER = ["NOOP", "ABS", "SQUARE", "SQRT", "POW"]
+_KERNEL = ["NONE", "LAPLACE", "GAUSSIAN"]
+
+
+def _fp(address):
+    return ctypes.cast(ctypes.c_void_p(address), POINTER(c_float)) if address else None
+
+
+def interpret_build_params(p: _backend.BuildKernelParams):
+    """Execute a build-kernel parameter block with the CPU oracle, in place, the way
+    the device kernel is specified to (include/kermac_amd.h)."""
+    def strides(ld, majorness):
+        return (1, ld) if majorness == _backend.COL_MAJOR else (ld, 1)
+    a_sm, a_sk = strides(p.a_ld, p.a_majorness)
+    b_sn, b_sk = strides(p.b_ld, p.b_majorness)
+    args_a = (_fp(p.a), c_int64(a_sm), c_int64(a_sk), c_int64(p.a_bs))
+    args_b = (_fp(p.b), c_int64(b_sn), c_int64(b_sk), c_int64(p.b_bs))
+    m, n, c_sm, c_sn, off_x, off_y = p.m, p.n, 1, p.c_ld, p.regularization_offset_x, p.regularization_offset_y
+    if p.flags & _backend.FLAG_NEGATE_DIFF:
+        # value(m, n) uses A - B: evaluate with the operands exchanged and write transposed
+        args_a, args_b = args_b, args_a
+        m, n, c_sm, c_sn, off_x, off_y = n, m, c_sn, c_sm, off_y, off_x
+    hyper = []
+    for ptr, bs, val in ((p.p_inner, p.p_inner_bs, p.p_inner_value), (p.p_outer, p.p_outer_bs, p.p_outer_value),
+                         (p.bandwidth, p.bandwidth_bs, p.bandwidth_value),
+                         (p.regularization, p.regularization_bs, p.regularization_value)):
+        if ptr:
+            hyper += [_fp(ptr), c_int64(bs)]
+        else:
+            keep = (c_float * 1)(val)
+            hyper += [keep, c_int64(0)]
+    _lib.kmo_build_kernel(
+        c_int(p.inner_operator), c_int(p.inner_power), c_int(p.outer_power), c_int(p.kernel_type),
+        c_int(m), c_int(n), c_int(p.k), c_int(p.l), *args_a, *args_b,
+        _fp(p.c), c_int64(c_sm), c_int64(c_sn), c_int64(p.c_bs), *hyper,
+        c_int(off_x), c_int(off_y), c_float(p.epsilon), c_int(1))
+
+
+def cpu_run_kernel(descriptor, a, b, out=None, p=None, inner_p=None, outer_p=None, bandwidth=None, epsilon=None,
+                   regularization=None, regularization_offset_x=0, regularization_offset_y=0):
+    plan = _plan_run_kernel(descriptor, a, b, out, p, inner_p, outer_p, bandwidth, epsilon, regularization,
+                            regularization_offset_x, regularization_offset_y, False, require_device=False)
+    interpret_build_params(plan.params)
+    return plan.out
+
+
+@pytest.mark.parametrize("a_col,b_col,c_col", list(product([False, True], repeat=3)))
+@pytest.mark.parametrize("p", [1.0, 1.3, 2.0])
+def test_marshalling_all_majorness_combinations(a_col, b_col, c_col, p):
+    # The reference's test matrix (tests/test_cdist.py:50-57) at a small size.
+    g = torch.Generator().manual_seed(11)
+    L, M, N, K = 2, 21, 17, 9
+    a = make_operand(L, M, K, a_col, "cpu", g)
+    b = make_operand(L, N, K, b_col, "cpu", g)
+    out = torch.full((L, N, M), float("nan")).transpose(1, 2) if c_col else torch.full((L, M, N), float("nan"))
+    descriptor, kwargs = {
+        1.0: (kermac.kernel_descriptor_l1_norm, {}),
+        2.0: (kermac.kernel_descriptor_l2_norm, {}),
+        1.3: (kermac.kernel_descriptor_p_norm, {"p": 1.3}),
+    }[p]
+    got = cpu_run_kernel(descriptor, a, b, out=out, **kwargs)
+    assert got is out
+    assert_close_to_truth(got, torch.cdist(a.double(), b.double(), p=p), rtol=1e-6, what="marshalled cdist")
+
+
+@pytest.mark.parametrize("c_col", [False, True])
+def test_marshalling_sign_and_offsets_survive_the_swap(c_col):
+    g = torch.Generator().manual_seed(12)
+    M, N, K = 13, 10, 6
+    a, b = torch.randn(M, K, generator=g), torch.randn(N, K, generator=g)
+    out = torch.empty(N, M).t() if c_col else torch.empty(M, N)
+    signed = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.NOOP, kermac.PowerType.NOOP,
+                                     kermac.KernelType.NONE)
+    got = cpu_run_kernel(signed, a, b, out=out)
+    truth = (b.double()[None, :, :] - a.double()[:, None, :]).sum(-1)        # sum_k (b - a), signed
+    assert_close_to_truth(got, truth, rtol=1e-6, atol=1e-9, what="signed difference")
+    got = cpu_run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, out=out, bandwidth=2.0, regularization=0.5,
+                         regularization_offset_x=4, regularization_offset_y=1)
+    truth = torch.exp(-torch.cdist(a.double(), b.double(), p=1.0) / 2.0)
+    for m in range(M):
+        if 0 <= m + 3 < N:
+            truth[m, m + 3] = 1.5
+    assert_close_to_truth(got, truth, rtol=1e-6, what="offset diagonal")
+
+
+def test_marshalling_broadcast_and_hyper_parameter_tensors():
+    g = torch.Generator().manual_seed(13)
+    L, M, N, K = 3, 8, 7, 5
+    a = torch.randn(L, M, K, generator=g)
+    b = torch.randn(N, K, generator=g)                       # broadcast over the batch
+    p = torch.tensor([1.5, 2.5, 0.7])
+    got = cpu_run_kernel(kermac.kernel_descriptor_p_norm, a, b, p=p)
+    assert got.shape == (L, M, N)
+    truth = torch.stack([torch.cdist(a[i].double(), b.double(), p=float(p[i])) for i in range(L)])
+    assert_close_to_truth(got, truth, rtol=2e-6, what="per-batch p")
+    bw = torch.tensor([1.0, 2.0, 4.0])
+    got = cpu_run_kernel(kermac.kernel_descriptor_laplace_l2, a, b, bandwidth=bw, regularization=torch.tensor(0.0))
+    truth = torch.exp(-torch.cdist(a.double(), b.double().expand(L, -1, -1), p=2.0) / bw.double()[:, None, None])
+    assert_close_to_truth(got, truth, rtol=2e-6, what="per-batch bandwidth")
+    # a one-element 1-D tensor broadcasts (the reference reads out of bounds here)
+    got = cpu_run_kernel(kermac.kernel_descriptor_laplace_l2, a, b, bandwidth=torch.tensor([2.0]))
+    truth = torch.exp(-torch.cdist(a.double(), b.double().expand(L, -1, -1), p=2.0) / 2.0)
+    assert_close_to_truth(got, truth, rtol=2e-6, what="1-element bandwidth")
+    # out=None allocates [L, M, N] zeros-initialised storage and 2-D inputs give L = 1
+    got = cpu_run_kernel(kermac.kernel_descriptor_l1_norm, a[0], b)
+    assert got.shape == (1, M, N)
+
+
+def test_scalar_p_rounding_matches_fp32_division():
+    plan = _plan_run_kernel(kermac.kernel_descriptor_p_norm, torch.zeros(2, 2), torch.zeros(2, 2), None, 1.3, None,
+                            None, None, None, None, 0, 0, False, require_device=False)
+    expect_inner = torch.tensor(1.3, dtype=torch.float32)
+    assert plan.params.p_inner_value == expect_inner.item()
+    assert plan.params.p_outer_value == (1.0 / expect_inner).item()
+    assert plan.params.p_inner is None and plan.params.p_outer is None
+    assert plan.params.epsilon == pytest.approx(1e-5)
+
+
+def interpret_grad_params(p: _backend.NormGradientParams):
+    keep = (c_float * 1)(p.p_value)
+    _lib.kmo_norm_kernel_gradient(
+        c_int(p.norm_type), c_int(p.m), c_int(p.n), c_int(p.o), c_int(p.k), c_int(p.l),
+        _fp(p.a), c_int64(p.a_ld), c_int64(1), c_int64(p.a_bs),
+        _fp(p.b), c_int64(p.b_ld), c_int64(1), c_int64(p.b_bs),
+        _fp(p.c), c_int64(p.c_ld), c_int64(1), c_int64(p.c_bs),
+        _fp(p.d), c_int64(p.d_ld), c_int64(1), c_int64(p.d_bs),
+        _fp(p.e), c_int64(p.e_ld_o), c_int64(p.e_ld_n), c_int64(1), c_int64(p.e_bs),
+        _fp(p.p) if p.p else keep, c_int64(p.p_bs), c_int(1))
+
+
+@pytest.mark.parametrize("p", [1.0, 2.0, 1.3, "tensor"])
+def test_gradient_marshalling(p):
+    g = torch.Generator().manual_seed(14)
+    L, M, N, O, K = 2, 12, 7, 3, 10
+    a = torch.rand(L, K, M, generator=g)
+    b = torch.randn(N, K, generator=g)                       # broadcast
+    c = torch.randn(L, O, K + 2, generator=g)[:, :, :K]      # leading dimension larger than K
+    d = torch.randn(L, N, M, generator=g)
+    out = torch.full((L, O, N, M), float("nan"))
+    p_arg = torch.tensor([1.5, 3.0]) if p == "tensor" else p
+    plan = _plan_cdist_grad(a, b, c, d, out, p_arg, require_device=False)
+    assert plan.params.norm_type == {1.0: 0, 2.0: 1}.get(p, 2)
+    interpret_grad_params(plan.params)
+    truth = oracle.cdist_grad(a, b, c.contiguous(), d, p=p_arg)
+    assert_close_to_truth(out, truth, rtol=1e-6, atol=1e-6, what="marshalled gradient")
+
+
+# ------------------------------------------------------------------ C ABI surface
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "kermac_amd.h").read_text()
+    declared = set(re.findall(r"^\s*(?:int|void|const char \*)\s*\*?(kmc_[a-z0-9_]+)\s*\(", header, flags=re.M))
+    assert len(declared) >= 14, declared
+    assert declared == set(_backend.SIGNATURES), declared ^ set(_backend.SIGNATURES)
+    lib = _backend.library()                                # raises if the library is not built
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in kermac_amd.h but not exported"
+    assert lib.kmc_abi_version() == _backend.ABI_VERSION
+    # struct layout agreed between header and binding: spot-check sizes
+    assert ctypes.sizeof(_backend.BuildKernelParams) % 8 == 0
+    assert _backend.build_kernel_has_variant(0, 1) and _backend.build_kernel_has_variant(0, 2)
+    assert _backend.build_kernel_has_variant(0, 4) and _backend.build_kernel_has_variant(1, 0)
+
+
+def test_c_abi_rejects_bad_arguments_without_a_gpu():
+    params = _backend.BuildKernelParams()
+    params.inner_operator = 7
+    with pytest.raises(_backend.BackendError) as info:
+        _backend.build_kernel(params, 0)
+    assert info.value.status == _backend.ERR_INVALID_ARGUMENT and "inner_operator" in str(info.value)
+    params = _backend.BuildKernelParams()
+    params.inner_power = 1
+    params.m = params.n = params.k = 4
+    params.l = 1
+    with pytest.raises(_backend.BackendError) as info:      # null operand pointers
+        _backend.build_kernel(params, 0)
+    assert info.value.status == _backend.ERR_INVALID_ARGUMENT
+    grad = _backend.NormGradientParams()
+    grad.norm_type = 9
+    with pytest.raises(_backend.BackendError):
+        _backend.norm_kernel_gradient(grad, 0)
