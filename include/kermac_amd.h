@@ -142,12 +142,21 @@ int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *params, void *strea
  */
 typedef struct kmc_kernel_coefficients_params {
     kmc_build_kernel_params kernel;
-    int32_t o;                                    /* coefficient columns, 1..64 */
+    int32_t o;                                    /* coefficient columns */
     const float *coef; int64_t coef_ld; int64_t coef_bs;  /* [n, o], o contiguous */
     float *out; int64_t out_ld; int64_t out_bs;           /* [m, o], o contiguous */
 } kmc_kernel_coefficients_params;
 
+/* Coefficient columns are processed in chunks of 32 per workgroup; o > 32 works
+ * (the kernel values are then recomputed per chunk).  Returns
+ * KMC_ERR_UNSUPPORTED_VARIANT when the (inner_operator, inner_power) pair is not
+ * among the ahead-of-time compiled ones. */
 int kmc_kernel_times_coefficients(const kmc_kernel_coefficients_params *params, void *stream);
+/* 1 when (inner_operator, inner_power) is compiled ahead of time for the fused
+ * coefficient kernel. */
+int kmc_kernel_times_coefficients_has_variant(int32_t inner_operator, int32_t inner_power);
+/* Launch a run-time compiled kmc::kernel_times_coefficients instantiation. */
+int kmc_kernel_times_coefficients_jit(void *function, const kmc_kernel_coefficients_params *params, void *stream);
 
 /* ---- run-time compilation (stands in for cuda.core Program / ObjectCode:
  *      src/kermac/module_cache/module_cache.py:13-51, 219-239) ---- */

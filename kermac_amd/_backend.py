@@ -86,6 +86,8 @@ SIGNATURES = {
     "kmc_build_kernel_load_modes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int32), POINTER(c_int32)]),
     "kmc_norm_kernel_gradient": (ctypes.c_int, [POINTER(NormGradientParams), c_void_p]),
     "kmc_kernel_times_coefficients": (ctypes.c_int, [POINTER(KernelCoefficientsParams), c_void_p]),
+    "kmc_kernel_times_coefficients_has_variant": (ctypes.c_int, [c_int32, c_int32]),
+    "kmc_kernel_times_coefficients_jit": (ctypes.c_int, [c_void_p, POINTER(KernelCoefficientsParams), c_void_p]),
     "kmc_jit_compile": (ctypes.c_int, [
         c_char_p, c_char_p,
         ctypes.c_int, POINTER(c_char_p), POINTER(c_char_p),
@@ -169,6 +171,14 @@ def norm_kernel_gradient(params: NormGradientParams, stream: int) -> None:
 
 def kernel_times_coefficients(params: KernelCoefficientsParams, stream: int) -> None:
     check(library().kmc_kernel_times_coefficients(byref(params), c_void_p(stream)))
+
+
+def kernel_times_coefficients_jit(function: int, params: KernelCoefficientsParams, stream: int) -> None:
+    check(library().kmc_kernel_times_coefficients_jit(c_void_p(function), byref(params), c_void_p(stream)))
+
+
+def kernel_times_coefficients_has_variant(inner_operator: int, inner_power: int) -> bool:
+    return bool(library().kmc_kernel_times_coefficients_has_variant(inner_operator, inner_power))
 
 
 def device_arch(device: int) -> str:

@@ -37,6 +37,9 @@ HIPCC_FLAGS = [
 # csrc/host/launcher_table.cpp.
 AOT_BUILD_KERNEL_VARIANTS = [(0, 0), (0, 1), (0, 2), (0, 4), (1, 0)]
 
+# Pairs compiled ahead of time for the fused kernel-matrix x coefficients kernel.
+AOT_COEFFICIENT_VARIANTS = [(0, 1), (0, 2), (0, 4)]
+
 HOST_SOURCES = [
     "host/runtime.cpp",
     "host/build_kernel_launch.cpp",
@@ -65,6 +68,10 @@ def _jobs():
     inst = CSRC / "kernels" / "build_kernel_inst.hip"
     for op, pw in AOT_BUILD_KERNEL_VARIANTS:
         jobs.append((inst, OBJ_DIR / f"build_kernel_inst_{op}_{pw}.o", [f"-DKMC_INNER_OP={op}", f"-DKMC_INNER_POW={pw}"]))
+    inst = CSRC / "kernels" / "kernel_coefficients_inst.hip"
+    for op, pw in AOT_COEFFICIENT_VARIANTS:
+        jobs.append((inst, OBJ_DIR / f"kernel_coefficients_inst_{op}_{pw}.o",
+                     [f"-DKMC_INNER_OP={op}", f"-DKMC_INNER_POW={pw}"]))
     for rel in EXTRA_DEVICE_SOURCES:
         src = CSRC / rel
         jobs.append((src, OBJ_DIR / (src.stem + ".o"), []))

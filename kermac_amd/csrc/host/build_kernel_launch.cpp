@@ -117,7 +117,7 @@ int kmc_build_kernel_load_modes(const kmc_build_kernel_params *params, int32_t *
 {
     kmc::BuildKernelArgs args;
     int la = 0, lb = 0;
-    int status = prepare(params, true, &args, &la, &lb);
+    int status = prepare(params, false, &args, &la, &lb);   // only a and b matter here
     if (status != KMC_OK) return status;
     if (load_a) *load_a = la;
     if (load_b) *load_b = lb;

@@ -254,6 +254,48 @@ __device__ __forceinline__ void accumulate_tile(
     }
 }
 
+// Epilogue on the register tile: outer power, epsilon mask, kernel function and
+// the diagonal regularisation (include/build_a_kernel.cuh:374-447).  Lane
+// (tx, ty) holds acc[j][i] for n = n0 + ty*4 + (j&3) + (j>>2)*64 and
+// m = m0 + tx*4 + (i&3) + (i>>2)*64.
+__device__ __forceinline__ void finish_tile(
+    float (&acc)[8][8], const BuildKernelArgs &args, int batch, int m0, int n0, int tx, int ty)
+{
+    const int outer_power = args.outer_power;
+    const int kernel_type = args.kernel_type;
+    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
+    if (outer_power == POW_POW) {
+        p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
+    }
+    if (kernel_type != KERNEL_NONE) {
+        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
+        neg_gamma = kernel_neg_gamma(kernel_type, bw);
+        regularization = args.regularization ? args.regularization[batch * args.regularization_bs]
+                                             : args.regularization_value;
+    }
+    const float epsilon = args.epsilon;
+    if (outer_power != POW_NOOP || kernel_type != KERNEL_NONE) {
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                acc[j][i] = epilogue_value(acc[j][i], outer_power, kernel_type, p_outer, neg_gamma, epsilon);
+    }
+    // include/build_a_kernel.cuh:429-447: the diagonal is replaced, not incremented.
+    if (kernel_type != KERNEL_NONE && regularization != 0.0f) {
+        const float diagonal_value = 1.0f + regularization;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int n_global = n0 + ty * 4 + (j & 3) + (j >> 2) * 64;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int m_global = m0 + tx * 4 + (i & 3) + (i >> 2) * 64;
+                if (args.reg_off_x + m_global == args.reg_off_y + n_global) acc[j][i] = diagonal_value;
+            }
+        }
+    }
+}
+
 template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
 __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs args)
 {
@@ -296,48 +338,25 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
             acc, load_a, load_b, lds_a, lds_b, args.k, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
     }
 
-    // Epilogue on registers.
-    const int outer_power = args.outer_power;
-    const int kernel_type = args.kernel_type;
-    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
-    if (outer_power == POW_POW) {
-        p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
-    }
-    if (kernel_type != KERNEL_NONE) {
-        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
-        neg_gamma = kernel_neg_gamma(kernel_type, bw);
-        regularization = args.regularization ? args.regularization[batch * args.regularization_bs]
-                                             : args.regularization_value;
-    }
-    const float epsilon = args.epsilon;
-    const bool regularize = kernel_type != KERNEL_NONE && regularization != 0.0f;
-    const float diagonal_value = 1.0f + regularization;
+    finish_tile(acc, args, batch, m0, n0, tx, ty);
 
+    // Store: each lane writes 16 pieces of 4 consecutive m.
     float *c_tile = args.c + batch * args.c_bs;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const int n_local = ty * 4 + (j & 3) + (j >> 2) * 64;
-        const int n_global = n0 + n_local;
+        if (n_local >= n_valid) continue;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const int m_local = tx * 4 + h * 64;
-            const int m_global = m0 + m_local;
-            float v[4];
+            float *dst = c_tile + (i64)(n0 + n_local) * args.c_ld + m0 + m_local;
+            if (args.c_vec && m_local + 3 < m_valid) {
+                *reinterpret_cast<float4 *>(dst) =
+                    make_float4(acc[j][4 * h], acc[j][4 * h + 1], acc[j][4 * h + 2], acc[j][4 * h + 3]);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                v[i] = epilogue_value(acc[j][4 * h + i], outer_power, kernel_type, p_outer, neg_gamma, epsilon);
-                // include/build_a_kernel.cuh:429-447: the diagonal is replaced, not incremented.
-                if (regularize && args.reg_off_x + m_global + i == args.reg_off_y + n_global) v[i] = diagonal_value;
-            }
-            if (n_local < n_valid) {
-                float *dst = c_tile + (i64)n_global * args.c_ld + m_global;
-                if (args.c_vec && m_local + 3 < m_valid) {
-                    *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        if (m_local + i < m_valid) dst[i] = v[i];
-                }
+                for (int i = 0; i < 4; i++)
+                    if (m_local + i < m_valid) dst[i] = acc[j][4 * h + i];
             }
         }
     }

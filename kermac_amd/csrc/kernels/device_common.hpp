@@ -83,4 +83,17 @@ __device__ __forceinline__ float kernel_neg_gamma(int kernel_type, float bandwid
     return 0.0f;
 }
 
+// 4 consecutive floats starting at p; elements at index >= valid read as 0.
+// `vec` says that p is 16-byte aligned.
+__device__ __forceinline__ float4 load4_guarded(const float *p, int valid, bool vec)
+{
+    if (vec && valid >= 4) return *reinterpret_cast<const float4 *>(p);
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (valid > 0) v.x = p[0];
+    if (valid > 1) v.y = p[1];
+    if (valid > 2) v.z = p[2];
+    if (valid > 3) v.w = p[3];
+    return v;
+}
+
 }  // namespace kmc

@@ -1,0 +1,50 @@
+// One (inner operator, inner power) pair of the fused kernel-matrix x
+// coefficients kernel, instantiated for all 16 (A loader, B loader) pairs.
+// Compiled several times with different -DKMC_INNER_OP / -DKMC_INNER_POW.
+#include <hip/hip_runtime.h>
+
+#include "kernel_coefficients.hpp"
+
+#ifndef KMC_INNER_OP
+#error "compile with -DKMC_INNER_OP=<0|1> -DKMC_INNER_POW=<0..4>"
+#endif
+
+#define KMC_CAT_(a, b, c, d) a##b##c##d
+#define KMC_CAT(a, b, c, d) KMC_CAT_(a, b, c, d)
+#define KMC_LAUNCHER_NAME KMC_CAT(launch_kernel_coefficients_, KMC_INNER_OP, _, KMC_INNER_POW)
+
+namespace kmc_host {
+
+template <int LOAD_A, int LOAD_B>
+static hipError_t launch_one(const kmc::KernelCoefficientsArgs &args, dim3 grid, hipStream_t stream)
+{
+    hipLaunchKernelGGL((kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>), grid,
+                       dim3(kmc::BK_THREADS), 0, stream, args);
+    return hipGetLastError();
+}
+
+hipError_t KMC_LAUNCHER_NAME(int load_a, int load_b, const kmc::KernelCoefficientsArgs &args, dim3 grid,
+                             hipStream_t stream)
+{
+    switch (load_a * 4 + load_b) {
+    case 0: return launch_one<0, 0>(args, grid, stream);
+    case 1: return launch_one<0, 1>(args, grid, stream);
+    case 2: return launch_one<0, 2>(args, grid, stream);
+    case 3: return launch_one<0, 3>(args, grid, stream);
+    case 4: return launch_one<1, 0>(args, grid, stream);
+    case 5: return launch_one<1, 1>(args, grid, stream);
+    case 6: return launch_one<1, 2>(args, grid, stream);
+    case 7: return launch_one<1, 3>(args, grid, stream);
+    case 8: return launch_one<2, 0>(args, grid, stream);
+    case 9: return launch_one<2, 1>(args, grid, stream);
+    case 10: return launch_one<2, 2>(args, grid, stream);
+    case 11: return launch_one<2, 3>(args, grid, stream);
+    case 12: return launch_one<3, 0>(args, grid, stream);
+    case 13: return launch_one<3, 1>(args, grid, stream);
+    case 14: return launch_one<3, 2>(args, grid, stream);
+    case 15: return launch_one<3, 3>(args, grid, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace kmc_host

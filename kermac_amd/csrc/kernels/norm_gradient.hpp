@@ -51,18 +51,6 @@ __device__ __forceinline__ float gradient_weight(float diff, float p_minus_1)
     return fast_pow_abs(__builtin_fabsf(diff), p_minus_1) * sign;
 }
 
-// 4 consecutive floats starting at p; elements at index >= valid read as 0.
-__device__ __forceinline__ float4 load4_guarded(const float *p, int valid, bool vec)
-{
-    if (vec && valid >= 4) return *reinterpret_cast<const float4 *>(p);
-    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    if (valid > 0) v.x = p[0];
-    if (valid > 1) v.y = p[1];
-    if (valid > 2) v.z = p[2];
-    if (valid > 3) v.w = p[3];
-    return v;
-}
-
 template <int NORM, int O_TILE>
 __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGradientArgs args)
 {

@@ -33,13 +33,19 @@ _INNER_OPERATOR_NAMES = ["kmc::OP_DIFF", "kmc::OP_DOT"]
 _POWER_NAMES = ["kmc::POW_NOOP", "kmc::POW_ABS", "kmc::POW_SQUARE", "kmc::POW_SQRT", "kmc::POW_POW"]
 _LOAD_MODE_NAMES = ["kmc::LOAD_COL_VEC", "kmc::LOAD_COL_SCALAR", "kmc::LOAD_ROW_VEC", "kmc::LOAD_ROW_SCALAR"]
 
-JIT_TRANSLATION_UNIT = '#include "build_kernel.hpp"\n'
-JIT_HEADERS = ["device_common.hpp", "build_kernel.hpp"]
+JIT_TRANSLATION_UNIT = '#include "kernel_coefficients.hpp"\n'
+JIT_HEADERS = ["device_common.hpp", "build_kernel.hpp", "kernel_coefficients.hpp"]
 
 
 def build_kernel_function_name(inner_operator: int, inner_power: int, load_a: int, load_b: int) -> str:
     """Template-id (a hiprtc name expression) of one kernel instantiation."""
     return (f"kmc::build_kernel<{_INNER_OPERATOR_NAMES[inner_operator]},{_POWER_NAMES[inner_power]},"
+            f"{_LOAD_MODE_NAMES[load_a]},{_LOAD_MODE_NAMES[load_b]}>")
+
+
+def kernel_coefficients_function_name(inner_operator: int, inner_power: int, load_a: int, load_b: int) -> str:
+    """Template-id of one fused kernel-matrix x coefficients instantiation."""
+    return (f"kmc::kernel_times_coefficients<{_INNER_OPERATOR_NAMES[inner_operator]},{_POWER_NAMES[inner_power]},"
             f"{_LOAD_MODE_NAMES[load_a]},{_LOAD_MODE_NAMES[load_b]}>")
 
 
