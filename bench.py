@@ -31,9 +31,10 @@ ALGORITHMIC_BYTES = 4.0 * (M * K + N * K + M * N)
 PEAK_FP32_VALU_TFLOPS = 157.3        # AMD's published MI355X fp32 vector peak
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per cdist launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/build_kernel_cdist_30000x30000x1024_pmc.txt); None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per p = 1 cdist launch measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each
+# scaled by what the counter reads for a 1 GiB copy kernel
+# (profiles/build_kernel_cdist_p1_30000x30000x1024.txt): 12.67 GB fetched + 3.62 GB written.
+MEASURED_TRAFFIC_BYTES = 16.3e9
 
 
 def log(*args):
@@ -70,7 +71,7 @@ def parity_slab(out, a, b, p, skip_epilogue):
     return worst
 
 
-def cpu_baseline(a_store_cpu, b_store_cpu, p=1.0, slab=2048):
+def cpu_baseline(a_store_cpu, b_store_cpu, p=1.0, slab=16384):
     """torch.cdist (the oracle of the reference's tests) on the host cores, on a
     bounded slab of the same workload: all of a, the first `slab` columns of b."""
     a = a_store_cpu.t()
@@ -109,6 +110,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=2)
     parser.add_argument("--skip-cpu", action="store_true", help="skip the host-CPU baseline leg")
     parser.add_argument("--only-p1", action="store_true", help="time only the headline p = 1.0 configuration")
+    parser.add_argument("--calibration-copy", action="store_true",
+                        help="also run one plain elementwise copy kernel over 1 GiB (read 1 GiB, write 1 GiB), so that "
+                             "hardware byte counters collected by a profiler can be scaled against a known transfer")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on one GPU only (it shards by giving each GPU its own slab of b "
@@ -126,6 +130,13 @@ def main():
     b_store = torch.randn(K, N, device=device)
     out_store = torch.empty(N, M, device=device)
     a, b, out = a_store.t(), b_store.t(), out_store.t()      # the operator's [M,K] / [N,K] / [M,N] views
+
+    if args.calibration_copy:
+        src = torch.ones(1 << 28, device=device)
+        dst = torch.empty_like(src)
+        torch.mul(src, 1.0, out=dst)                         # one elementwise kernel: 2^30 bytes in, 2^30 bytes out
+        torch.cuda.synchronize()
+        del src, dst
 
     log("timing p = 1.0 (headline)")
     wall_ms, kernel_ms = time_cdist(kermac, a, b, out, 1.0, False, args.steps, args.warmup)

@@ -7,12 +7,14 @@ and the stream handle.
 from __future__ import annotations
 
 import ctypes
+import os
 import threading
 from ctypes import POINTER, Structure, byref, c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
 from pathlib import Path
 from typing import List, Optional, Sequence, Tuple
 
-LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libkermac_amd.so"
+# KERMAC_AMD_LIBRARY points at another build of the same ABI (e.g. an experimental one).
+LIB_PATH = Path(os.environ.get("KERMAC_AMD_LIBRARY") or Path(__file__).resolve().parent / "_lib" / "libkermac_amd.so")
 
 ABI_VERSION = 1
 

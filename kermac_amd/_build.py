@@ -86,13 +86,18 @@ def _newest_source_mtime() -> float:
     return newest
 
 
-def build(force: bool = True, verbose: bool = False, workers: int | None = None) -> Path:
+def build(force: bool = True, verbose: bool = False, workers: int | None = None,
+          extra_flags: list | None = None, lib_path: Path | None = None) -> Path:
     """Compile every translation unit and link the shared library.
 
     force=False skips objects that are newer than every source file (used while
     developing); the default always recompiles.
     """
     hipcc = _hipcc()
+    extra_flags = list(extra_flags or [])
+    lib_path = Path(lib_path) if lib_path else LIB_PATH
+    if extra_flags:
+        force = True            # objects of a differently-flagged build must not be reused
     OBJ_DIR.mkdir(exist_ok=True)
     LIB_DIR.mkdir(exist_ok=True)
     newest = _newest_source_mtime()
@@ -101,7 +106,7 @@ def build(force: bool = True, verbose: bool = False, workers: int | None = None)
         src, obj, defines = job
         if not force and obj.exists() and obj.stat().st_mtime > newest:
             return obj
-        cmd = [hipcc, *HIPCC_FLAGS, *defines, "-c", str(src), "-o", str(obj)]
+        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, *defines, "-c", str(src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
         proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -113,15 +118,19 @@ def build(force: bool = True, verbose: bool = False, workers: int | None = None)
     with ThreadPoolExecutor(max_workers=workers) as pool:
         objects = list(pool.map(compile_one, _jobs()))
 
-    tmp = LIB_PATH.with_suffix(".so.tmp")
+    lib_path.parent.mkdir(parents=True, exist_ok=True)
+    tmp = lib_path.with_suffix(".so.tmp")
     cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objects), "-lhiprtc"]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, lib_path)
+    if extra_flags:
+        for _, obj, _ in _jobs():       # leave no differently-flagged objects behind
+            obj.unlink(missing_ok=True)
+    return lib_path
 
 
 if __name__ == "__main__":

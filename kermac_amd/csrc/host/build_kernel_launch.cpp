@@ -62,7 +62,8 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
     }
     const int64_t tiles_m = ceil_div(p->m, kmc::BK_TILE_M);
     const int64_t tiles_n = ceil_div(p->n, kmc::BK_TILE_N);
-    if (tiles_m * tiles_n > INT_MAX) return fail(KMC_ERR_INVALID_ARGUMENT, "m x n needs more than 2^31 tiles");
+    const int64_t tiles_n_padded = (tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
+    if (tiles_m * tiles_n_padded > INT_MAX) return fail(KMC_ERR_INVALID_ARGUMENT, "m x n needs more than 2^31 tiles");
 
     args->m = p->m; args->n = p->n; args->k = p->k; args->l = p->l;
     args->a = p->a; args->a_ld = p->a_ld; args->a_bs = p->a_bs;
@@ -83,6 +84,7 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
                   p->c_bs % 4 == 0;
     args->tiles_m = static_cast<int>(tiles_m);
     args->tiles_n = static_cast<int>(tiles_n);
+    args->tiles_n_padded = static_cast<int>(tiles_n_padded);
     *load_a = pick_load_mode(p->a, p->a_ld, p->a_bs, p->a_majorness, p->flags);
     *load_b = pick_load_mode(p->b, p->b_ld, p->b_bs, p->b_majorness, p->flags);
     return KMC_OK;
@@ -139,7 +141,7 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
     if (args.m == 0 || args.n == 0 || args.l == 0) return KMC_OK;
     status = require_gfx950();
     if (status != KMC_OK) return status;
-    const dim3 grid(static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n), args.l, 1);
+    const dim3 grid(static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n_padded), args.l, 1);
     hipError_t e = launch(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail_hip(e, "build_kernel launch");
     return KMC_OK;
@@ -158,7 +160,7 @@ int kmc_build_kernel_jit(void *function, const kmc_build_kernel_params *params, 
     size_t size = sizeof(args);
     void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
     hipError_t e = hipModuleLaunchKernel(static_cast<hipFunction_t>(function),
-                                         static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n),
+                                         static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n_padded),
                                          args.l, 1, kmc::BK_THREADS, 1, 1, 0, static_cast<hipStream_t>(stream), nullptr,
                                          config);
     if (e != hipSuccess) return fail_hip(e, "build_kernel (run-time compiled) launch");

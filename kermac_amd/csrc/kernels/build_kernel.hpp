@@ -43,12 +43,15 @@ struct BuildKernelArgs {
     int outer_power, kernel_type;
     int c_vec;     // c, c_ld and c_bs are multiples of 16 bytes: 128-bit stores allowed
     int tiles_m, tiles_n;
+    int tiles_n_padded;  // tiles_n rounded up to a multiple of 8; grid.x = tiles_m * tiles_n_padded
 };
 
 constexpr int BK_TILE_M = 128;
 constexpr int BK_TILE_N = 128;
 constexpr int BK_TILE_K = 16;
 constexpr int BK_THREADS = 256;
+constexpr int BK_XCDS = 8;     // MI355X: 8 accelerator dies, 32 CUs and one L2 each
+constexpr int BK_BAND_N = 64;  // height, in tiles, of the bands the tile order walks: 8 per XCD
 // Row pitch of an LDS slice in floats.  +4 keeps rows 16-byte aligned and skews
 // the banks so that the transposing (k-contiguous) loaders write conflict-free.
 constexpr int BK_LDS_PITCH = BK_TILE_M + 4;
@@ -305,8 +308,31 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
 
     const int tid = threadIdx.x;
     const int batch = blockIdx.y;
+    // Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin
+    // over the 8 XCDs, each with its own L2, so XCD x runs ids x, x+8, x+16, ...
+    // The tile order walks the output in bands of 64 tiles along n, n fastest:
+    // within a band XCD x therefore owns the 8 n-tiles x, x+8, ..., x+56 and sweeps
+    // m.  The ~100 workgroups resident on an XCD at any time cover roughly 8 x 12
+    // tiles and share their A and B panels through that XCD's L2, while ids are
+    // still handed out in one global order (no XCD can run dry early).  Band
+    // heights are rounded up to a multiple of 8 to keep that ownership in the last
+    // band; the padding workgroups exit at once.
+#ifndef KMC_TILE_ORDER
+#define KMC_TILE_ORDER 1
+#endif
+#if KMC_TILE_ORDER == 0
     const int tile_m = blockIdx.x % args.tiles_m;
     const int tile_n = blockIdx.x / args.tiles_m;
+#else
+    const int linear = blockIdx.x;
+    const int band_tiles = BK_BAND_N * args.tiles_m;
+    const int band = linear / band_tiles;
+    const int band_height = min(BK_BAND_N, args.tiles_n_padded - band * BK_BAND_N);
+    const int in_band = linear - band * band_tiles;
+    const int tile_m = in_band / band_height;
+    const int tile_n = band * BK_BAND_N + in_band % band_height;
+#endif
+    if (tile_n >= args.tiles_n) return;
     const int m0 = tile_m * BK_TILE_M;
     const int n0 = tile_n * BK_TILE_N;
     const int m_valid = args.m - m0;   // rows of A that exist from m0 on (may exceed 128)
