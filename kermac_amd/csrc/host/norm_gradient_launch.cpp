@@ -1,6 +1,6 @@
 // C-ABI entry point for the fused kernel-gradient contraction.
 #include "host_common.hpp"
-#include "../kernels/norm_gradient.hpp"
+#include "../kernels/norm_gradient_mfma.hpp"
 
 using namespace kmc_host;
 
@@ -35,11 +35,14 @@ extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void 
         p->b_bs < 0 || p->c_bs < 0 || p->d_bs < 0 || p->e_bs < 0 || p->p_bs < 0)
         return fail(KMC_ERR_INVALID_ARGUMENT, "negative stride");
 
-    const int o_tile = p->o <= 4 ? 4 : (p->o <= 8 ? 8 : 16);
+    // Up to 8 outputs: vector-ALU kernel (4 or 8 accumulators per (m,n)).  More:
+    // matrix-core kernel with 16 or 32 output columns per workgroup.
+    const int o_tile = p->o <= 4 ? 4 : (p->o <= 8 ? 8 : (p->o <= 16 ? 16 : 32));
+    const bool matrix_core = o_tile >= 16;
     const int o_chunks = ceil_div(p->o, o_tile);
     const int64_t grid_z = static_cast<int64_t>(p->l) * o_chunks;
-    const int tiles_m = ceil_div(p->m, kmc::NG_TILE_M);
-    const int tiles_n = ceil_div(p->n, kmc::NG_TILE_N);
+    const int tiles_m = ceil_div(p->m, matrix_core ? kmc::NGM_TILE_M : kmc::NG_TILE_M);
+    const int tiles_n = ceil_div(p->n, matrix_core ? kmc::NGM_TILE_N : kmc::NG_TILE_N);
     if (grid_z > 65535 || tiles_n > 65535)
         return fail(KMC_ERR_INVALID_ARGUMENT, "grid too large (n tiles %d, batch x o chunks %lld; limit 65535)", tiles_n,
                     static_cast<long long>(grid_z));

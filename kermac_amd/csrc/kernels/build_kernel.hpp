@@ -169,6 +169,61 @@ struct TileLoader {
     }
 };
 
+// One row of the register tile for the two transcendental-free distance kernels,
+// written out as 8 independent subtractions followed by 8 independent
+// accumulations, so that no instruction waits on the one issued just before it
+// (the compiler's own schedule pairs each subtraction with its dependent
+// accumulate; measured on the same board that costs 1 % for |x| and 5 % for x^2).
+#define KMC_SUB8 \
+    "v_sub_f32 %8, %24, %16\n\tv_sub_f32 %9, %24, %17\n\tv_sub_f32 %10, %24, %18\n\tv_sub_f32 %11, %24, %19\n\t" \
+    "v_sub_f32 %12, %24, %20\n\tv_sub_f32 %13, %24, %21\n\tv_sub_f32 %14, %24, %22\n\tv_sub_f32 %15, %24, %23\n\t"
+#define KMC_ROW_OPERANDS(accrow, fa, b) \
+    : "+v"(accrow[0]), "+v"(accrow[1]), "+v"(accrow[2]), "+v"(accrow[3]), "+v"(accrow[4]), "+v"(accrow[5]), \
+      "+v"(accrow[6]), "+v"(accrow[7]), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), \
+      "=&v"(t6), "=&v"(t7) \
+    : "v"(fa[0]), "v"(fa[1]), "v"(fa[2]), "v"(fa[3]), "v"(fa[4]), "v"(fa[5]), "v"(fa[6]), "v"(fa[7]), "v"(b)
+
+__device__ __forceinline__ void row_abs_diff(float (&accrow)[8], const float (&fa)[8], float b)
+{
+    float t0, t1, t2, t3, t4, t5, t6, t7;
+    asm volatile(KMC_SUB8
+                 "v_add_f32 %0, |%8|, %0\n\tv_add_f32 %1, |%9|, %1\n\tv_add_f32 %2, |%10|, %2\n\t"
+                 "v_add_f32 %3, |%11|, %3\n\tv_add_f32 %4, |%12|, %4\n\tv_add_f32 %5, |%13|, %5\n\t"
+                 "v_add_f32 %6, |%14|, %6\n\tv_add_f32 %7, |%15|, %7"
+                 KMC_ROW_OPERANDS(accrow, fa, b));
+}
+
+__device__ __forceinline__ void row_square_diff(float (&accrow)[8], const float (&fa)[8], float b)
+{
+    float t0, t1, t2, t3, t4, t5, t6, t7;
+    asm volatile(KMC_SUB8
+                 "v_fmac_f32 %0, %8, %8\n\tv_fmac_f32 %1, %9, %9\n\tv_fmac_f32 %2, %10, %10\n\t"
+                 "v_fmac_f32 %3, %11, %11\n\tv_fmac_f32 %4, %12, %12\n\tv_fmac_f32 %5, %13, %13\n\t"
+                 "v_fmac_f32 %6, %14, %14\n\tv_fmac_f32 %7, %15, %15"
+                 KMC_ROW_OPERANDS(accrow, fa, b));
+}
+
+// acc[j][i] += inner(fa[i], fb[j]) for the whole 8 x 8 register tile.
+template <int INNER_OP, int INNER_POW>
+__device__ __forceinline__ void rank1_update(
+    float (&acc)[8][8], const float (&fa)[8], const float (&fb)[8], float p_inner, float diff_sign)
+{
+    if (INNER_OP == OP_DIFF && INNER_POW == POW_ABS) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) row_abs_diff(acc[j], fa, fb[j]);
+        return;
+    }
+    if (INNER_OP == OP_DIFF && INNER_POW == POW_SQUARE) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) row_square_diff(acc[j], fa, fb[j]);
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[j][i] += inner_term<INNER_OP, INNER_POW>(fa[i], fb[j], p_inner, diff_sign);
+}
+
 // 8 floats of one LDS row: columns [0,4) and [64,68) relative to p.
 __device__ __forceinline__ void read_fragment(float (&f)[8], const float *p)
 {
@@ -234,19 +289,13 @@ __device__ __forceinline__ void accumulate_tile(
         for (int kk = 0; kk < BK_TILE_K; kk += 2) {
             read_fragment(fa1, sa + (kk + 1) * BK_LDS_PITCH);
             read_fragment(fb1, sb + (kk + 1) * BK_LDS_PITCH);
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-#pragma unroll
-                for (int i = 0; i < 8; i++) acc[j][i] += inner_term<INNER_OP, INNER_POW>(fa0[i], fb0[j], p_inner, diff_sign);
+            rank1_update<INNER_OP, INNER_POW>(acc, fa0, fb0, p_inner, diff_sign);
             // On the last trip this reads row 16: the first row of the other
             // buffer or the pad row.  The values are never used; reading them
             // unconditionally keeps the loop free of register copies.
             read_fragment(fa0, sa + (kk + 2) * BK_LDS_PITCH);
             read_fragment(fb0, sb + (kk + 2) * BK_LDS_PITCH);
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-#pragma unroll
-                for (int i = 0; i < 8; i++) acc[j][i] += inner_term<INNER_OP, INNER_POW>(fa1[i], fb1[j], p_inner, diff_sign);
+            rank1_update<INNER_OP, INNER_POW>(acc, fa1, fb1, p_inner, diff_sign);
         }
 
         if (has_next) {

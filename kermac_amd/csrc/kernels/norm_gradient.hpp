@@ -92,8 +92,20 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
     const bool b_row_valid = stages_b && n0 + bc_row < args.n;
     const bool c_row_valid = stages_c && o0 + bc_row < args.o;
 
+    // Interior workgroup with 16-byte aligned operands and K a multiple of the
+    // slice depth: plain 128-bit loads, nothing to predicate, so the loads of the
+    // next slice stay in flight while the current one is consumed.
+    const bool fast = args.a_vec && args.b_vec && args.c_vec && args.k % 16 == 0 && m0 + NG_TILE_M <= args.m &&
+                      n0 + NG_TILE_N <= args.n && o0 + O_TILE <= args.o;
+    const float *bc_ptr = stages_b ? b_ptr : c_ptr;
+    const bool stages_bc = stages_b || stages_c;
     float4 stage_a, stage_bc;
     auto fetch = [&](int k0) {
+        if (fast) {
+            stage_a = *reinterpret_cast<const float4 *>(a_ptr + (i64)k0 * args.a_ld);
+            if (stages_bc) stage_bc = *reinterpret_cast<const float4 *>(bc_ptr + k0);
+            return;
+        }
         const int k_left = args.k - k0;
         stage_a = a_k < k_left ? load4_guarded(a_ptr + (i64)k0 * args.a_ld, a_m_valid, args.a_vec)
                                : make_float4(0.0f, 0.0f, 0.0f, 0.0f);

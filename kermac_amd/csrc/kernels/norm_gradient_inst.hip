@@ -1,8 +1,9 @@
-// Ahead-of-time instantiations of the kernel-gradient contraction:
-// 3 norm types x 3 output-tile widths.
+// Ahead-of-time instantiations of the kernel-gradient contraction: 3 norm types
+// x (vector-ALU kernel with 4 or 8 outputs per lane tile, matrix-core kernel with
+// 16 or 32 output columns).
 #include <hip/hip_runtime.h>
 
-#include "norm_gradient.hpp"
+#include "norm_gradient_mfma.hpp"
 
 namespace kmc_host {
 
@@ -13,7 +14,8 @@ static hipError_t launch_norm(int o_tile, const kmc::NormGradientArgs &args, dim
     switch (o_tile) {
     case 4: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 4>), grid, block, 0, stream, args); break;
     case 8: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 8>), grid, block, 0, stream, args); break;
-    case 16: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 16>), grid, block, 0, stream, args); break;
+    case 16: hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 1>), grid, block, 0, stream, args); break;
+    case 32: hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 2>), grid, block, 0, stream, args); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
