@@ -103,6 +103,103 @@ def cpu_baseline(a_store_cpu, b_store_cpu, p=1.0, slab=16384):
     return result
 
 
+def calibration_copy(device):
+    """One plain elementwise kernel that reads 2^30 bytes and writes 2^30 bytes."""
+    src = torch.ones(1 << 28, device=device)
+    dst = torch.empty_like(src)
+    torch.mul(src, 1.0, out=dst)
+    torch.cuda.synchronize()
+
+
+def time_call(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return wall_ms, sum(s.elapsed_time(e) for s, e in zip(starts, stops)) / steps
+
+
+def side_line(metric, workload, wall_ms, kernel_ms, ops, algorithmic_bytes, bound, peak, extra, args):
+    achieved = ops / kernel_ms / 1e9
+    return {
+        "metric": metric, "value": round(wall_ms, 3), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 3), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": workload},
+        "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None, "ops_per_launch": ops,
+                     "hbm_gbps": round(algorithmic_bytes / kernel_ms / 1e6, 1)},
+        **extra,
+    }
+
+
+def bench_cdist_grad(kermac, device, args):
+    """x[K=512,N=8192], centres z[512,8192] ~ N(0,1)/sqrt(512), c[16,8192] ~ N(0,1), kernel-gradient weights
+    g[8192,8192] ~ U(0,1), p = 1: in the operator's names a = g [K_ref=8192, M_ref=8192], b = z [N_ref=512, K_ref],
+    c [O=16, K_ref], d = x [N_ref, M_ref], out [O, N_ref, M_ref].  Work (2*O + 3) per (m, n, k)."""
+    torch.manual_seed(3)
+    k_ref, m_ref, n_ref, o = 8192, 8192, 512, 16
+    a = torch.rand(k_ref, m_ref, device=device)
+    b = torch.randn(n_ref, k_ref, device=device) / 512 ** 0.5
+    c = torch.randn(o, k_ref, device=device)
+    d = torch.randn(n_ref, m_ref, device=device) / 512 ** 0.5
+    out = torch.empty(1, o, n_ref, m_ref, device=device)
+    if args.calibration_copy:
+        calibration_copy(device)
+    wall_ms, kernel_ms = time_call(lambda: kermac.cdist_grad(a, b, c, d, out=out, p=1.0), args.steps, args.warmup)
+    ms, ns = slice(0, 48), slice(0, 16)
+    diff = d[ns, ms].double()[:, :, None] - b[ns].double()[:, None, :]
+    sign = torch.where(torch.signbit(diff), -1.0, 1.0).double()
+    truth = torch.einsum("ok,km,nmk->onm", c.double(), a[:, ms].double(), sign)
+    err = ((out[0][:, ns, ms].double() - truth).abs().max() / truth.abs().mean()).item()
+    log(f"cdist_grad p=1: {kernel_ms:.2f} ms kernel, slab max abs err / mean |truth| = {err:.2e}")
+    if err > 1e-4:
+        sys.exit(f"bench.py: cdist_grad parity failure: {err:.3e}")
+    ops = (2.0 * o + 3.0) * m_ref * n_ref * k_ref
+    nbytes = 4.0 * (k_ref * m_ref + n_ref * k_ref + o * k_ref + n_ref * m_ref + o * n_ref * m_ref)
+    return side_line("cdist_grad ms, Laplace-kernel RFM gradient M=8192 N=512 O=16 K=8192 p=1",
+                     "cdist_grad p=1.0 fp32: a[8192,8192] U(0,1), b[512,8192], d[512,8192] N(0,1)/sqrt(512), "
+                     "c[16,8192] N(0,1), out[16,512,8192] (BASELINE configs[3])",
+                     wall_ms, kernel_ms, ops, nbytes, "mfma_fp32", 157.3,
+                     {"parity_max_err_over_mean": err}, args)
+
+
+def bench_kernel_coef(kermac, device, args):
+    """batch 4, x[4,K=256,N=16384], centres z[K=256,M=16384] shared by the batch, U(-1,1); exp(-||x-z||_1/10)
+    contracted with coeffs[4,16384,32] -> out[4,16384,32]; the 16384 x 16384 matrix is never stored."""
+    torch.manual_seed(5)
+    L, k, nx, mz, o = 4, 256, 16384, 16384, 32
+    x = torch.rand(L, k, nx, device=device) * 2 - 1
+    z = torch.rand(k, mz, device=device) * 2 - 1
+    coef = torch.randn(L, mz, o, device=device)
+    out = torch.empty(L, nx, o, device=device)
+    if args.calibration_copy:
+        calibration_copy(device)
+    call = lambda: kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x.transpose(1, 2), z.t(), out=out,
+                                     bandwidth=10.0, coefficients=coef)
+    wall_ms, kernel_ms = time_call(call, args.steps, args.warmup)
+    rows = slice(0, 64)
+    truth = torch.exp(-torch.cdist(x[0, :, rows].t().double(), z.t().double(), p=1.0) / 10.0) @ coef[0].double()
+    err = ((out[0, rows].double() - truth).abs().max() / truth.abs().mean()).item()
+    log(f"kernel x coefficients: {kernel_ms:.2f} ms kernel, slab max abs err / mean |truth| = {err:.2e}")
+    if err > 1e-4:
+        sys.exit(f"bench.py: kernel x coefficients parity failure: {err:.3e}")
+    ops = float(L) * nx * mz * (3 * k + 2 * o)
+    nbytes = 4.0 * (L * k * nx + k * mz + 2 * L * nx * o)
+    return side_line("fused Laplace kernel matrix x coefficients ms, L=4 N=M=16384 K=256 O=32",
+                     "run_kernel(laplace_l1, x[4,16384,256] view, z[16384,256] view, bandwidth=10, "
+                     "coefficients[4,16384,32]) -> out[4,16384,32] (BASELINE configs[4])",
+                     wall_ms, kernel_ms, ops, nbytes, "valu_fp32", 157.3,
+                     {"parity_max_err_over_mean": err}, args)
+
+
 def main():
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--gpus", type=int, default=1)
@@ -110,6 +207,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=2)
     parser.add_argument("--skip-cpu", action="store_true", help="skip the host-CPU baseline leg")
     parser.add_argument("--only-p1", action="store_true", help="time only the headline p = 1.0 configuration")
+    parser.add_argument("--workload", choices=["cdist", "cdist_grad", "kernel_coef"], default="cdist",
+                        help="cdist (default, the headline metric); cdist_grad = the Laplace-kernel RFM gradient "
+                             "configuration; kernel_coef = the fused Laplace kernel matrix x coefficients configuration")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also run one plain elementwise copy kernel over 1 GiB (read 1 GiB, write 1 GiB), so that "
                              "hardware byte counters collected by a profiler can be scaled against a known transfer")
@@ -124,6 +224,10 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.workload != "cdist":
+        line = (bench_cdist_grad if args.workload == "cdist_grad" else bench_kernel_coef)(kermac, device, args)
+        print(json.dumps(line), flush=True)
+        return
     log(f"device: {torch.cuda.get_device_name(0)}; allocating {ALGORITHMIC_BYTES / 1e9:.2f} GB")
     torch.manual_seed(1)
     a_store = torch.randn(K, M, device=device)
@@ -132,11 +236,7 @@ def main():
     a, b, out = a_store.t(), b_store.t(), out_store.t()      # the operator's [M,K] / [N,K] / [M,N] views
 
     if args.calibration_copy:
-        src = torch.ones(1 << 28, device=device)
-        dst = torch.empty_like(src)
-        torch.mul(src, 1.0, out=dst)                         # one elementwise kernel: 2^30 bytes in, 2^30 bytes out
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(device)
 
     log("timing p = 1.0 (headline)")
     wall_ms, kernel_ms = time_cdist(kermac, a, b, out, 1.0, False, args.steps, args.warmup)

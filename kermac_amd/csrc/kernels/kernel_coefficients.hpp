@@ -12,17 +12,20 @@
 // coefficient columns) and walks over all n in tiles of 128:
 //   1. the tile's 128 x 32 block of coefficients is staged in LDS;
 //   2. the tile's kernel values are produced in registers exactly as in
-//      build_kernel (same K walk, same epilogue);
-//   3. they are written to LDS 32 n at a time and contracted: every lane owns
-//      4 rows m x 8 columns o and half of the 32 n, so one pass is 16 steps of
-//      three 128-bit LDS reads and 32 multiply-adds.
-// Step 3 costs 2 x 32 VALU operations per (m, n) against 2 x K for step 2.  The
-// two n-halves are summed through LDS once, at the very end.
+//      build_kernel (same K walk on the vector ALU, same epilogue);
+//   3. they are written to LDS 32 n at a time (into the staging buffers of step
+//      2, which are idle by then) and contracted on the matrix cores:
+//      out[128 m x 32 o] += Kv[128 m x 32 n] * coef[32 n x 32 o] as 16 x 16 x 4
+//      fp32 MFMAs, each wave owning 32 m x 32 o.
+// Step 3 runs on the matrix pipe, so it overlaps with step 2 of the other
+// workgroups resident on the same CU instead of competing for VALU issue slots.
 #pragma once
 
 #include "build_kernel.hpp"
 
 namespace kmc {
+
+typedef float kc_float4 __attribute__((ext_vector_type(4)));
 
 struct KernelCoefficientsArgs {
     BuildKernelArgs kernel;        // c / c_ld / c_bs unused
@@ -35,14 +38,22 @@ struct KernelCoefficientsArgs {
 
 constexpr int KC_COLUMNS = 32;      // coefficient columns per workgroup
 constexpr int KC_PASS_N = 32;       // n per contraction pass
+// [n][m] pitch of the kernel values in LDS: the 4 n-rows an MFMA operand read
+// touches land in 4 disjoint groups of 16 banks.
+constexpr int KC_KV_PITCH = BK_TILE_M + 16;
+constexpr int KC_STAGE_FLOATS = 2 * (2 * BK_LDS_SLICE + BK_LDS_PITCH);
 
 template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
 __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const KernelCoefficientsArgs kc)
 {
-    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE + BK_LDS_PITCH];
-    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE + BK_LDS_PITCH];
-    __shared__ __attribute__((aligned(16))) float lds_kv[KC_PASS_N * BK_LDS_PITCH];   // [n][m]
+    static_assert(KC_PASS_N * KC_KV_PITCH <= KC_STAGE_FLOATS, "kernel values must fit in the staging buffers");
+    // Staging buffers of the K walk; between two K walks the same memory holds
+    // one pass of kernel values.
+    __shared__ __attribute__((aligned(16))) float lds_stage[KC_STAGE_FLOATS];
     __shared__ __attribute__((aligned(16))) float lds_coef[BK_TILE_N * KC_COLUMNS];   // [n][o]
+    float *lds_a = lds_stage;
+    float *lds_b = lds_stage + KC_STAGE_FLOATS / 2;
+    float *lds_kv = lds_stage;
 
     const BuildKernelArgs &args = kc.kernel;
     const int tid = threadIdx.x;
@@ -58,18 +69,21 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
         p_inner = args.p_inner ? args.p_inner[batch * args.p_inner_bs] : args.p_inner_value;
     }
 
-    // Contraction role of this lane: rows 4*row_group .. +3, columns 8*col_group .. +7
-    // (relative to o_base), and the n of parity-half n_half of every pass.
-    const int row_group = tid & 31;
-    const int col_group = (tid >> 5) & 3;
-    const int n_half = tid >> 7;
+    // Contraction role (v_mfma_f32_16x16x4_f32, lane = 16 q + r): wave w owns rows
+    // 32 w .. 32 w + 31 as two row blocks of 16, times two column blocks of 16.
+    // Operand A: lane supplies Kv[m = r][n = q]; operand B: coef[n = q][o = r];
+    // result: lane holds rows 4 q .. 4 q + 3 of column r.
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int q = lane >> 4;
+    const int r = lane & 15;
     const float *coef_batch = kc.coef + batch * kc.coef_bs;
     const bool coef_vec = kc.coef_vec;
-    float out_acc[4][8];
+    kc_float4 out_acc[2][2];   // [row block][column block]
 #pragma unroll
-    for (int r = 0; r < 4; r++)
+    for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-        for (int o = 0; o < 8; o++) out_acc[r][o] = 0.0f;
+        for (int ob = 0; ob < 2; ob++) out_acc[mb][ob] = kc_float4{0.0f, 0.0f, 0.0f, 0.0f};
 
     for (int n0 = 0; n0 < args.n; n0 += BK_TILE_N) {
         const int n_valid = args.n - n0;
@@ -84,11 +98,11 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
             const bool row_live = n_local < n_valid;
             const float *src = coef_batch + (i64)(n0 + n_local) * kc.coef_ld + o_base + c0;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int cols_left = kc.o - (o_base + c0 + 4 * q);
+            for (int v4 = 0; v4 < 4; v4++) {
+                const int cols_left = kc.o - (o_base + c0 + 4 * v4);
                 float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                if (row_live) v = load4_guarded(src + 4 * q, cols_left, coef_vec);
-                *reinterpret_cast<float4 *>(lds_coef + n_local * KC_COLUMNS + c0 + 4 * q) = v;
+                if (row_live) v = load4_guarded(src + 4 * v4, cols_left, coef_vec);
+                *reinterpret_cast<float4 *>(lds_coef + n_local * KC_COLUMNS + c0 + 4 * v4) = v;
             }
         }
 
@@ -112,8 +126,9 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
         if (args.k == 0) __syncthreads();   // no K walk, no barrier: publish lds_coef here
         finish_tile(acc, args, batch, m0, n0, tx, ty);
 
-        // 3. four passes of 32 n.  Pass q holds n_local in [32 q, 32 q + 32); those
-        //    are rows j with (j >> 2) == (q >> 1) of the lanes with (ty >> 3) == (q & 1).
+        // 3. four passes of 32 n.  Pass p holds n_local in [32 p, 32 p + 32): rows j
+        //    with (j >> 2) == (p >> 1) of the lanes with (ty >> 3) == (p & 1).  The K
+        //    walk ended with a barrier, so its staging memory is free.
 #pragma unroll
         for (int pass = 0; pass < BK_TILE_N / KC_PASS_N; pass++) {
             if ((ty >> 3) == (pass & 1)) {
@@ -126,53 +141,45 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
                     for (int h = 0; h < 2; h++) {
                         float4 v = make_float4(acc[j][4 * h], acc[j][4 * h + 1], acc[j][4 * h + 2], acc[j][4 * h + 3]);
                         if (!live) v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                        *reinterpret_cast<float4 *>(lds_kv + n_pass * BK_LDS_PITCH + tx * 4 + h * 64) = v;
+                        *reinterpret_cast<float4 *>(lds_kv + n_pass * KC_KV_PITCH + tx * 4 + h * 64) = v;
                     }
                 }
             }
             __syncthreads();
-            const float *kv_src = lds_kv + row_group * 4;
-            const float *coef_src = lds_coef + pass * KC_PASS_N * KC_COLUMNS + col_group * 8;
-#pragma unroll 4
-            for (int step = 0; step < KC_PASS_N / 2; step++) {
-                const int n_pass = 2 * step + n_half;
-                const float4 kv = *reinterpret_cast<const float4 *>(kv_src + n_pass * BK_LDS_PITCH);
-                const float4 w0 = *reinterpret_cast<const float4 *>(coef_src + n_pass * KC_COLUMNS);
-                const float4 w1 = *reinterpret_cast<const float4 *>(coef_src + n_pass * KC_COLUMNS + 4);
-                const float kvv[4] = {kv.x, kv.y, kv.z, kv.w};
-                const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+            const float *kv_src = lds_kv + q * KC_KV_PITCH + wave * 32 + r;
+            const float *coef_src = lds_coef + (pass * KC_PASS_N + q) * KC_COLUMNS + r;
 #pragma unroll
-                for (int r = 0; r < 4; r++)
+            for (int chunk = 0; chunk < KC_PASS_N / 4; chunk++) {
+                float fa[2], fb[2];
 #pragma unroll
-                    for (int o = 0; o < 8; o++) out_acc[r][o] += kvv[r] * wv[o];
+                for (int mb = 0; mb < 2; mb++) fa[mb] = kv_src[chunk * 4 * KC_KV_PITCH + mb * 16];
+#pragma unroll
+                for (int ob = 0; ob < 2; ob++) fb[ob] = coef_src[chunk * 4 * KC_COLUMNS + ob * 16];
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int ob = 0; ob < 2; ob++)
+                        out_acc[mb][ob] =
+                            __builtin_amdgcn_mfma_f32_16x16x4f32(fa[mb], fb[ob], out_acc[mb][ob], 0, 0, 0);
             }
             __syncthreads();
         }
     }
 
-    // Sum the two n-halves through LDS (lds_kv is free after the last barrier) and store.
-    float *exchange = lds_kv;   // 128 lanes x 32 floats = 4096 <= 32 * 132
-    if (n_half == 1) {
+    // Store: this lane holds rows 32 wave + 16 mb + 4 q + i, column 16 ob + r.
+    float *out_batch = kc.out + batch * kc.out_bs;
 #pragma unroll
-        for (int r = 0; r < 4; r++)
+    for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-            for (int o = 0; o < 8; o++) exchange[(r * 8 + o) * 128 + (tid & 127)] = out_acc[r][o];
-    }
-    __syncthreads();
-    if (n_half == 0) {
-        float *out_batch = kc.out + batch * kc.out_bs;
+        for (int ob = 0; ob < 2; ob++) {
+            const int o = o_base + ob * 16 + r;
+            if (o >= kc.o) continue;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int m_local = row_group * 4 + r;
-            if (m_local >= m_valid) continue;
-            float *dst = out_batch + (i64)(m0 + m_local) * kc.out_ld + o_base + col_group * 8;
-#pragma unroll
-            for (int o = 0; o < 8; o++) {
-                const float total = out_acc[r][o] + exchange[(r * 8 + o) * 128 + (tid & 127)];
-                if (o_base + col_group * 8 + o < kc.o) dst[o] = total;
+            for (int i = 0; i < 4; i++) {
+                const int m_local = wave * 32 + mb * 16 + q * 4 + i;
+                if (m_local < m_valid) out_batch[(i64)(m0 + m_local) * kc.out_ld + o] = out_acc[mb][ob][i];
             }
         }
-    }
 }
 
 }  // namespace kmc
