@@ -54,7 +54,16 @@ enum kmc_flags {
     /* Compute A(m,k) - B(n,k) instead of B(n,k) - A(m,k).  Set by callers that
      * swapped the operands to obtain a row-major result; only matters for the
      * sign-sensitive inner powers (NOOP, SQRT). */
-    KMC_FLAG_NEGATE_DIFF = 2
+    KMC_FLAG_NEGATE_DIFF = 2,
+    /* Only for inner_operator DIFF + inner_power SQUARE: compute the sum of squared
+     * differences as |a|^2 + |b|^2 - 2 a.b with the cross term on the matrix cores
+     * (fp32 MFMA), then recompute with the direct subtract-square-accumulate kernel
+     * every 128 x 128 tile that contains an element below
+     * gram_trust * (|a|^2 + |b|^2) (cancellation).  Two launches on the stream.
+     * Trusted elements carry a relative error of about sqrt(K) * 2^-24 / gram_trust
+     * on the squared distance; repaired tiles are bit-identical to the direct path.
+     * The reference has no such path (include/build_a_kernel.cuh:339-370 is SIMT only). */
+    KMC_FLAG_L2_GRAM = 4
 };
 
 /*
@@ -94,6 +103,7 @@ typedef struct kmc_build_kernel_params {
     int32_t regularization_offset_x;
     int32_t regularization_offset_y;
     float epsilon;
+    float gram_trust;           /* used with KMC_FLAG_L2_GRAM; <= 0 selects 0.25 */
 } kmc_build_kernel_params;
 
 /* Stands in for launch(stream, config, cute_build_kernel<...>, *args)

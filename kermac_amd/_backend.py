@@ -31,6 +31,7 @@ ROW_MAJOR = 1
 
 FLAG_FORCE_SCALAR_ACCESS = 1
 FLAG_NEGATE_DIFF = 2
+FLAG_L2_GRAM = 4
 
 _float_p = c_void_p  # device pointers are passed as integers
 
@@ -50,6 +51,7 @@ class BuildKernelParams(Structure):
         ("regularization", _float_p), ("regularization_bs", c_int64), ("regularization_value", c_float),
         ("regularization_offset_x", c_int32), ("regularization_offset_y", c_int32),
         ("epsilon", c_float),
+        ("gram_trust", c_float),
     ]
 
 

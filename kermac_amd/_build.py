@@ -50,7 +50,7 @@ HOST_SOURCES = [
 
 
 # Device translation units without per-variant defines.
-EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip"]
+EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_inst.hip"]
 
 
 def _hipcc() -> str:

@@ -13,6 +13,7 @@ View convention (torch.cdist's): ``a`` is ``[L?, M, K]``, ``b`` is ``[L?, N, K]`
 """
 from __future__ import annotations
 
+import os
 from enum import Enum, auto
 from itertools import product
 from typing import Any, List, Optional, Union
@@ -181,6 +182,39 @@ def _hyper_parameter(name, value, L, device, require_device):
     return value.data_ptr(), value.stride(0), 0.0, value
 
 
+# How DIFF + SQUARE descriptors (L2 norm, Laplace-L2, Gaussian) are evaluated.
+#   "direct": subtract, square, accumulate on the vector ALU (the reference's arithmetic).
+#   "gram":   |a|^2 + |b|^2 - 2 a.b with the cross term on the matrix cores, and the
+#             direct kernel re-run on every 128 x 128 tile where cancellation makes
+#             that untrustworthy (any element below trust * (|a|^2 + |b|^2)).
+_l2_mode = {"mode": os.environ.get("KERMAC_AMD_L2_MODE", "direct"), "trust": None}
+
+
+def set_l2_mode(mode: str, trust: Optional[float] = None) -> None:
+    """Choose how squared-difference descriptors are evaluated: ``"direct"`` (default)
+    or ``"gram"`` (matrix cores + automatic repair of ill-conditioned tiles).
+
+    ``trust`` (gram only) is the fraction of ``|a|^2 + |b|^2`` below which a squared
+    distance is recomputed directly.  The default keeps the relative error of the
+    squared distance below about 8e-6: ``max(0.25, sqrt(K) * 2**-24 / 8e-6)``.
+    """
+    if mode not in ("direct", "gram"):
+        raise ValueError(f"l2 mode must be 'direct' or 'gram', got {mode!r}")
+    if trust is not None and not trust > 0.0:
+        raise ValueError("trust must be positive")
+    _l2_mode["mode"], _l2_mode["trust"] = mode, trust
+
+
+def get_l2_mode() -> str:
+    return _l2_mode["mode"]
+
+
+def _gram_trust(K: int) -> float:
+    if _l2_mode["trust"] is not None:
+        return float(_l2_mode["trust"])
+    return max(0.25, (K ** 0.5) * 2.0 ** -24 / 8e-6)
+
+
 class _LaunchPlan:
     """Everything needed to launch: the C parameter block, the tensor that will
     be returned, and references that keep device memory alive until launch."""
@@ -315,6 +349,10 @@ def _plan_run_kernel(
     params.a_majorness = _MAJORNESS_ABI[stats_a.majorness]
     params.b_majorness = _MAJORNESS_ABI[stats_b.majorness]
     params.flags = _backend.FLAG_NEGATE_DIFF if swapped else 0
+    if (_l2_mode["mode"] == "gram" and d._inner_operator is InnerOperator.DIFF
+            and d._inner_power is PowerType.SQUARE and stats_c is not None):
+        params.flags |= _backend.FLAG_L2_GRAM
+        params.gram_trust = _gram_trust(K)
     params.m, params.n, params.k, params.l = M, N, K, L
     params.a, params.a_ld, params.a_bs = a.data_ptr(), stats_a.leading_dimension_stride, stats_a.batch_stride
     params.b, params.b_ld, params.b_bs = b.data_ptr(), stats_b.leading_dimension_stride, stats_b.batch_stride

@@ -78,6 +78,8 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
     args->reg_off_y = p->regularization_offset_y;
     args->epsilon = p->epsilon;
     args->diff_sign = (p->flags & KMC_FLAG_NEGATE_DIFF) ? -1.0f : 1.0f;
+    args->repair_only = 0;
+    args->gram_trust = p->gram_trust > 0.0f ? p->gram_trust : 0.25f;
     args->outer_power = p->outer_power;
     args->kernel_type = p->kernel_type;
     args->c_vec = need_c && !(p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) && aligned16(p->c) && p->c_ld % 4 == 0 &&
@@ -100,6 +102,10 @@ kmc_host::build_launcher_fn find_launcher(int inner_operator, int inner_power)
 }
 
 }  // namespace
+
+namespace kmc_host {
+hipError_t launch_gram_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
+}
 
 namespace kmc_host {
 int prepare_build_kernel(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs *args, int *load_a, int *load_b)
@@ -142,6 +148,14 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
     status = require_gfx950();
     if (status != KMC_OK) return status;
     const dim3 grid(static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n_padded), args.l, 1);
+    if (params->flags & KMC_FLAG_L2_GRAM) {
+        if (params->inner_operator != KMC_OP_DIFF || params->inner_power != KMC_POW_SQUARE)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L2_GRAM needs inner_operator DIFF and inner_power SQUARE");
+        // Matrix-core pass over every tile, then the direct kernel over the tiles it marked.
+        hipError_t g = launch_gram_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
+        if (g != hipSuccess) return fail_hip(g, "gram_l2_kernel launch");
+        args.repair_only = 1;
+    }
     hipError_t e = launch(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail_hip(e, "build_kernel launch");
     return KMC_OK;

@@ -44,6 +44,8 @@ struct BuildKernelArgs {
     int c_vec;     // c, c_ld and c_bs are multiples of 16 bytes: 128-bit stores allowed
     int tiles_m, tiles_n;
     int tiles_n_padded;  // tiles_n rounded up to a multiple of 8; grid.x = tiles_m * tiles_n_padded
+    int repair_only;     // recompute only the tiles that carry BK_REPAIR_MARKER (see gram_kernel.hpp)
+    float gram_trust;    // gram_kernel.hpp: distrust d^2 below gram_trust * (|a|^2 + |b|^2)
 };
 
 constexpr int BK_TILE_M = 128;
@@ -105,6 +107,22 @@ struct TileLoader {
         if (MODE == LOAD_COL_SCALAR) return (i64)(2 * i) * ld;
         if (MODE == LOAD_ROW_VEC) return (i64)(i >> 2) * 64 * ld + (i & 3);
         return (i64)(16 * i) * ld;
+    }
+
+    // Row of register i relative to lane_row (a compile-time constant per mode), how
+    // many lanes hold registers of the same row, and this lane's index among them.
+    // Used by kernels that reduce per-row quantities over what the lanes staged.
+    static __device__ __forceinline__ constexpr int row_offset_of(int i)
+    {
+        return MODE == LOAD_COL_VEC ? (i & 3) : MODE == LOAD_COL_SCALAR ? 0 : MODE == LOAD_ROW_VEC ? (i >> 2) * 64 : 16 * i;
+    }
+    static __device__ __forceinline__ constexpr int lanes_per_row()
+    {
+        return MODE == LOAD_COL_VEC ? 8 : MODE == LOAD_COL_SCALAR ? 2 : MODE == LOAD_ROW_VEC ? 4 : 16;
+    }
+    static __device__ __forceinline__ int share_index(int tid)
+    {
+        return MODE == LOAD_COL_VEC ? tid >> 5 : MODE == LOAD_COL_SCALAR ? tid >> 7 : MODE == LOAD_ROW_VEC ? tid & 3 : tid & 15;
     }
 
     // Whole slice inside the matrix: no predicates.
@@ -348,6 +366,33 @@ __device__ __forceinline__ void finish_tile(
     }
 }
 
+// Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin
+// over the 8 XCDs, each with its own L2, so XCD x runs ids x, x+8, x+16, ...
+// The tile order walks the output in bands of 64 tiles along n, n fastest:
+// within a band XCD x therefore owns the 8 n-tiles x, x+8, ..., x+56 and sweeps
+// m.  The ~100 workgroups resident on an XCD at any time cover roughly 8 x 12
+// tiles and share their A and B panels through that XCD's L2, while ids are
+// still handed out in one global order (no XCD can run dry early).  Band
+// heights are rounded up to a multiple of 8 to keep that ownership in the last
+// band; the padding workgroups get `false` and exit at once.
+__device__ __forceinline__ bool tile_of_workgroup(const BuildKernelArgs &args, int &tile_m, int &tile_n)
+{
+    const int linear = blockIdx.x;
+    const int band_tiles = BK_BAND_N * args.tiles_m;
+    const int band = linear / band_tiles;
+    const int band_height = min(BK_BAND_N, args.tiles_n_padded - band * BK_BAND_N);
+    const int in_band = linear - band * band_tiles;
+    tile_m = in_band / band_height;
+    tile_n = band * BK_BAND_N + in_band % band_height;
+    return tile_n < args.tiles_n;
+}
+
+// Marker the matrix-core L2 kernel (gram_kernel.hpp) leaves in the first element
+// of a tile whose result it does not trust: a quiet NaN with a payload no
+// arithmetic produces.  In repair mode the kernel below recomputes exactly the
+// marked tiles.
+constexpr unsigned BK_REPAIR_MARKER = 0x7fc5a5a5u;
+
 template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
 __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs args)
 {
@@ -357,37 +402,19 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
 
     const int tid = threadIdx.x;
     const int batch = blockIdx.y;
-    // Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin
-    // over the 8 XCDs, each with its own L2, so XCD x runs ids x, x+8, x+16, ...
-    // The tile order walks the output in bands of 64 tiles along n, n fastest:
-    // within a band XCD x therefore owns the 8 n-tiles x, x+8, ..., x+56 and sweeps
-    // m.  The ~100 workgroups resident on an XCD at any time cover roughly 8 x 12
-    // tiles and share their A and B panels through that XCD's L2, while ids are
-    // still handed out in one global order (no XCD can run dry early).  Band
-    // heights are rounded up to a multiple of 8 to keep that ownership in the last
-    // band; the padding workgroups exit at once.
-#ifndef KMC_TILE_ORDER
-#define KMC_TILE_ORDER 1
-#endif
-#if KMC_TILE_ORDER == 0
-    const int tile_m = blockIdx.x % args.tiles_m;
-    const int tile_n = blockIdx.x / args.tiles_m;
-#else
-    const int linear = blockIdx.x;
-    const int band_tiles = BK_BAND_N * args.tiles_m;
-    const int band = linear / band_tiles;
-    const int band_height = min(BK_BAND_N, args.tiles_n_padded - band * BK_BAND_N);
-    const int in_band = linear - band * band_tiles;
-    const int tile_m = in_band / band_height;
-    const int tile_n = band * BK_BAND_N + in_band % band_height;
-#endif
-    if (tile_n >= args.tiles_n) return;
+    int tile_m, tile_n;
+    if (!tile_of_workgroup(args, tile_m, tile_n)) return;
     const int m0 = tile_m * BK_TILE_M;
     const int n0 = tile_n * BK_TILE_N;
     const int m_valid = args.m - m0;   // rows of A that exist from m0 on (may exceed 128)
     const int n_valid = args.n - n0;
     const int tx = tid & 15;
     const int ty = tid >> 4;
+
+    if (args.repair_only) {
+        const float first = args.c[batch * args.c_bs + (i64)n0 * args.c_ld + m0];
+        if (__float_as_uint(first) != BK_REPAIR_MARKER) return;   // uniform over the workgroup
+    }
 
     float p_inner = 0.0f;
     if (INNER_POW == POW_POW) {

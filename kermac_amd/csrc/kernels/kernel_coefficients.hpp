@@ -148,19 +148,30 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
             __syncthreads();
             const float *kv_src = lds_kv + q * KC_KV_PITCH + wave * 32 + r;
             const float *coef_src = lds_coef + (pass * KC_PASS_N + q) * KC_COLUMNS + r;
+            // Operand double buffer: reads of chunk c+1 go out before the MFMAs of chunk c.
+            float fa[2][2], fb[2][2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                fa[0][t] = kv_src[t * 16];
+                fb[0][t] = coef_src[t * 16];
+            }
 #pragma unroll
             for (int chunk = 0; chunk < KC_PASS_N / 4; chunk++) {
-                float fa[2], fb[2];
+                const int use = chunk & 1;
+                if (chunk + 1 < KC_PASS_N / 4) {
 #pragma unroll
-                for (int mb = 0; mb < 2; mb++) fa[mb] = kv_src[chunk * 4 * KC_KV_PITCH + mb * 16];
-#pragma unroll
-                for (int ob = 0; ob < 2; ob++) fb[ob] = coef_src[chunk * 4 * KC_COLUMNS + ob * 16];
+                    for (int t = 0; t < 2; t++) {
+                        fa[use ^ 1][t] = kv_src[(chunk + 1) * 4 * KC_KV_PITCH + t * 16];
+                        fb[use ^ 1][t] = coef_src[(chunk + 1) * 4 * KC_COLUMNS + t * 16];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);   // keep those reads above the MFMAs
 #pragma unroll
                 for (int mb = 0; mb < 2; mb++)
 #pragma unroll
                     for (int ob = 0; ob < 2; ob++)
                         out_acc[mb][ob] =
-                            __builtin_amdgcn_mfma_f32_16x16x4f32(fa[mb], fb[ob], out_acc[mb][ob], 0, 0, 0);
+                            __builtin_amdgcn_mfma_f32_16x16x4f32(fa[use][mb], fb[use][ob], out_acc[mb][ob], 0, 0, 0);
             }
             __syncthreads();
         }

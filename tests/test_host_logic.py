@@ -278,6 +278,34 @@ def test_scalar_p_rounding_matches_fp32_division():
     assert plan.params.epsilon == pytest.approx(1e-5)
 
 
+def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
+    a, b = torch.zeros(4, 64), torch.zeros(5, 64)
+    def flags(descriptor, **kw):
+        plan = _plan_run_kernel(descriptor, a, b, None, kw.get("p"), None, None, kw.get("bandwidth"), None, None, 0, 0,
+                                False, require_device=False)
+        return plan.params.flags, plan.params.gram_trust
+    assert flags(kermac.kernel_descriptor_l2_norm)[0] & _backend.FLAG_L2_GRAM == 0
+    kermac.set_l2_mode("gram")
+    try:
+        f, trust = flags(kermac.kernel_descriptor_l2_norm)
+        assert f & _backend.FLAG_L2_GRAM and trust == pytest.approx(0.25)
+        assert flags(kermac.kernel_descriptor_laplace_l2, bandwidth=1.0)[0] & _backend.FLAG_L2_GRAM
+        assert flags(kermac.kernel_descriptor_l1_norm)[0] & _backend.FLAG_L2_GRAM == 0
+        assert flags(kermac.kernel_descriptor_p_norm, p=1.3)[0] & _backend.FLAG_L2_GRAM == 0
+        kermac.set_l2_mode("gram", trust=0.5)
+        assert flags(kermac.kernel_descriptor_l2_norm)[1] == pytest.approx(0.5)
+    finally:
+        kermac.set_l2_mode("direct")
+    # the default trust grows with K so that very long sums fall back to the direct kernel
+    from kermac_amd.build_a_kernel import _gram_trust
+    assert _gram_trust(1024) == pytest.approx(0.25) and _gram_trust(1 << 20) > 2.0
+    # the C ABI refuses the flag for other inner powers
+    params = _backend.BuildKernelParams()
+    params.inner_power, params.flags, params.l = 1, _backend.FLAG_L2_GRAM, 1
+    params.m = params.n = params.k = 0
+    _backend.build_kernel(params, 0)          # empty problem: accepted, nothing launched
+
+
 def interpret_grad_params(p: _backend.NormGradientParams):
     keep = (c_float * 1)(p.p_value)
     _lib.kmo_norm_kernel_gradient(

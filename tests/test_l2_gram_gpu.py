@@ -1,0 +1,119 @@
+"""GPU tests of the opt-in matrix-core path for squared-difference descriptors
+(``kermac_amd.set_l2_mode("gram")``): |a|^2 + |b|^2 - 2 a.b on the MFMA units with
+automatic repair of ill-conditioned tiles by the direct kernel.
+
+Stated tolerance: the same 1e-5 relative to the float64 truth as the direct p = 2
+path -- trusted tiles by the error bound of the expansion, repaired tiles because
+they are recomputed with the direct arithmetic.
+"""
+import pytest
+import torch
+
+import kermac_amd as kermac
+from oracle import oracle
+from tests.helpers import assert_close_to_truth, make_operand
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def gram_mode():
+    kermac.set_l2_mode("gram")
+    yield
+    kermac.set_l2_mode("direct")
+
+
+def test_mode_switch_validation():
+    with pytest.raises(ValueError):
+        kermac.set_l2_mode("fast")
+    with pytest.raises(ValueError):
+        kermac.set_l2_mode("gram", trust=0.0)
+    assert kermac.get_l2_mode() == "direct"
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (128, 128, 16), (129, 127, 17), (300, 515, 70), (1000, 1000, 64),
+                                   (257, 64, 1024)])
+@pytest.mark.parametrize("layout", ["cc", "rr", "cr", "rc"])
+def test_random_data_matches_truth(device, gram_mode, M, N, K, layout):
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
+    a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False)
+    b = make_operand(1, N, K, layout[1] == "c", device, g, batch=False)
+    for c_col in (False, True):
+        out = torch.empty(N, M, device=device).t() if c_col else torch.empty(M, N, device=device)
+        got = kermac.cdist(a, b, out=out, p=2.0)
+        assert_close_to_truth(got, oracle.cdist(a.cpu(), b.cpu(), p=2.0)[0], rtol=1e-5,
+                              what=f"gram {M}x{N}x{K} {layout} out col-major={c_col}")
+
+
+def test_misaligned_operands(device, gram_mode):
+    g = torch.Generator().manual_seed(3)
+    M, N, K = 200, 150, 37
+    flat = torch.randn(K * (M + 3) + 1, generator=g).to(device)
+    a = flat[1:].view(K, M + 3)[:, :M].t()
+    b = torch.randn(N, K + 5, generator=g).to(device)[:, 2:2 + K]
+    got = kermac.cdist(a, b, p=2.0)
+    assert_close_to_truth(got, oracle.cdist(a.cpu(), b.cpu(), p=2.0), rtol=1e-5, what="gram misaligned")
+
+
+def test_near_duplicates_are_repaired(device, gram_mode):
+    # 40 cluster centres far from the origin, points = centre + tiny noise: most
+    # distances inside a cluster are 1e-4 of the norms, hopeless for the expansion.
+    g = torch.Generator().manual_seed(4)
+    K = 96
+    centres = torch.randn(40, K, generator=g) * 3 + 5
+    pts = centres[torch.randint(0, 40, (700,), generator=g)] + 1e-3 * torch.randn(700, K, generator=g)
+    x = pts.to(device)
+    got = kermac.cdist(x, x, p=2.0)[0]
+    truth = oracle.cdist(pts, pts, p=2.0)[0]
+    assert_close_to_truth(got, truth, rtol=1e-5, what="gram clustered")
+    assert torch.all(torch.diagonal(got) == 0), "identical points must give exactly 0"
+    assert torch.equal(got, got.t())
+    # every tile is repaired here, so the result is bit-identical to the direct path
+    kermac.set_l2_mode("direct")
+    assert torch.equal(got, kermac.cdist(x, x, p=2.0)[0])
+
+
+def test_offset_data_falls_back_everywhere(device, gram_mode):
+    g = torch.Generator().manual_seed(5)
+    a = (torch.rand(300, 50, generator=g) + 100).to(device)
+    b = (torch.rand(260, 50, generator=g) + 100).to(device)
+    got = kermac.cdist(a, b, p=2.0)
+    assert_close_to_truth(got, oracle.cdist(a.cpu(), b.cpu(), p=2.0), rtol=1e-5, what="gram offset data")
+
+
+def test_kernels_batches_and_regularisation(device, gram_mode):
+    g = torch.Generator().manual_seed(6)
+    L, N, K = 3, 333, 24
+    data = torch.randn(L, N, K, generator=g).to(device)
+    bw = torch.tensor([2.0, 5.0, 9.0], device=device)
+    got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, data, data, bandwidth=bw, regularization=0.125,
+                            regularization_offset_x=2, regularization_offset_y=0)
+    truth = oracle.build_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", data.cpu(), data.cpu(), bandwidth=bw.cpu(),
+                                regularization=0.125, regularization_offset_x=2, regularization_offset_y=0)
+    assert_close_to_truth(got, truth, rtol=1e-5, what="gram laplace-l2")
+    gaussian = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP,
+                                       kermac.KernelType.GAUSSIAN)
+    got = kermac.run_kernel(gaussian, data, data[0], bandwidth=3.0)
+    truth = oracle.build_kernel("DIFF", "SQUARE", "NOOP", "GAUSSIAN", data.cpu(), data[0].cpu(), bandwidth=3.0)
+    assert_close_to_truth(got, truth, rtol=2e-5, what="gram gaussian")   # exp(-d^2 / 18): doubles the error of d
+    skipped = kermac.cdist(data, data[0], p=2.0, skip_epilogue=True)
+    assert_close_to_truth(skipped, oracle.cdist(data.cpu(), data[0].cpu(), p=2.0, skip_epilogue=True), rtol=1e-5,
+                          atol=1e-4, what="gram squared distances")
+
+
+def test_full_size(device, gram_mode):
+    M = N = 30000
+    K = 1024
+    torch.manual_seed(1)
+    a_store = torch.randn(K, M, device=device)
+    b_store = torch.randn(K, N, device=device)
+    out_store = torch.empty(N, M, device=device)
+    out = kermac.cdist(a_store.t(), b_store.t(), out=out_store.t(), p=2.0)
+    for ms, ns in ((slice(0, 300), slice(0, 2000)), (slice(29900, 30000), slice(29800, 30000))):
+        truth = torch.cdist(a_store.t()[ms].double(), b_store.t()[ns].double(), p=2.0)
+        assert_close_to_truth(out[ms, ns], truth, rtol=1e-5, what="gram slab")
+    assert not torch.isnan(out_store[::128, ::128]).any(), "a repair marker was left behind"
+    del out_store, out
+    self_out = kermac.cdist(a_store.t()[:5000], a_store.t()[:5000], p=2.0)[0]
+    assert torch.all(torch.diagonal(self_out) == 0)
+    assert torch.equal(self_out, self_out.t())
