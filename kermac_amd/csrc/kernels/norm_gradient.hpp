@@ -51,6 +51,33 @@ __device__ __forceinline__ float gradient_weight(float diff, float p_minus_1)
     return fast_pow_abs(__builtin_fabsf(diff), p_minus_1) * sign;
 }
 
+// For the L1 norm only the sign of d - b is needed, and copysign(1, d - b) is
+// negative exactly when d < b or (d, b) = (-0, +0).  Mapping a float to the
+// integer  bits ^ ((bits >> 31) & 0x7fffffff)  turns that rule into one signed
+// integer comparison (-0 maps to -1, +0 to 0, everything else keeps its order),
+// so D and B are held as such keys and a term costs two instructions, compare
+// and select, instead of subtract, sign transfer and multiply.
+__device__ __forceinline__ float sign_order_key(float x)
+{
+    const int bits = __float_as_int(x);
+    return __int_as_float(bits ^ ((bits >> 31) & 0x7fffffff));
+}
+
+// What D and B are replaced by when they enter registers / LDS.
+template <int NORM>
+__device__ __forceinline__ float gradient_operand(float x)
+{
+    return NORM == NORM_L1 ? sign_order_key(x) : x;
+}
+
+// a * g(d - b) with d and b prepared by gradient_operand.
+template <int NORM>
+__device__ __forceinline__ float gradient_term(float a, float d, float b, float p_minus_1)
+{
+    if (NORM == NORM_L1) return __float_as_int(d) < __float_as_int(b) ? -a : a;
+    return a * gradient_weight<NORM>(d - b, p_minus_1);
+}
+
 template <int NORM, int O_TILE>
 __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGradientArgs args)
 {
@@ -117,7 +144,10 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
         *reinterpret_cast<float4 *>(lds_a + (buffer * NG_TILE_K + a_k) * NG_PITCH_A + a_m) = stage_a;
         if (stages_b) {
             float *dst = lds_b + (buffer * NG_TILE_K + bc_k) * NG_PITCH_B + bc_row;
-            dst[0] = stage_bc.x; dst[NG_PITCH_B] = stage_bc.y; dst[2 * NG_PITCH_B] = stage_bc.z; dst[3 * NG_PITCH_B] = stage_bc.w;
+            dst[0] = gradient_operand<NORM>(stage_bc.x);
+            dst[NG_PITCH_B] = gradient_operand<NORM>(stage_bc.y);
+            dst[2 * NG_PITCH_B] = gradient_operand<NORM>(stage_bc.z);
+            dst[3 * NG_PITCH_B] = gradient_operand<NORM>(stage_bc.w);
         } else if (stages_c) {
             float *dst = lds_c + (buffer * NG_TILE_K + bc_k) * O_TILE + bc_row;
             dst[0] = stage_bc.x; dst[O_TILE] = stage_bc.y; dst[2 * O_TILE] = stage_bc.z; dst[3 * O_TILE] = stage_bc.w;
@@ -132,7 +162,7 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int m = m0 + tx * 4 + i;
-            dval[j][i] = (n < args.n && m < args.m) ? d_base[(i64)n * args.d_ld + m] : 0.0f;
+            dval[j][i] = gradient_operand<NORM>((n < args.n && m < args.m) ? d_base[(i64)n * args.d_ld + m] : 0.0f);
         }
     }
 
@@ -158,7 +188,7 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const float t = av[i] * gradient_weight<NORM>(dval[j][i] - bv[j], p_minus_1);
+                const float t = gradient_term<NORM>(av[i], dval[j][i], bv[j], p_minus_1);
 #pragma unroll
                 for (int o = 0; o < O_TILE; o++) acc[j][i][o] += fc[o] * t;
             }

@@ -1,6 +1,6 @@
 // Ahead-of-time instantiations of the kernel-gradient contraction: 3 norm types
 // x (vector-ALU kernel with 4 or 8 outputs per lane tile, matrix-core kernel with
-// 16 or 32 output columns).
+// 16 or 32 output columns, with and without a partial last K slice).
 #include <hip/hip_runtime.h>
 
 #include "norm_gradient_mfma.hpp"
@@ -11,11 +11,18 @@ template <int NORM>
 static hipError_t launch_norm(int o_tile, const kmc::NormGradientArgs &args, dim3 grid, hipStream_t stream)
 {
     const dim3 block(kmc::NG_THREADS);
+    const bool k_tail = args.k % kmc::NGM_TILE_K != 0;
     switch (o_tile) {
     case 4: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 4>), grid, block, 0, stream, args); break;
     case 8: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 8>), grid, block, 0, stream, args); break;
-    case 16: hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 1>), grid, block, 0, stream, args); break;
-    case 32: hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 2>), grid, block, 0, stream, args); break;
+    case 16:
+        if (k_tail) hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 1, true>), grid, block, 0, stream, args);
+        else hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 1, false>), grid, block, 0, stream, args);
+        break;
+    case 32:
+        if (k_tail) hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 2, true>), grid, block, 0, stream, args);
+        else hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 2, false>), grid, block, 0, stream, args);
+        break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -7,7 +7,7 @@
 // this formulation is used when O > 8.  For a fixed n the contraction is a small
 // GEMM: rows = 16 consecutive m, columns = 16 outputs o, depth = k.  Its left
 // operand T does not exist in memory: every lane computes the one element it has
-// to supply (3 VALU instructions: subtract, sign, multiply) right before the
+// to supply (2 to 3 VALU instructions, see gradient_term) right before the
 // v_mfma_f32_16x16x4_f32 that consumes it, so the vector ALU generates operands
 // while the matrix core does the 2*O flops per (m,n,k) that dominate the work.
 //
@@ -36,7 +36,8 @@ constexpr int NGM_THREADS = 256;
 constexpr int NGM_PITCH_A = 80;
 constexpr int NGM_PITCH_B = 16;
 
-template <int NORM, int COLUMN_BLOCKS>
+// K_TAIL = false: K is a multiple of the slice depth, no term needs a select.
+template <int NORM, int COLUMN_BLOCKS, bool K_TAIL>
 __global__ __launch_bounds__(NGM_THREADS) void norm_kernel_gradient_mfma(const NormGradientArgs args)
 {
     constexpr int O_TILE = 16 * COLUMN_BLOCKS;
@@ -102,7 +103,10 @@ __global__ __launch_bounds__(NGM_THREADS) void norm_kernel_gradient_mfma(const N
         *reinterpret_cast<float4 *>(lds_a + (buffer * NGM_TILE_K + a_k) * NGM_PITCH_A + a_m) = stage_a;
         if (stages_b) {
             float *dst = lds_b + (buffer * NGM_TILE_K + bc_k) * NGM_PITCH_B + bc_row;
-            dst[0] = stage_bc.x; dst[NGM_PITCH_B] = stage_bc.y; dst[2 * NGM_PITCH_B] = stage_bc.z; dst[3 * NGM_PITCH_B] = stage_bc.w;
+            dst[0] = gradient_operand<NORM>(stage_bc.x);
+            dst[NGM_PITCH_B] = gradient_operand<NORM>(stage_bc.y);
+            dst[2 * NGM_PITCH_B] = gradient_operand<NORM>(stage_bc.z);
+            dst[3 * NGM_PITCH_B] = gradient_operand<NORM>(stage_bc.w);
         } else if (stages_c) {
             float *dst = lds_c + (buffer * NGM_TILE_K + bc_k) * O_TILE + bc_row;
             dst[0] = stage_bc.x; dst[O_TILE] = stage_bc.y; dst[2 * O_TILE] = stage_bc.z; dst[3 * O_TILE] = stage_bc.w;
@@ -117,7 +121,7 @@ __global__ __launch_bounds__(NGM_THREADS) void norm_kernel_gradient_mfma(const N
 #pragma unroll
         for (int mb = 0; mb < 4; mb++) {
             const int m = m0 + mb * 16 + r;
-            dval[nb][mb] = (n < args.n && m < args.m) ? d_base[(i64)n * args.d_ld + m] : 0.0f;
+            dval[nb][mb] = gradient_operand<NORM>((n < args.n && m < args.m) ? d_base[(i64)n * args.d_ld + m] : 0.0f);
         }
     }
 
@@ -162,8 +166,8 @@ __global__ __launch_bounds__(NGM_THREADS) void norm_kernel_gradient_mfma(const N
             for (int nb = 0; nb < 4; nb++)
 #pragma unroll
                 for (int mb = 0; mb < 4; mb++) {
-                    float t = fa[mb] * gradient_weight<NORM>(dval[nb][mb] - fb[nb], p_minus_1);
-                    if (k_here < NGM_TILE_K) t = k_real ? t : 0.0f;
+                    float t = gradient_term<NORM>(fa[mb], dval[nb][mb], fb[nb], p_minus_1);
+                    if (K_TAIL) t = k_real ? t : 0.0f;
 #pragma unroll
                     for (int cb = 0; cb < COLUMN_BLOCKS; cb++)
                         acc[nb][mb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(t, fc[cb], acc[nb][mb][cb], 0, 0, 0);

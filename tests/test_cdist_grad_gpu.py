@@ -107,6 +107,31 @@ def test_gradient_sign_convention_and_linearity(device):
     assert_close_to_truth(f(c1 + c2), f(c1) + f(c2), rtol=1e-4, atol=1e-4, what="linearity in c")
 
 
+@pytest.mark.parametrize("O", [1, 8, 16, 32])
+@pytest.mark.parametrize("K", [3, 16, 35])
+def test_gradient_l1_sign_of_zero_differences(device, O, K):
+    """copysign(1, d - b) for the four combinations of signed zeros, equal non-zero
+    values, denormals and ordinary values, in every kernel variant (vector-ALU and
+    matrix-core, with and without a partial K slice): d - b is -0 only for
+    (d, b) = (-0, +0); the result must equal the oracle bit for bit because every
+    product c * a below is a small integer."""
+    g = torch.Generator().manual_seed(93 + O + K)
+    specials = torch.tensor([0.0, -0.0, 1.5, -1.5, 1e-45, -1e-45, 3e-39, -3e-39, float(2 ** -126), 7.0])
+    M, N = 70, 2 * len(specials)
+    d = specials[torch.randint(len(specials), (N, M), generator=g)]
+    b = specials[torch.randint(len(specials), (N, K), generator=g)]
+    a = torch.randint(-3, 4, (K, M), generator=g).float()
+    c = torch.randint(-2, 3, (O, K), generator=g).float()
+    got = kermac.cdist_grad(a.to(device), b.to(device), c.to(device), d.to(device), p=1.0)
+    truth = oracle.cdist_grad(a, b, c, d, p=1.0)
+    assert torch.equal(got.cpu().double(), truth.double())
+    # and the rule itself, independent of the oracle
+    diff = d[:, :, None] - b[:, None, :]                                    # [n, m, k], IEEE fp32
+    sign = torch.where(torch.signbit(diff), -1.0, 1.0)
+    expected = torch.einsum("ok,km,nmk->onm", c, a, sign)
+    assert torch.equal(got[0].cpu(), expected)
+
+
 def test_gradient_rfm_shape_against_slab_truth(device):
     """The Laplace-kernel RFM gradient configuration (x[512,8192], centres
     z[512,8192], 16 classes, 8192 centres) at p = 1: check float64 slabs."""
