@@ -114,6 +114,11 @@ class BackendError(RuntimeError):
         self.status = status
 
 
+class WrongDeviceError(BackendError, ValueError):
+    """The current device is not a gfx950.  Also a ValueError, like the reference's
+    rejection of an unsupported compute capability (src/kermac/module_cache/module_cache.py:166-167)."""
+
+
 _lib = None
 _lib_lock = threading.Lock()
 
@@ -147,6 +152,8 @@ def last_error() -> str:
 
 
 def check(status: int) -> None:
+    if status == ERR_WRONG_DEVICE:
+        raise WrongDeviceError(status, last_error())
     if status != OK:
         raise BackendError(status, last_error())
 

@@ -369,3 +369,8 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     grad.norm_type = 9
     with pytest.raises(_backend.BackendError):
         _backend.norm_kernel_gradient(grad, 0)
+    # a device that is not a gfx950 is a ValueError, as an unsupported compute capability is in
+    # the reference (src/kermac/module_cache/module_cache.py:166-167), and still a BackendError
+    with pytest.raises(ValueError) as info:
+        _backend.check(_backend.ERR_WRONG_DEVICE)
+    assert isinstance(info.value, _backend.BackendError) and info.value.status == _backend.ERR_WRONG_DEVICE
