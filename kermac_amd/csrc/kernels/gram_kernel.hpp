@@ -19,8 +19,8 @@
 // subtract-square-accumulate arithmetic.  Trusted tiles keep a relative error of
 // at most about sqrt(K) * 2^-24 / gram_trust on d^2.
 //
-// Tiling: workgroup 256 lanes = 2 x 2 waves, tile 128 x 128, K slices of 16 staged
-// exactly like the direct kernel (same loaders, same LDS layout).  A wave owns
+// Tiling: workgroup 256 lanes = 2 x 2 waves, tile 128 x 128, K staged through LDS
+// with the loaders and the layout of the direct kernel, two of its slices at a time.  A wave owns
 // 64 x 64 as 2 x 2 MFMA tiles of 32 x 32.  Operand layouts (lane = 32 h + i):
 //   A (32 x 2): lane supplies A[row i][k h];  B (2 x 32): lane supplies B[k h][column i]
 //   D (32 x 32): register v of the lane is D[row 8 (v/4) + 4 h + v%4][column i]
@@ -64,8 +64,21 @@ __device__ __forceinline__ void row_norms(
     }
 }
 
+// Loader slices (of BK_TILE_K = 16 k) per pipeline stage.  One stage is what sits
+// between two barriers and what the global loads run ahead by: at 32 k a stage
+// keeps the matrix pipe busy for about 1.8 us, longer than a global load that
+// misses the L2 takes, and there are half as many barriers as with 16.
+#ifndef GRAM_DEPTH
+#define GRAM_DEPTH 1
+#endif
+#ifndef GRAM_WAVES
+#define GRAM_WAVES 4
+#endif
+constexpr int GRAM_STAGE_K = GRAM_DEPTH * BK_TILE_K;
+constexpr int GRAM_STAGE_FLOATS = GRAM_DEPTH * BK_LDS_SLICE;   // per operand and buffer
+
 // The K walk of one tile: stage slices through LDS (double buffered, loads of
-// slice t+1 in flight while slice t is consumed), feed the matrix cores, and keep
+// stage t+1 in flight while stage t is consumed), feed the matrix cores, and keep
 // per-register sums of squares of everything staged.  FULL = no load needs a
 // predicate.  Ends with a barrier.
 template <int LOAD_A, int LOAD_B, bool FULL>
@@ -76,44 +89,52 @@ __device__ __forceinline__ void gram_walk(
 {
     const int k_slices = (k_total + BK_TILE_K - 1) / BK_TILE_K;
     const int k_tail = k_total - (k_slices - 1) * BK_TILE_K;
-    float stage_a[8], stage_b[8];
+    const int stages = (k_slices + GRAM_DEPTH - 1) / GRAM_DEPTH;
+    float stage_a[GRAM_DEPTH][8], stage_b[GRAM_DEPTH][8];
 
-    auto fetch = [&](int slice) {
-        if (FULL) {
-            load_a.load_full(stage_a);
-            load_b.load_full(stage_b);
-        } else {
-            const int kv = slice + 1 == k_slices ? k_tail : BK_TILE_K;
-            load_a.load_edge(stage_a, m_valid, kv);    // zero fill: adds 0 to norms and dot products
-            load_b.load_edge(stage_b, n_valid, kv);
+    // The loaders point at the next slice to fetch and move on after every fetch.
+    auto fetch = [&](int stage) {
+#pragma unroll
+        for (int d = 0; d < GRAM_DEPTH; d++) {
+            if (FULL) {
+                load_a.load_full(stage_a[d]);
+                load_b.load_full(stage_b[d]);
+            } else {
+                const int slice = stage * GRAM_DEPTH + d;
+                // slices past the end: k_valid 0, nothing is dereferenced, zeros are staged
+                const int kv = slice + 1 < k_slices ? BK_TILE_K : (slice + 1 == k_slices ? k_tail : 0);
+                load_a.load_edge(stage_a[d], m_valid, kv);    // zero fill: adds 0 to norms and dot products
+                load_b.load_edge(stage_b[d], n_valid, kv);
+            }
+            load_a.advance();
+            load_b.advance();
         }
     };
     auto commit = [&](int buffer) {
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            square_a[s] += stage_a[s] * stage_a[s];
-            square_b[s] += stage_b[s] * stage_b[s];
+        for (int d = 0; d < GRAM_DEPTH; d++) {
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                square_a[s] += stage_a[d][s] * stage_a[d][s];
+                square_b[s] += stage_b[d][s] * stage_b[d][s];
+            }
+            load_a.store(lds_a + buffer * GRAM_STAGE_FLOATS + d * BK_LDS_SLICE, stage_a[d]);
+            load_b.store(lds_b + buffer * GRAM_STAGE_FLOATS + d * BK_LDS_SLICE, stage_b[d]);
         }
-        load_a.store(lds_a + buffer * BK_LDS_SLICE, stage_a);
-        load_b.store(lds_b + buffer * BK_LDS_SLICE, stage_b);
     };
 
-    if (k_slices > 0) {
+    if (stages > 0) {
         fetch(0);
         commit(0);
     }
     __syncthreads();
 
-    for (int slice = 0; slice < k_slices; slice++) {
-        const int cur = slice & 1;
-        const bool has_next = slice + 1 < k_slices;
-        if (has_next) {
-            load_a.advance();
-            load_b.advance();
-            fetch(slice + 1);
-        }
-        const float *sa = frag_a + cur * BK_LDS_SLICE;
-        const float *sb = frag_b + cur * BK_LDS_SLICE;
+    for (int stage = 0; stage < stages; stage++) {
+        const int cur = stage & 1;
+        const bool has_next = stage + 1 < stages;
+        if (has_next) fetch(stage + 1);
+        const float *sa = frag_a + cur * GRAM_STAGE_FLOATS;
+        const float *sb = frag_b + cur * GRAM_STAGE_FLOATS;
         // Operand double buffer: the LDS reads of pair p+1 are issued before the
         // four MFMAs of pair p, so the matrix pipe never waits for LDS latency.
         float fa[2][2], fb[2][2];
@@ -123,9 +144,9 @@ __device__ __forceinline__ void gram_walk(
             fb[0][t] = sb[t * 32];
         }
 #pragma unroll
-        for (int pair = 0; pair < BK_TILE_K / 2; pair++) {
+        for (int pair = 0; pair < GRAM_STAGE_K / 2; pair++) {
             const int use = pair & 1;
-            if (pair + 1 < BK_TILE_K / 2) {
+            if (pair + 1 < GRAM_STAGE_K / 2) {
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     fa[use ^ 1][t] = sa[(pair + 1) * 2 * BK_LDS_PITCH + t * 32];
@@ -147,10 +168,10 @@ __device__ __forceinline__ void gram_walk(
 }
 
 template <int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(BK_THREADS, 2) void gram_l2_kernel(const BuildKernelArgs args)
+__global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const BuildKernelArgs args)
 {
-    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE];
-    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE];
+    __shared__ __attribute__((aligned(16))) float lds_a[2 * GRAM_STAGE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds_b[2 * GRAM_STAGE_FLOATS];
     __shared__ float lds_norm_a[BK_TILE_M];
     __shared__ float lds_norm_b[BK_TILE_N];
 
@@ -188,7 +209,7 @@ __global__ __launch_bounds__(BK_THREADS, 2) void gram_l2_kernel(const BuildKerne
 
     const float *frag_a = lds_a + h * BK_LDS_PITCH + wave_m + i;
     const float *frag_b = lds_b + h * BK_LDS_PITCH + wave_n + i;
-    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
+    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % GRAM_STAGE_K == 0) {
         gram_walk<LOAD_A, LOAD_B, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
                                         args.k, m_valid, n_valid);
     } else {
@@ -218,26 +239,39 @@ __global__ __launch_bounds__(BK_THREADS, 2) void gram_l2_kernel(const BuildKerne
     const bool regularize = kernel_type != KERNEL_NONE && regularization != 0.0f;
     const float diagonal_value = 1.0f + regularization;
 
+    // d^2, trust check, epilogue.  Loop order: one norm of a per (mt, v), used for both
+    // column tiles, so that only a few of the 32 norms a lane needs are live (with the
+    // column tile outermost the kernel needs 206 registers instead of 127).  The
+    // square root is the hardware one (1 ulp; this path's tolerance is 1e-5 anyway),
+    // the rest is the general routine of the direct kernel.
+    const int outer_rest = outer_power == POW_SQRT ? POW_NOOP : outer_power;
     int distrust = 0;
+    float norm_b[2];
+    int n_local[2];
 #pragma unroll
     for (int nt = 0; nt < 2; nt++) {
-        const int n_local = wave_n + nt * 32 + i;
-        const float norm_b = lds_norm_b[n_local];
+        n_local[nt] = wave_n + nt * 32 + i;
+        norm_b[nt] = lds_norm_b[n_local[nt]];
+    }
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++)
+    for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m_local = wave_m + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-                const float norms = lds_norm_a[m_local] + norm_b;
+        for (int v = 0; v < 16; v++) {
+            const int m_local = wave_m + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+            const float norm_a = lds_norm_a[m_local];
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++) {
+                const float norms = norm_a + norm_b[nt];
                 float d2 = norms - 2.0f * acc[mt][nt][v];
                 // NaN compares false: a NaN result is stored as is, not repaired.
-                if (m_local < m_valid && n_local < n_valid && d2 < args.gram_trust * norms) distrust = 1;
+                if (m_local < m_valid && n_local[nt] < n_valid && d2 < args.gram_trust * norms) distrust = 1;
                 d2 = fmaxf(d2, 0.0f);
-                float value = epilogue_value(d2, outer_power, kernel_type, p_outer, neg_gamma, args.epsilon);
-                if (regularize && args.reg_off_x + m0 + m_local == args.reg_off_y + n0 + n_local) value = diagonal_value;
+                if (outer_power == POW_SQRT) d2 = __builtin_amdgcn_sqrtf(d2);
+                float value = epilogue_value(d2, outer_rest, kernel_type, p_outer, neg_gamma, args.epsilon);
+                if (regularize && args.reg_off_x + m0 + m_local == args.reg_off_y + n0 + n_local[nt]) value = diagonal_value;
                 acc[mt][nt][v] = value;
             }
-    }
+        }
     const bool repair = __syncthreads_or(distrust) != 0;
 
     float *c_tile = args.c + batch * args.c_bs;
