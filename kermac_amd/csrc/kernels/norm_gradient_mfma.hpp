@@ -172,6 +172,11 @@ __global__ __launch_bounds__(NGM_THREADS) void norm_kernel_gradient_mfma(const N
                     for (int cb = 0; cb < COLUMN_BLOCKS; cb++)
                         acc[nb][mb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(t, fc[cb], acc[nb][mb][cb], 0, 0, 0);
                 }
+            // Keeps the scheduler from hoisting the operand reads of later chunks above
+            // this one: with them hoisted the kernel needs 136 registers, without 128,
+            // which is the step from 3 to 4 waves per SIMD (10.2 -> 9.95 ms at the
+            // benchmark shape, same board).
+            __builtin_amdgcn_sched_barrier(0);
         }
 
         if (has_next) commit(cur ^ 1);
