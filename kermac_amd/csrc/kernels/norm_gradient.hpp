@@ -212,8 +212,11 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
         const int k_here = min(NG_TILE_K, args.k - slice * NG_TILE_K);
         if (k_here == NG_TILE_K) {
             // Full slice: two k-steps per trip with the next fragments requested
-            // before the current ones are consumed.  Kept rolled so that the
-            // register count stays low enough for two waves per SIMD.
+            // before the current ones are consumed.  Kept rolled, and for the L1 and
+            // L2 norms fenced so that the scheduler leaves each group of reads one
+            // step ahead of its use instead of gathering all reads of a trip at the
+            // top, which exposes the LDS latency once per trip (O = 8, same board:
+            // 7.68 -> 7.38 ms; the fractional norm is 3 % faster without fences).
             float4 fa0 = *reinterpret_cast<const float4 *>(sa);
             float2 fb0 = *reinterpret_cast<const float2 *>(sb);
             float fc0[O_TILE], fc1[O_TILE];
@@ -223,13 +226,17 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
                 const float4 fa1 = *reinterpret_cast<const float4 *>(sa + (kk + 1) * NG_PITCH_A);
                 const float2 fb1 = *reinterpret_cast<const float2 *>(sb + (kk + 1) * NG_PITCH_B);
                 read_c(fc1, sc + (kk + 1) * O_TILE);
+                if (NORM != NORM_P) __builtin_amdgcn_sched_barrier(0);
                 step(fa0, fb0, fc0);
+                if (NORM != NORM_P) __builtin_amdgcn_sched_barrier(0);
                 // kk + 2 == 16 reads the first row of the other buffer / the pad
                 // row; those values are never used.
                 fa0 = *reinterpret_cast<const float4 *>(sa + (kk + 2) * NG_PITCH_A);
                 fb0 = *reinterpret_cast<const float2 *>(sb + (kk + 2) * NG_PITCH_B);
                 read_c(fc0, sc + (kk + 2) * O_TILE);
+                if (NORM != NORM_P) __builtin_amdgcn_sched_barrier(0);
                 step(fa1, fb1, fc1);
+                if (NORM != NORM_P) __builtin_amdgcn_sched_barrier(0);
             }
         } else {
             // K tail: only the k that exist, so that g(d - 0) * 0 of a padded k
