@@ -35,7 +35,8 @@ HIPCC_FLAGS = [
 
 # (inner operator, inner power) pairs compiled ahead of time; must match
 # csrc/host/launcher_table.cpp.
-AOT_BUILD_KERNEL_VARIANTS = [(0, 0), (0, 1), (0, 2), (0, 4), (1, 0)]
+# (0, 5) .. (0, 8) are the special exponents 0.5, 1.5, 3, 4 the library substitutes for (0, 4).
+AOT_BUILD_KERNEL_VARIANTS = [(0, 0), (0, 1), (0, 2), (0, 4), (0, 5), (0, 6), (0, 7), (0, 8), (1, 0)]
 
 # Pairs compiled ahead of time for the fused kernel-matrix x coefficients kernel.
 AOT_COEFFICIENT_VARIANTS = [(0, 1), (0, 2), (0, 4)]

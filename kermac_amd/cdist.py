@@ -32,7 +32,9 @@ def cdist(
         a: ``[L?, M, K]`` fp32 on the GPU, row- or column-major.
         b: ``[L?, N, K]`` fp32 on the GPU.
         out: optional ``[L?, M, N]`` fp32 result, written in place and returned.
-        p: norm order; 1.0 and 2.0 take paths without transcendental functions.
+        p: norm order; 1.0 and 2.0 take paths without transcendental functions,
+            3.0 and 4.0 too, 0.5 and 1.5 need one square root per term; any other
+            value costs a log2 and an exp2 per term.
         skip_epilogue: return ``sum_k |b - a|**p``.
         try_to_align: accepted for compatibility; aligned operands always use
             128-bit accesses.

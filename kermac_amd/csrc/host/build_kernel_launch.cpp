@@ -118,7 +118,8 @@ extern "C" {
 
 int kmc_build_kernel_has_variant(int32_t inner_operator, int32_t inner_power)
 {
-    return find_launcher(inner_operator, inner_power) != nullptr;
+    // the special exponents (device_common.hpp, SpecialPower) are internal, not variants a caller can ask for
+    return inner_power <= KMC_POW_POW && find_launcher(inner_operator, inner_power) != nullptr;
 }
 
 int kmc_build_kernel_load_modes(const kmc_build_kernel_params *params, int32_t *load_a, int32_t *load_b)
@@ -138,7 +139,16 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
     int load_a = 0, load_b = 0;
     int status = prepare(params, true, &args, &load_a, &load_b);
     if (status != KMC_OK) return status;
-    kmc_host::build_launcher_fn launch = find_launcher(params->inner_operator, params->inner_power);
+    int inner_power = params->inner_power;
+    if (params->inner_operator == KMC_OP_DIFF && inner_power == KMC_POW_POW && !params->p_inner &&
+        !(params->flags & KMC_FLAG_GENERIC_POWER)) {
+        // Scalar exponents with a cheaper exact form (device_common.hpp, SpecialPower).
+        const float p = params->p_inner_value;
+        const int special = p == 0.5f ? kmc::POW_ABS_HALF : p == 1.5f ? kmc::POW_ABS_THREE_HALVES
+                          : p == 3.0f ? kmc::POW_ABS_CUBE : p == 4.0f ? kmc::POW_ABS_FOURTH : inner_power;
+        if (find_launcher(params->inner_operator, special)) inner_power = special;
+    }
+    kmc_host::build_launcher_fn launch = find_launcher(params->inner_operator, inner_power);
     if (!launch) {
         return fail(KMC_ERR_UNSUPPORTED_VARIANT,
                     "inner_operator=%d inner_power=%d is not compiled ahead of time; compile it at run time",

@@ -17,6 +17,10 @@ KMC_DECLARE_BUILD(0, 0)  // DIFF, NOOP
 KMC_DECLARE_BUILD(0, 1)  // DIFF, ABS      (L1 norm, Laplace-L1)
 KMC_DECLARE_BUILD(0, 2)  // DIFF, SQUARE   (L2 norm, Laplace-L2, Gaussian)
 KMC_DECLARE_BUILD(0, 4)  // DIFF, POW      (fractional p norm)
+KMC_DECLARE_BUILD(0, 5)  // DIFF, |x|^0.5  (substituted for POW with a scalar exponent, see device_common.hpp)
+KMC_DECLARE_BUILD(0, 6)  // DIFF, |x|^1.5
+KMC_DECLARE_BUILD(0, 7)  // DIFF, |x|^3
+KMC_DECLARE_BUILD(0, 8)  // DIFF, |x|^4
 KMC_DECLARE_BUILD(1, 0)  // DOT,  NOOP     (plain a @ b.T)
 
 KMC_DECLARE_COEF(0, 1)
@@ -28,6 +32,10 @@ const BuildLauncher build_launchers[] = {
     {0, 1, launch_build_kernel_0_1},
     {0, 2, launch_build_kernel_0_2},
     {0, 4, launch_build_kernel_0_4},
+    {0, 5, launch_build_kernel_0_5},
+    {0, 6, launch_build_kernel_0_6},
+    {0, 7, launch_build_kernel_0_7},
+    {0, 8, launch_build_kernel_0_8},
     {1, 0, launch_build_kernel_1_0},
 };
 const int build_launcher_count = sizeof(build_launchers) / sizeof(build_launchers[0]);

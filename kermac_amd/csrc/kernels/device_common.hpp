@@ -14,6 +14,10 @@ namespace kmc {
 // Reference enums: include/kermac_internal_common.cuh:41-74.
 enum InnerOperator : int { OP_DIFF = 0, OP_DOT = 1 };
 enum PowerType : int { POW_NOOP = 0, POW_ABS = 1, POW_SQUARE = 2, POW_SQRT = 3, POW_POW = 4 };
+// Not part of the C ABI: inner powers the host substitutes for POW_POW when the
+// exponent is a scalar equal to 0.5, 1.5, 3 or 4.  |x|^p then needs one square
+// root or none instead of a logarithm and an exponential.
+enum SpecialPower : int { POW_ABS_HALF = 5, POW_ABS_THREE_HALVES = 6, POW_ABS_CUBE = 7, POW_ABS_FOURTH = 8 };
 enum KernelType : int { KERNEL_NONE = 0, KERNEL_LAPLACE = 1, KERNEL_GAUSSIAN = 2 };
 enum NormType : int { NORM_L1 = 0, NORM_L2 = 1, NORM_P = 2 };
 
@@ -52,7 +56,12 @@ __device__ __forceinline__ float inner_term(float a, float b, float p_inner, flo
     if (INNER_POW == POW_ABS) return __builtin_fabsf(t);
     if (INNER_POW == POW_SQUARE) return t * t;
     if (INNER_POW == POW_SQRT) return __builtin_amdgcn_sqrtf(t);
-    return fast_pow_abs(__builtin_fabsf(t), p_inner);
+    const float x = __builtin_fabsf(t);
+    if (INNER_POW == POW_ABS_HALF) return __builtin_amdgcn_sqrtf(x);
+    if (INNER_POW == POW_ABS_THREE_HALVES) return x * __builtin_amdgcn_sqrtf(x);
+    if (INNER_POW == POW_ABS_CUBE) return x * (t * t);
+    if (INNER_POW == POW_ABS_FOURTH) return (t * t) * (t * t);
+    return fast_pow_abs(x, p_inner);
 }
 
 // Epilogue of one accumulator: outer power, epsilon mask, kernel function.

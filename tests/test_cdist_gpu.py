@@ -209,6 +209,35 @@ def test_run_kernel_batched_hyper_parameters(device):
     assert_close_to_truth(out, truth, rtol=1e-4, what="gaussian p-norm")
 
 
+@pytest.mark.parametrize("p", [0.5, 1.5, 3.0, 4.0])
+def test_scalar_exponents_with_exact_forms(device, p):
+    """A float exponent of 0.5, 1.5, 3 or 4 is evaluated as sqrt|x|, |x| sqrt|x|,
+    |x| x^2, (x^2)^2 inside the library; the same exponent as a tensor takes the
+    generic exp2(p log2|x|).  Both must meet the fractional-p tolerance against the
+    float64 oracle, for every layout, ragged shapes, zeros and the kernel epilogues."""
+    g = torch.Generator().manual_seed(int(p * 10) + 83)
+    for (M, N, K), a_col, b_col in (((300, 170, 70), True, True), ((129, 257, 33), False, False),
+                                    ((64, 200, 16), True, False)):
+        a = make_operand(1, M, K, a_col, device, g, batch=False)
+        b = make_operand(1, N, K, b_col, device, g, batch=False)
+        b[:3] = a[:3]                                                # exact zeros among the differences
+        truth = oracle.cdist(a.cpu(), b.cpu(), p=p)
+        special = kermac.cdist(a, b, p=p)
+        assert_close_to_truth(special, truth, rtol=1e-4, what=f"exact form p={p} {M}x{N}x{K}")
+        generic = kermac.run_kernel(kermac.kernel_descriptor_p_norm, a, b, p=torch.tensor(p, device=device))
+        assert_close_to_truth(generic, truth, rtol=1e-4, what=f"generic power p={p}")
+        assert_close_to_truth(special, generic.double(), rtol=2e-5, what=f"exact form vs generic p={p}")
+        skipped = kermac.cdist(a, b, p=p, skip_epilogue=True)
+        assert_close_to_truth(skipped, truth.double() ** p, rtol=1e-4, what=f"skip_epilogue p={p}")
+    desc = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.POW, kermac.PowerType.POW,
+                                   kermac.KernelType.LAPLACE)
+    out = kermac.run_kernel(desc, a, b, p=p, bandwidth=5.0)
+    truth = oracle.build_kernel("DIFF", "POW", "POW", "LAPLACE", a.cpu(), b.cpu(), p_inner=p, p_outer=1.0 / p,
+                                bandwidth=5.0)
+    # exp(-d / bw) turns a relative error of d into d / bw times as much: absolute floor for tiny values
+    assert_close_to_truth(out, truth, rtol=1e-4, atol=1e-7, what=f"laplace on the {p}-norm")
+
+
 def test_run_kernel_epsilon_mask(device):
     a = torch.zeros(1, 2, device=device)
     b = torch.tensor([[1e-6, 0.0], [1.0, 0.0]], device=device)
