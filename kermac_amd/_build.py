@@ -128,10 +128,27 @@ def build(force: bool = True, verbose: bool = False, workers: int | None = None,
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
     os.replace(tmp, lib_path)
+    if lib_path == LIB_PATH:
+        build_c_example(verbose=verbose)
     if extra_flags:
         for _, obj, _ in _jobs():       # leave no differently-flagged objects behind
             obj.unlink(missing_ok=True)
     return lib_path
+
+
+def build_c_example(verbose: bool = False) -> Path:
+    """Link examples/c_abi_cdist.cpp (a HIP host program that uses nothing but the C
+    ABI) against the library, next to it, with an rpath relative to the binary."""
+    source = PACKAGE_DIR.parent / "examples" / "c_abi_cdist.cpp"
+    target = LIB_DIR / "c_abi_cdist"
+    cmd = [_hipcc(), f"--offload-arch={ARCH}", "-O2", "-std=c++17", f"-I{PACKAGE_DIR.parent / 'include'}", str(source),
+           f"-L{LIB_DIR}", "-lkermac_amd", "-Wl,-rpath,$ORIGIN", "-o", str(target)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building {source.name} failed:\n{proc.stdout}\n{proc.stderr}")
+    return target
 
 
 if __name__ == "__main__":

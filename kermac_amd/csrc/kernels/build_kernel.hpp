@@ -326,8 +326,9 @@ __device__ __forceinline__ void accumulate_tile(
         // step are requested before the 128 VALU operations of the current one
         // are issued.  The loop is kept rolled (two k-steps per trip) on purpose:
         // fully unrolled, the compiler hoists all 64 LDS reads of a slice to the
-        // top and needs > 300 registers; rolled, it needs ~128 and four waves
-        // fit on each SIMD.
+        // top and needs > 300 registers; rolled, it needs 134 to 142 and three
+        // waves fit on each SIMD (a fourth, forced by a register limit of 128,
+        // changes nothing measurable).
         float fa0[8], fb0[8], fa1[8], fb1[8];
         read_fragment(fa0, sa);
         read_fragment(fb0, sb);

@@ -352,6 +352,45 @@ def test_library_exports_every_declared_symbol():
     assert _backend.build_kernel_has_variant(0, 4) and _backend.build_kernel_has_variant(1, 0)
 
 
+def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
+    """include/kermac_amd.h must compile as C11 on its own, and every struct must
+    have, field by field, the size and offsets the ctypes binding assumes.  The
+    probe program is generated from the binding's field names, so a field that is
+    missing, renamed or reordered in either place fails here."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    structs = {"kmc_build_kernel_params": _backend.BuildKernelParams,
+               "kmc_norm_gradient_params": _backend.NormGradientParams,
+               "kmc_kernel_coefficients_params": _backend.KernelCoefficientsParams}
+    lines = ['#include "kermac_amd.h"', "#include <stddef.h>", "#include <stdio.h>", "int main(void) {"]
+    for c_name, binding in structs.items():
+        lines.append(f'  printf("{c_name} size %zu\\n", sizeof(struct {c_name}));')
+        for field, _ in binding._fields_:
+            lines.append(f'  printf("{c_name} {field} %zu\\n", offsetof(struct {c_name}, {field}));')
+    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER"):
+        lines.append(f'  printf("flag {flag} %d\\n", (int)KMC_FLAG_{flag});')
+    lines += ['  printf("err WRONG_DEVICE %d\\n", (int)KMC_ERR_WRONG_DEVICE);', "  return 0;", "}"]
+    source = tmp_path / "probe.c"
+    source.write_text("\n".join(lines))
+    exe = tmp_path / "probe"
+    subprocess.run([gcc, "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{ROOT / 'include'}", str(source),
+                    "-o", str(exe)], check=True)
+    reported = {}
+    for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines():
+        *key, value = line.split()
+        reported[tuple(key)] = int(value)
+    for c_name, binding in structs.items():
+        assert reported[(c_name, "size")] == ctypes.sizeof(binding), c_name
+        for field, _ in binding._fields_:
+            assert reported[(c_name, field)] == getattr(binding, field).offset, f"{c_name}.{field}"
+    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER"):
+        assert reported[("flag", flag)] == getattr(_backend, f"FLAG_{flag}")
+    assert reported[("err", "WRONG_DEVICE")] == _backend.ERR_WRONG_DEVICE
+
+
 def test_c_abi_rejects_bad_arguments_without_a_gpu():
     params = _backend.BuildKernelParams()
     params.inner_operator = 7
