@@ -70,7 +70,16 @@ enum kmc_flags {
      * and closer to the exact power than the reference's ex2(p * lg2|x|)
      * (include/kermac_internal_common.cuh:139-161).  This flag keeps the generic
      * exp2(p * log2|x|) evaluation for those exponents too. */
-    KMC_FLAG_GENERIC_POWER = 8
+    KMC_FLAG_GENERIC_POWER = 8,
+    /* kmc_build_kernel notices when both operands are the same panel (a == b, same
+     * strides, majorness and extent, equal regularisation offsets) and the inner term
+     * does not change when its operands are exchanged (DOT; ABS, SQUARE or POW of a
+     * difference).  The result is then symmetric bit for bit, so only the 128 x 128
+     * tiles on and below the diagonal are computed and each is stored twice: about
+     * half the time for x-against-x matrices.  The reference computes every tile
+     * (its Symmetry enum, src/kermac/build_a_kernel.py:35-37, is not used anywhere).
+     * This flag switches the shortcut off. */
+    KMC_FLAG_NO_SYMMETRY = 16
 };
 
 /*

@@ -349,6 +349,10 @@ def _plan_run_kernel(
     params.a_majorness = _MAJORNESS_ABI[stats_a.majorness]
     params.b_majorness = _MAJORNESS_ABI[stats_b.majorness]
     params.flags = _backend.FLAG_NEGATE_DIFF if swapped else 0
+    if os.environ.get("KERMAC_AMD_NO_SYMMETRY", "0") not in ("", "0"):
+        # the library computes x-against-x matrices from the tiles on and below the diagonal
+        # (bit-identical result, about half the time); this keeps it to the full computation
+        params.flags |= _backend.FLAG_NO_SYMMETRY
     if (_l2_mode["mode"] == "gram" and d._inner_operator is InnerOperator.DIFF
             and d._inner_power is PowerType.SQUARE and stats_c is not None):
         params.flags |= _backend.FLAG_L2_GRAM

@@ -79,6 +79,14 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
     args->epsilon = p->epsilon;
     args->diff_sign = (p->flags & KMC_FLAG_NEGATE_DIFF) ? -1.0f : 1.0f;
     args->repair_only = 0;
+    // Same panel on both sides, same offsets, and an inner term that does not change
+    // when its operands are exchanged (every DOT term; |x|, x^2, |x|^p of a
+    // difference): C(n, m) equals C(m, n) bit for bit, so half the tiles suffice.
+    const bool exchangeable = p->inner_operator == KMC_OP_DOT || p->inner_power == KMC_POW_ABS ||
+                              p->inner_power == KMC_POW_SQUARE || p->inner_power == KMC_POW_POW;
+    args->symmetric = need_c && !(p->flags & KMC_FLAG_NO_SYMMETRY) && exchangeable && p->a == p->b && p->m == p->n &&
+                      p->a_ld == p->b_ld && p->a_bs == p->b_bs && p->a_majorness == p->b_majorness &&
+                      p->regularization_offset_x == p->regularization_offset_y && tiles_m > 1;
     args->gram_trust = p->gram_trust > 0.0f ? p->gram_trust : 0.25f;
     args->outer_power = p->outer_power;
     args->kernel_type = p->kernel_type;

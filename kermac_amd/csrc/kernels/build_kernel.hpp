@@ -45,6 +45,8 @@ struct BuildKernelArgs {
     int tiles_m, tiles_n;
     int tiles_n_padded;  // tiles_n rounded up to a multiple of 8; grid.x = tiles_m * tiles_n_padded
     int repair_only;     // recompute only the tiles that carry BK_REPAIR_MARKER (see gram_kernel.hpp)
+    int symmetric;       // A and B are the same panel and the result is symmetric: only tiles with
+                         // tile_m >= tile_n are computed, each is also stored mirrored
     float gram_trust;    // gram_kernel.hpp: distrust d^2 below gram_trust * (|a|^2 + |b|^2)
 };
 
@@ -413,6 +415,8 @@ __device__ __forceinline__ bool tile_of_workgroup(const BuildKernelArgs &args, i
     const int in_band = linear - band * band_tiles;
     tile_m = in_band / band_height;
     tile_n = band * BK_BAND_N + in_band % band_height;
+    // Symmetric result: the workgroups of the upper triangle have nothing to do.
+    if (args.symmetric && tile_n > tile_m) return false;
     return tile_n < args.tiles_n;
 }
 
@@ -488,6 +492,29 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     if (m_local + i < m_valid) dst[i] = acc[j][4 * h + i];
+            }
+        }
+    }
+
+    // Symmetric result: the same values also belong at C(n, m).  There the four
+    // consecutive n of a lane are the contiguous ones: 16 pieces of 4 again.
+    if (args.symmetric && tile_m != tile_n) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int m_local = tx * 4 + (i & 3) + (i >> 2) * 64;
+            if (m_local >= m_valid) continue;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int n_local = ty * 4 + h * 64;
+                float *dst = c_tile + (i64)(m0 + m_local) * args.c_ld + n0 + n_local;
+                if (args.c_vec && n_local + 3 < n_valid) {
+                    *reinterpret_cast<float4 *>(dst) =
+                        make_float4(acc[4 * h][i], acc[4 * h + 1][i], acc[4 * h + 2][i], acc[4 * h + 3][i]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (n_local + j < n_valid) dst[j] = acc[4 * h + j][i];
+                }
             }
         }
     }

@@ -296,6 +296,24 @@ __global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const B
                 }
             }
     }
+
+    // Symmetric result (a and b are the same panel): the same values also belong at
+    // C(n, m), where the 32 consecutive n of a half wave are the contiguous ones.
+    // A distrusted tile is recomputed and mirrored by the repair launch.
+    if (args.symmetric && tile_m != tile_n && !repair) {
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+            const int n_local = wave_n + nt * 32 + i;
+            if (n_local >= n_valid) continue;
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int m_local = wave_m + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+                    if (m_local < m_valid) c_tile[(i64)(m0 + m_local) * args.c_ld + n0 + n_local] = acc[mt][nt][v];
+                }
+        }
+    }
 }
 
 }  // namespace kmc
