@@ -242,9 +242,7 @@ __global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const B
     // d^2, trust check, epilogue.  Loop order: one norm of a per (mt, v), used for both
     // column tiles, so that only a few of the 32 norms a lane needs are live (with the
     // column tile outermost the kernel needs 206 registers instead of 127).  The
-    // square root is the hardware one (1 ulp; this path's tolerance is 1e-5 anyway),
-    // the rest is the general routine of the direct kernel.
-    const int outer_rest = outer_power == POW_SQRT ? POW_NOOP : outer_power;
+    // epilogue is the routine of the direct kernel.
     int distrust = 0;
     float norm_b[2];
     int n_local[2];
@@ -266,8 +264,7 @@ __global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const B
                 // NaN compares false: a NaN result is stored as is, not repaired.
                 if (m_local < m_valid && n_local[nt] < n_valid && d2 < args.gram_trust * norms) distrust = 1;
                 d2 = fmaxf(d2, 0.0f);
-                if (outer_power == POW_SQRT) d2 = __builtin_amdgcn_sqrtf(d2);
-                float value = epilogue_value(d2, outer_rest, kernel_type, p_outer, neg_gamma, args.epsilon);
+                float value = epilogue_value(d2, outer_power, kernel_type, p_outer, neg_gamma, args.epsilon);
                 if (regularize && args.reg_off_x + m0 + m_local == args.reg_off_y + n0 + n_local[nt]) value = diagonal_value;
                 acc[mt][nt][v] = value;
             }
