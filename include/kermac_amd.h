@@ -62,6 +62,9 @@ enum kmc_flags {
      * gram_trust * (|a|^2 + |b|^2) (cancellation).  Two launches on the stream.
      * Trusted elements carry a relative error of about sqrt(K) * 2^-24 / gram_trust
      * on the squared distance; repaired tiles are bit-identical to the direct path.
+     * kmc_kernel_times_coefficients honours the flag too (in kernel.flags): the kernel
+     * values of each tile then come from the matrix cores, and a distrusted tile is
+     * recomputed inside the same kernel (one launch).
      * The reference has no such path (include/build_a_kernel.cuh:339-370 is SIMT only). */
     KMC_FLAG_L2_GRAM = 4,
     /* kmc_build_kernel evaluates inner_operator DIFF + inner_power POW with a scalar

@@ -51,7 +51,8 @@ HOST_SOURCES = [
 
 
 # Device translation units without per-variant defines.
-EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_inst.hip"]
+EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_inst.hip",
+                        "kernels/gram_coefficients_inst.hip"]
 
 
 def _hipcc() -> str:

@@ -354,7 +354,8 @@ def _plan_run_kernel(
         # (bit-identical result, about half the time); this keeps it to the full computation
         params.flags |= _backend.FLAG_NO_SYMMETRY
     if (_l2_mode["mode"] == "gram" and d._inner_operator is InnerOperator.DIFF
-            and d._inner_power is PowerType.SQUARE and stats_c is not None):
+            and d._inner_power is PowerType.SQUARE):
+        # also for the fused coefficient product (no out matrix here): it has a matrix-core variant too
         params.flags |= _backend.FLAG_L2_GRAM
         params.gram_trust = _gram_trust(K)
     params.m, params.n, params.k, params.l = M, N, K, L

@@ -8,6 +8,8 @@ using namespace kmc_host;
 namespace kmc_host {
 int prepare_build_kernel(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs *args, int *load_a,
                          int *load_b);
+hipError_t launch_gram_coefficients(int load_a, int load_b, const kmc::KernelCoefficientsArgs &args, dim3 grid,
+                                    hipStream_t stream);
 }
 
 namespace {
@@ -67,6 +69,11 @@ int kmc_kernel_times_coefficients(const kmc_kernel_coefficients_params *params, 
     int status = prepare(params, &kc, &load_a, &load_b, &grid, &empty);
     if (status != KMC_OK) return status;
     kmc_host::coef_launcher_fn launch = find_launcher(params->kernel.inner_operator, params->kernel.inner_power);
+    if (params->kernel.flags & KMC_FLAG_L2_GRAM) {
+        if (params->kernel.inner_operator != KMC_OP_DIFF || params->kernel.inner_power != KMC_POW_SQUARE)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L2_GRAM needs inner_operator DIFF and inner_power SQUARE");
+        launch = kmc_host::launch_gram_coefficients;   // kernel values from the matrix cores
+    }
     if (!launch) {
         return fail(KMC_ERR_UNSUPPORTED_VARIANT,
                     "inner_operator=%d inner_power=%d is not compiled ahead of time; compile it at run time",
