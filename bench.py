@@ -196,13 +196,34 @@ def bench_kernel_coef(kermac, device, args):
     log(f"kernel x coefficients: {kernel_ms:.2f} ms kernel, slab max abs err / mean |truth| = {err:.2e}")
     if err > 1e-4:
         sys.exit(f"bench.py: kernel x coefficients parity failure: {err:.3e}")
+    # Beside it: the same shape with a Gaussian kernel, vector kernel and opt-in matrix-core kernel.
+    gaussian = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP,
+                                       kermac.KernelType.GAUSSIAN)
+    call = lambda: kermac.run_kernel(gaussian, x.transpose(1, 2), z.t(), out=out, bandwidth=9.0, coefficients=coef)
+    side_steps = max(2, min(args.steps, 5))
+    _, gaussian_ms = time_call(call, side_steps, 1)
+    kermac.set_l2_mode("gram")
+    try:
+        _, gaussian_mfma_ms = time_call(call, side_steps, 1)
+    finally:
+        kermac.set_l2_mode("direct")
+    d2 = torch.cdist(x[0, :, rows].t().double(), z.t().double(), p=2.0) ** 2
+    truth = torch.exp(-d2 / (2 * 9.0 ** 2)) @ coef[0].double()
+    gaussian_err = ((out[0, rows].double() - truth).abs().max() / truth.abs().mean()).item()
+    log(f"gaussian x coefficients: vector {gaussian_ms:.2f} ms, matrix cores {gaussian_mfma_ms:.2f} ms, "
+        f"slab max abs err / mean |truth| = {gaussian_err:.2e}")
+    if gaussian_err > 1e-4:
+        sys.exit(f"bench.py: gaussian x coefficients (matrix cores) parity failure: {gaussian_err:.3e}")
     ops = float(L) * nx * mz * (3 * k + 2 * o)
     nbytes = 4.0 * (L * k * nx + k * mz + 2 * L * nx * o)
     return side_line("fused Laplace kernel matrix x coefficients ms, L=4 N=M=16384 K=256 O=32",
                      "run_kernel(laplace_l1, x[4,16384,256] view, z[16384,256] view, bandwidth=10, "
                      "coefficients[4,16384,32]) -> out[4,16384,32] (BASELINE configs[4])",
                      wall_ms, kernel_ms, ops, nbytes, "valu_fp32", 157.3,
-                     {"parity_max_err_over_mean": err}, args)
+                     {"parity_max_err_over_mean": err,
+                      "gaussian_same_shape": {"vector_ms": round(gaussian_ms, 3), "matrix_core_ms": round(gaussian_mfma_ms, 3),
+                                              "matrix_core_parity_max_err_over_mean": gaussian_err,
+                                              "opt_in": "kermac_amd.set_l2_mode('gram')"}}, args)
 
 
 def main():
