@@ -58,6 +58,25 @@ def test_cdist_output_beyond_2_31_elements(device):
     assert_close_to_truth(col_sum, truth_sum, rtol=2e-6, what="column sums of the large matrix")
 
 
+def test_self_matrix_beyond_2_31_elements(device):
+    """A set against itself with more than 2^31 results: the mirrored stores of the
+    symmetric shortcut use 64-bit offsets too.  Must equal the full computation."""
+    M, K = 46500, 8
+    if free_bytes(device) < 3 * 4 * M * M:
+        pytest.skip("not enough free device memory")
+    g = torch.Generator().manual_seed(2035)
+    x_store = torch.randn(K, M, generator=g).to(device)
+    out_self = torch.full((M, M), float("nan"), device=device)
+    out_full = torch.empty(M, M, device=device)
+    kermac.cdist(x_store.t(), x_store.t(), p=2.0, out=out_self.t())
+    kermac.cdist(x_store.t(), x_store.clone().t(), p=2.0, out=out_full.t())
+    assert torch.equal(out_self, out_full)
+    del out_full
+    truth = oracle.cdist(x_store[:, -200:].t().cpu(), x_store[:, :200].t().cpu(), p=2.0)[0]
+    assert_close_to_truth(out_self[:200, -200:].t(), truth, rtol=1e-5, what="corner of the large self matrix")
+    assert_close_to_truth(out_self[-200:, :200], truth, rtol=1e-5, what="mirrored corner of the large self matrix")
+
+
 def test_cdist_batch_stride_beyond_2_31(device):
     """Three batches of 27000 x 27000: the third batch starts past element 2^31 only
     through the batch stride."""
