@@ -301,7 +301,9 @@ def _plan_run_kernel(
         if L_c != L and L != 1:
             raise ValueError(f"out must have batch dimension (L={L}), got {(L_c)}")
     elif allocate_out:
-        out = torch.zeros((L, M, N), dtype=torch.float32, device=device)
+        # every element is written by the kernel (also for K = 0), so no fill is needed; the
+        # reference allocates zeros (build_a_kernel.py:259), which costs 0.6 ms at 30000 x 30000
+        out = torch.empty((L, M, N), dtype=torch.float32, device=device)
         stats_c = tensor_stats(out)
     else:
         stats_c = None

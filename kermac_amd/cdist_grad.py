@@ -109,7 +109,8 @@ def _plan_cdist_grad(a, b, c, d, out, p, require_device=True) -> _GradPlan:
         norm_type = _NORM_P
 
     if out is None:
-        out = torch.zeros((L, O, N, M), dtype=torch.float32, device=device)
+        # every element is written by the kernel, so no fill is needed
+        out = torch.empty((L, O, N, M), dtype=torch.float32, device=device)
 
     params = _backend.NormGradientParams()
     params.norm_type = norm_type

@@ -73,7 +73,8 @@ def _plan_run_kernel_coefficients(
         if out.stride(-1) != 1 and O > 1:
             raise ValueError("out must have stride 1 in last dimension")
     else:
-        out = torch.zeros((L, M, O), dtype=torch.float32, device=device)
+        # every element is written by the kernel (zeros when N = 0), so no fill is needed
+        out = torch.empty((L, M, O), dtype=torch.float32, device=device)
 
     def batch_stride(t):
         return t.stride(0) if t.dim() == 3 and t.size(0) != 1 else 0

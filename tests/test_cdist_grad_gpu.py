@@ -148,3 +148,13 @@ def test_gradient_rfm_shape_against_slab_truth(device):
         truth = torch.einsum("ok,km,nmk->onm", c.double(), a[:, ms].double(), sign)
         assert_close_to_truth(out[:, ns, ms], truth, rtol=1e-5, atol=1e-5 * float(truth.abs().mean()) * 10,
                               what="RFM slab")
+
+
+def test_gradient_empty_contraction_writes_zeros(device):
+    """K = 0: the result buffer is allocated uninitialised, the kernel must still write
+    every element (an empty sum)."""
+    junk = torch.full((1, 5, 9, 70), float("nan"), device=device)      # make a recycled allocation visible
+    del junk
+    got = kermac.cdist_grad(torch.zeros(0, 70, device=device), torch.zeros(9, 0, device=device),
+                            torch.zeros(5, 0, device=device), torch.randn(9, 70, device=device), p=1.0)
+    assert got.shape == (1, 5, 9, 70) and torch.all(got == 0)

@@ -101,3 +101,14 @@ def test_laplace_times_coefficients_headline_shape(device):
         d = torch.cdist(x_store[l, :, rows].t().double(), z_store.t().double(), p=1.0)
         truth = torch.exp(-d / 10.0) @ coef[l].double()
         assert_close_to_truth(out[l, rows], truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"slab batch {l}")
+
+
+def test_no_centres_gives_zeros(device):
+    """N = 0: the result buffer is allocated uninitialised, the kernel must still write
+    every element (an empty sum)."""
+    junk = torch.full((1, 200, 7), float("nan"), device=device)         # make a recycled allocation visible
+    del junk
+    a = torch.randn(200, 6, device=device)
+    got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, torch.zeros(0, 6, device=device), bandwidth=2.0,
+                            coefficients=torch.zeros(0, 7, device=device))
+    assert got.shape == (1, 200, 7) and torch.all(got == 0)
