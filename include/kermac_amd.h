@@ -82,7 +82,18 @@ enum kmc_flags {
      * half the time for x-against-x matrices.  The reference computes every tile
      * (its Symmetry enum, src/kermac/build_a_kernel.py:35-37, is not used anywhere).
      * This flag switches the shortcut off. */
-    KMC_FLAG_NO_SYMMETRY = 16
+    KMC_FLAG_NO_SYMMETRY = 16,
+    /* kmc_build_kernel only; implies KMC_FLAG_L2_GRAM (same trust rule, same repair
+     * launch, same stated tolerance), with the cross term a.b on the bf16 matrix
+     * instruction: every fp32 operand is split into three bf16 pieces (exactly: the
+     * pieces sum to the operand) while it is staged, and the six largest of the nine
+     * piece products are accumulated in fp32.  The error of the cross term stays that of
+     * an fp32 dot product (measured 9e-8 |a||b| at K = 1024); the launch takes about two
+     * thirds of the fp32 matrix-core time.  The six products are not summed in an order
+     * that is symmetric in a and b, so C(m,n) and C(n,m) of an x-against-x matrix agree
+     * to rounding only, unless the symmetric shortcut (see KMC_FLAG_NO_SYMMETRY) mirrors
+     * them.  kmc_kernel_times_coefficients does not look at this flag. */
+    KMC_FLAG_L2_GRAM_BF16 = 32
 };
 
 /*

@@ -34,6 +34,7 @@ FLAG_NEGATE_DIFF = 2
 FLAG_L2_GRAM = 4
 FLAG_GENERIC_POWER = 8
 FLAG_NO_SYMMETRY = 16
+FLAG_L2_GRAM_BF16 = 32
 
 _float_p = c_void_p  # device pointers are passed as integers
 

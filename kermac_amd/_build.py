@@ -52,7 +52,7 @@ HOST_SOURCES = [
 
 # Device translation units without per-variant defines.
 EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_inst.hip",
-                        "kernels/gram_coefficients_inst.hip"]
+                        "kernels/gram_coefficients_inst.hip", "kernels/gram_bf16_kernel_inst.hip"]
 
 
 def _hipcc() -> str:

@@ -113,6 +113,7 @@ kmc_host::build_launcher_fn find_launcher(int inner_operator, int inner_power)
 
 namespace kmc_host {
 hipError_t launch_gram_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
+hipError_t launch_gram_bf16_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
 }
 
 namespace kmc_host {
@@ -166,11 +167,13 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
     status = require_gfx950();
     if (status != KMC_OK) return status;
     const dim3 grid(static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n_padded), args.l, 1);
-    if (params->flags & KMC_FLAG_L2_GRAM) {
+    if (params->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16)) {
         if (params->inner_operator != KMC_OP_DIFF || params->inner_power != KMC_POW_SQUARE)
             return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L2_GRAM needs inner_operator DIFF and inner_power SQUARE");
         // Matrix-core pass over every tile, then the direct kernel over the tiles it marked.
-        hipError_t g = launch_gram_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
+        hipError_t g = (params->flags & KMC_FLAG_L2_GRAM_BF16)
+                           ? launch_gram_bf16_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream))
+                           : launch_gram_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
         if (g != hipSuccess) return fail_hip(g, "gram_l2_kernel launch");
         args.repair_only = 1;
     }

@@ -225,92 +225,7 @@ __global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const B
     row_norms<LOAD_B>(load_b, square_b, lds_b, lds_norm_b, tid);
     __syncthreads();
 
-    // d^2, trust check, epilogue.
-    const int outer_power = args.outer_power;
-    const int kernel_type = args.kernel_type;
-    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
-    if (outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
-    if (kernel_type != KERNEL_NONE) {
-        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
-        neg_gamma = kernel_neg_gamma(kernel_type, bw);
-        regularization = args.regularization ? args.regularization[batch * args.regularization_bs]
-                                             : args.regularization_value;
-    }
-    const bool regularize = kernel_type != KERNEL_NONE && regularization != 0.0f;
-    const float diagonal_value = 1.0f + regularization;
-
-    // d^2, trust check, epilogue.  Loop order: one norm of a per (mt, v), used for both
-    // column tiles, so that only a few of the 32 norms a lane needs are live (with the
-    // column tile outermost the kernel needs 206 registers instead of 127).  The
-    // epilogue is the routine of the direct kernel.
-    int distrust = 0;
-    float norm_b[2];
-    int n_local[2];
-#pragma unroll
-    for (int nt = 0; nt < 2; nt++) {
-        n_local[nt] = wave_n + nt * 32 + i;
-        norm_b[nt] = lds_norm_b[n_local[nt]];
-    }
-#pragma unroll
-    for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int m_local = wave_m + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-            const float norm_a = lds_norm_a[m_local];
-#pragma unroll
-            for (int nt = 0; nt < 2; nt++) {
-                const float norms = norm_a + norm_b[nt];
-                float d2 = norms - 2.0f * acc[mt][nt][v];
-                // NaN compares false: a NaN result is stored as is, not repaired.
-                if (m_local < m_valid && n_local[nt] < n_valid && d2 < args.gram_trust * norms) distrust = 1;
-                d2 = fmaxf(d2, 0.0f);
-                float value = epilogue_value(d2, outer_power, kernel_type, p_outer, neg_gamma, args.epsilon);
-                if (regularize && args.reg_off_x + m0 + m_local == args.reg_off_y + n0 + n_local[nt]) value = diagonal_value;
-                acc[mt][nt][v] = value;
-            }
-        }
-    const bool repair = __syncthreads_or(distrust) != 0;
-
-    float *c_tile = args.c + batch * args.c_bs;
-#pragma unroll
-    for (int nt = 0; nt < 2; nt++) {
-        const int n_local = wave_n + nt * 32 + i;
-        if (n_local >= n_valid) continue;
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int m_local = wave_m + mt * 32 + 8 * g + 4 * h;
-                float v4[4] = {acc[mt][nt][4 * g], acc[mt][nt][4 * g + 1], acc[mt][nt][4 * g + 2], acc[mt][nt][4 * g + 3]};
-                if (repair && m_local == 0 && n_local == 0) v4[0] = __uint_as_float(BK_REPAIR_MARKER);
-                float *dst = c_tile + (i64)(n0 + n_local) * args.c_ld + m0 + m_local;
-                if (args.c_vec && m_local + 3 < m_valid) {
-                    *reinterpret_cast<float4 *>(dst) = make_float4(v4[0], v4[1], v4[2], v4[3]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (m_local + e < m_valid) dst[e] = v4[e];
-                }
-            }
-    }
-
-    // Symmetric result (a and b are the same panel): the same values also belong at
-    // C(n, m), where the 32 consecutive n of a half wave are the contiguous ones.
-    // A distrusted tile is recomputed and mirrored by the repair launch.
-    if (args.symmetric && tile_m != tile_n && !repair) {
-#pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
-            const int n_local = wave_n + nt * 32 + i;
-            if (n_local >= n_valid) continue;
-#pragma unroll
-            for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int m_local = wave_m + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-                    if (m_local < m_valid) c_tile[(i64)(m0 + m_local) * args.c_ld + n0 + n_local] = acc[mt][nt][v];
-                }
-        }
-    }
+#include "gram_epilogue.inc"
 }
 
 }  // namespace kmc

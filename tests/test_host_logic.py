@@ -370,7 +370,7 @@ def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
         lines.append(f'  printf("{c_name} size %zu\\n", sizeof(struct {c_name}));')
         for field, _ in binding._fields_:
             lines.append(f'  printf("{c_name} {field} %zu\\n", offsetof(struct {c_name}, {field}));')
-    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY"):
+    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16"):
         lines.append(f'  printf("flag {flag} %d\\n", (int)KMC_FLAG_{flag});')
     lines += ['  printf("err WRONG_DEVICE %d\\n", (int)KMC_ERR_WRONG_DEVICE);', "  return 0;", "}"]
     source = tmp_path / "probe.c"
@@ -386,7 +386,7 @@ def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
         assert reported[(c_name, "size")] == ctypes.sizeof(binding), c_name
         for field, _ in binding._fields_:
             assert reported[(c_name, field)] == getattr(binding, field).offset, f"{c_name}.{field}"
-    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY"):
+    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16"):
         assert reported[("flag", flag)] == getattr(_backend, f"FLAG_{flag}")
     assert reported[("err", "WRONG_DEVICE")] == _backend.ERR_WRONG_DEVICE
 

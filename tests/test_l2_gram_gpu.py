@@ -1,6 +1,7 @@
 """GPU tests of the opt-in matrix-core path for squared-difference descriptors
-(``kermac_amd.set_l2_mode("gram")``): |a|^2 + |b|^2 - 2 a.b on the MFMA units with
-automatic repair of ill-conditioned tiles by the direct kernel.
+(``kermac_amd.set_l2_mode("gram")`` and ``"gram_bf16"``): |a|^2 + |b|^2 - 2 a.b on the
+MFMA units (fp32 operands, or three bf16 pieces per operand) with automatic repair of
+ill-conditioned tiles by the direct kernel.
 
 Stated tolerance: the same 1e-5 relative to the float64 truth as the direct p = 2
 path -- trusted tiles by the error bound of the expansion, repaired tiles because
@@ -16,9 +17,9 @@ from tests.helpers import assert_close_to_truth, make_operand
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture()
-def gram_mode():
-    kermac.set_l2_mode("gram")
+@pytest.fixture(params=["gram", "gram_bf16"])
+def gram_mode(request):
+    kermac.set_l2_mode(request.param)
     yield
     kermac.set_l2_mode("direct")
 

@@ -27,7 +27,7 @@ DESCRIPTORS = {
 }
 
 
-@pytest.fixture(params=["direct", "gram"])
+@pytest.fixture(params=["direct", "gram", "gram_bf16"])
 def l2_mode(request):
     kermac.set_l2_mode(request.param)
     yield request.param
@@ -63,7 +63,13 @@ def test_batched_self_matrix_and_matrix_core_mode(device, l2_mode):
     got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, x, bandwidth=bw, regularization=1e-3)
     full = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, x.clone(memory_format=torch.preserve_format),
                              bandwidth=bw, regularization=1e-3)
-    assert torch.equal(got, full) and torch.equal(got, got.transpose(1, 2))
+    assert torch.equal(got, got.transpose(1, 2))
+    if l2_mode == "gram_bf16":
+        # the six piece products are summed in an order that is not symmetric in a and b, so the
+        # full computation is symmetric only up to rounding; the shortcut mirrors one half exactly
+        torch.testing.assert_close(got, full, rtol=2e-6, atol=1e-7)
+    else:
+        assert torch.equal(got, full)
     truth = oracle.build_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", x.cpu().contiguous(), x.cpu().contiguous(),
                                 bandwidth=bw.cpu(), regularization=1e-3)
     assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-7, what=f"batched self matrix, l2 mode {l2_mode}")
@@ -72,7 +78,11 @@ def test_batched_self_matrix_and_matrix_core_mode(device, l2_mode):
     y[150:] = y[:150] + 1e-4 * torch.randn(150, 24, generator=g).to(device)
     d_self = kermac.cdist(y, y, p=2.0)[0]
     d_full = kermac.cdist(y, y.clone(), p=2.0)[0]
-    assert torch.equal(d_self, d_full) and torch.equal(d_self, d_self.t())
+    assert torch.equal(d_self, d_self.t())
+    if l2_mode == "gram_bf16":
+        torch.testing.assert_close(d_self, d_full, rtol=2e-6, atol=1e-7)
+    else:
+        assert torch.equal(d_self, d_full)
     assert_close_to_truth(d_self, oracle.cdist(y.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, what="near duplicates")
 
 
