@@ -290,20 +290,22 @@ def main():
 
         # Opt-in matrix-core path for p = 2 (|a|^2 + |b|^2 - 2 a.b on fp32 MFMA, ill-conditioned tiles
         # recomputed directly); same 1e-5 tolerance.  Reported beside the default direct path.
-        log("timing p = 2.0, l2 mode 'gram'")
-        kermac.set_l2_mode("gram")
-        try:
-            _, k_ms = time_cdist(kermac, a, b, out, 2.0, False, side_steps, 1)
-            e = parity_slab(out, a, b, 2.0, False)
-        finally:
-            kermac.set_l2_mode("direct")
-        log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
-        if e > 1e-5:
-            sys.exit(f"bench.py: parity failure for p=2.0 (gram): slab max rel err {e:.3e} > 1e-5")
-        per_p["2.0_gram_mfma"] = {"ms": round(k_ms, 3), "tflops_3op": round(OPS_PER_CALL / k_ms / 1e9, 2),
-                                  "pct_fp32_valu_peak": round(OPS_PER_CALL / k_ms / 1e9 / PEAK_FP32_VALU_TFLOPS * 100, 2),
-                                  "mfma_tflops": round(2.0 * M * N * K / k_ms / 1e9, 2),
-                                  "parity_max_rel_err": e, "rtol": 1e-5, "opt_in": "kermac_amd.set_l2_mode('gram')"}
+        # "gram_bf16": the cross term on the bf16 matrix instruction from three exact bf16 pieces per operand.
+        for mode, label in (("gram", "2.0_gram_mfma"), ("gram_bf16", "2.0_gram_bf16_mfma")):
+            log(f"timing p = 2.0, l2 mode '{mode}'")
+            kermac.set_l2_mode(mode)
+            try:
+                _, k_ms = time_cdist(kermac, a, b, out, 2.0, False, side_steps, 1)
+                e = parity_slab(out, a, b, 2.0, False)
+            finally:
+                kermac.set_l2_mode("direct")
+            log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
+            if e > 1e-5:
+                sys.exit(f"bench.py: parity failure for p=2.0 ({mode}): slab max rel err {e:.3e} > 1e-5")
+            per_p[label] = {"ms": round(k_ms, 3), "tflops_3op": round(OPS_PER_CALL / k_ms / 1e9, 2),
+                            "pct_fp32_valu_peak": round(OPS_PER_CALL / k_ms / 1e9 / PEAK_FP32_VALU_TFLOPS * 100, 2),
+                            "mfma_tflops": round((1 if mode == "gram" else 6) * 2.0 * M * N * K / k_ms / 1e9, 2),
+                            "parity_max_rel_err": e, "rtol": 1e-5, "opt_in": f"kermac_amd.set_l2_mode('{mode}')"}
 
         # x against x (the kernel matrix of a training set): the library computes the tiles on and
         # below the diagonal only and stores each twice; bit-identical to the full computation.
