@@ -55,7 +55,10 @@ constexpr int BK_TILE_N = 128;
 constexpr int BK_TILE_K = 16;
 constexpr int BK_THREADS = 256;
 constexpr int BK_XCDS = 8;     // MI355X: 8 accelerator dies, 32 CUs and one L2 each
-constexpr int BK_BAND_N = 64;  // height, in tiles, of the bands the tile order walks: 8 per XCD
+#ifndef BK_BAND_TILES
+#define BK_BAND_TILES 64
+#endif
+constexpr int BK_BAND_N = BK_BAND_TILES;  // height, in tiles, of the bands the tile order walks: 8 per XCD
 // Row pitch of an LDS slice in floats.  +4 keeps rows 16-byte aligned and skews
 // the banks so that the transposing (k-contiguous) loaders write conflict-free.
 constexpr int BK_LDS_PITCH = BK_TILE_M + 4;
@@ -375,13 +378,24 @@ __device__ __forceinline__ void finish_tile(
                                              : args.regularization_value;
     }
     const float epsilon = args.epsilon;
-    if (outer_power != POW_NOOP || kernel_type != KERNEL_NONE) {
+    // One uniform branch per tile and step, not per element: with the switch inside the
+    // loops the compiler keeps it there, and 64 branch chains per lane cost a quarter
+    // of the run time of a store-bound (small K) problem.
+    auto for_each = [&](auto &&f) {
 #pragma unroll
         for (int j = 0; j < 8; j++)
 #pragma unroll
-            for (int i = 0; i < 8; i++)
-                acc[j][i] = epilogue_value(acc[j][i], outer_power, kernel_type, p_outer, neg_gamma, epsilon);
+            for (int i = 0; i < 8; i++) acc[j][i] = f(acc[j][i]);
+    };
+    switch (outer_power) {
+    case POW_ABS: for_each([](float v) { return __builtin_fabsf(v); }); break;
+    case POW_SQUARE: for_each([](float v) { return v * v; }); break;
+    case POW_SQRT: for_each([](float v) { return __builtin_amdgcn_sqrtf(v); }); break;
+    case POW_POW: for_each([p_outer](float v) { return exp2f(p_outer * log2f(v)); }); break;
+    default: break;
     }
+    if (kernel_type != KERNEL_NONE)
+        for_each([epsilon, neg_gamma](float v) { return expf((v < epsilon ? 0.0f : v) * neg_gamma); });
     // include/build_a_kernel.cuh:429-447: the diagonal is replaced, not incremented.
     if (kernel_type != KERNEL_NONE && regularization != 0.0f) {
         const float diagonal_value = 1.0f + regularization;
