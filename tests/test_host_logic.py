@@ -294,6 +294,11 @@ def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
         assert flags(kermac.kernel_descriptor_p_norm, p=1.3)[0] & _backend.FLAG_L2_GRAM == 0
         kermac.set_l2_mode("gram", trust=0.5)
         assert flags(kermac.kernel_descriptor_l2_norm)[1] == pytest.approx(0.5)
+        assert flags(kermac.kernel_descriptor_l2_norm)[0] & _backend.FLAG_L2_GRAM_BF16 == 0
+        kermac.set_l2_mode("gram_bf16")
+        f, trust = flags(kermac.kernel_descriptor_l2_norm)
+        assert f & _backend.FLAG_L2_GRAM and f & _backend.FLAG_L2_GRAM_BF16 and trust == pytest.approx(0.25)
+        assert flags(kermac.kernel_descriptor_l1_norm)[0] & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16) == 0
     finally:
         kermac.set_l2_mode("direct")
     # the default trust grows with K so that very long sums fall back to the direct kernel

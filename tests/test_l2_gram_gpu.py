@@ -102,6 +102,35 @@ def test_kernels_batches_and_regularisation(device, gram_mode):
                           atol=1e-4, what="gram squared distances")
 
 
+def test_empty_contraction_gives_zeros(device, gram_mode):
+    a = torch.empty(200, 0, device=device)
+    b = torch.empty(150, 0, device=device)
+    out = torch.full((1, 200, 150), 7.0, device=device)
+    assert kermac.cdist(a, b, out=out, p=2.0) is out
+    assert torch.count_nonzero(out) == 0
+
+
+def test_bf16_flag_alone_through_the_c_abi(device):
+    """KMC_FLAG_L2_GRAM_BF16 implies the matrix-core path; a caller of the C ABI need not set both flags."""
+    from kermac_amd import _backend
+    from kermac_amd.build_a_kernel import _plan_run_kernel
+    g = torch.Generator().manual_seed(8)
+    a = torch.randn(300, 48, generator=g).to(device)
+    b = torch.randn(257, 48, generator=g).to(device)
+    out = torch.empty(1, 300, 257, device=device)
+    plan = _plan_run_kernel(kermac.kernel_descriptor_l2_norm, a, b, out, None, None, None, None, None, None, 0, 0, False)
+    assert plan.params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16) == 0
+    plan.params.flags |= _backend.FLAG_L2_GRAM_BF16
+    plan.params.gram_trust = 0.25
+    _backend.build_kernel(plan.params, torch.cuda.current_stream(device).cuda_stream)
+    assert_close_to_truth(out, oracle.cdist(a.cpu(), b.cpu(), p=2.0), rtol=1e-5, what="bf16 flag alone")
+    kermac.set_l2_mode("gram_bf16")
+    try:
+        assert torch.equal(out, kermac.cdist(a, b, p=2.0))
+    finally:
+        kermac.set_l2_mode("direct")
+
+
 def test_full_size(device, gram_mode):
     M = N = 30000
     K = 1024
