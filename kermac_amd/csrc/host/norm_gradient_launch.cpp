@@ -35,36 +35,63 @@ extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void 
         p->b_bs < 0 || p->c_bs < 0 || p->d_bs < 0 || p->e_bs < 0 || p->p_bs < 0)
         return fail(KMC_ERR_INVALID_ARGUMENT, "negative stride");
 
-    // Up to 8 outputs: vector-ALU kernel (4 or 8 accumulators per (m,n)).  More:
-    // matrix-core kernel with 16 or 32 output columns per workgroup.
-    const int o_tile = p->o <= 4 ? 4 : (p->o <= 8 ? 8 : (p->o <= 16 ? 16 : 32));
-    const bool matrix_core = o_tile >= 16;
-    const int o_chunks = ceil_div(p->o, o_tile);
-    const int64_t grid_z = static_cast<int64_t>(p->l) * o_chunks;
-    const int tiles_m = ceil_div(p->m, matrix_core ? kmc::NGM_TILE_M : kmc::NG_TILE_M);
-    const int tiles_n = ceil_div(p->n, matrix_core ? kmc::NGM_TILE_N : kmc::NG_TILE_N);
-    if (grid_z > 65535 || tiles_n > 65535)
-        return fail(KMC_ERR_INVALID_ARGUMENT, "grid too large (n tiles %d, batch x o chunks %lld; limit 65535)", tiles_n,
-                    static_cast<long long>(grid_z));
-
-    kmc::NormGradientArgs args;
-    args.m = p->m; args.n = p->n; args.o = p->o; args.k = p->k; args.l = p->l;
-    args.a = p->a; args.a_ld = p->a_ld; args.a_bs = p->a_bs;
-    args.b = p->b; args.b_ld = p->b_ld; args.b_bs = p->b_bs;
-    args.c = p->c; args.c_ld = p->c_ld; args.c_bs = p->c_bs;
-    args.d = p->d; args.d_ld = p->d_ld; args.d_bs = p->d_bs;
-    args.e = p->e; args.e_ld_n = p->e_ld_n; args.e_ld_o = p->e_ld_o; args.e_bs = p->e_bs;
-    args.p = p->p; args.p_bs = p->p_bs; args.p_value = p->p_value;
-    args.o_chunks = o_chunks;
-    args.a_vec = vec_ok(p->a, p->a_ld, p->a_bs, 0, p->flags);
-    args.b_vec = vec_ok(p->b, p->b_ld, p->b_bs, 0, p->flags);
-    args.c_vec = vec_ok(p->c, p->c_ld, p->c_bs, 0, p->flags);
-    args.e_vec = vec_ok(p->e, p->e_ld_n, p->e_ld_o, p->e_bs, p->flags);
+    // The outputs are cut into at most three runs, each with the kernel that suits its
+    // width: whole groups of 32 (and a remainder of 25..31) on the matrix-core kernel with
+    // 32 output columns, a remainder of 9..24 as 16 columns on the matrix-core kernel with
+    // 16 plus, above 16, the rest on the vector-ALU kernel, which holds 1, 2, 4 or 8
+    // accumulators per (m, n).  O = 17 therefore costs a 16-wide and a 1-wide launch
+    // instead of one 32-wide launch that is half padding (18.5 -> 12.4 ms at M = K = 8192,
+    // N = 512 for the L1 norm; O = 48: 36.6 -> 28.0 ms).
+    struct Run { int begin, count, tile; };
+    Run runs[3];
+    int run_count = 0;
+    {
+        auto small_tile = [](int o) { return o <= 1 ? 1 : o <= 2 ? 2 : o <= 4 ? 4 : 8; };
+        int begin = 0, left = p->o;
+        const int wide = left % 32 >= 25 ? left : left - left % 32;     // columns for the 32-wide kernel
+        if (wide > 0) { runs[run_count++] = {begin, wide, 32}; begin += wide; left -= wide; }
+        if (left >= 17 && p->norm_type == KMC_NORM_P) {
+            // every run recomputes |d - b|^(p-1) with two transcendentals per (m, n, k): measured,
+            // one padded 32-wide launch (24.5 ms at the benchmark shape) beats 16 + rest (25.6 .. 32 ms)
+            runs[run_count++] = {begin, left, 32};
+            left = 0;
+        }
+        if (left >= 9) { const int take = left < 16 ? left : 16; runs[run_count++] = {begin, take, 16}; begin += take; left -= take; }
+        if (left > 0) runs[run_count++] = {begin, left, small_tile(left)};
+    }
 
     int status = require_gfx950();
     if (status != KMC_OK) return status;
-    const dim3 grid(tiles_m, tiles_n, static_cast<unsigned>(grid_z));
-    hipError_t e = launch_norm_gradient(p->norm_type, o_tile, args, grid, static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return fail_hip(e, "norm_kernel_gradient launch");
+    for (int r = 0; r < run_count; r++) {
+        const Run &run = runs[r];
+        const bool matrix_core = run.tile >= 16;
+        const int o_chunks = ceil_div(run.count, run.tile);
+        const int64_t grid_z = static_cast<int64_t>(p->l) * o_chunks;
+        const int tiles_m = ceil_div(p->m, matrix_core ? kmc::NGM_TILE_M : kmc::NG_TILE_M);
+        const int tiles_n = ceil_div(p->n, matrix_core ? kmc::NGM_TILE_N : kmc::NG_TILE_N);
+        if (grid_z > 65535 || tiles_n > 65535)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "grid too large (n tiles %d, batch x o chunks %lld; limit 65535)", tiles_n,
+                        static_cast<long long>(grid_z));
+
+        kmc::NormGradientArgs args;
+        args.m = p->m; args.n = p->n; args.o = run.count; args.k = p->k; args.l = p->l;
+        args.a = p->a; args.a_ld = p->a_ld; args.a_bs = p->a_bs;
+        args.b = p->b; args.b_ld = p->b_ld; args.b_bs = p->b_bs;
+        args.c = p->c ? p->c + static_cast<int64_t>(run.begin) * p->c_ld : p->c;
+        args.c_ld = p->c_ld; args.c_bs = p->c_bs;
+        args.d = p->d; args.d_ld = p->d_ld; args.d_bs = p->d_bs;
+        args.e = p->e + static_cast<int64_t>(run.begin) * p->e_ld_o;
+        args.e_ld_n = p->e_ld_n; args.e_ld_o = p->e_ld_o; args.e_bs = p->e_bs;
+        args.p = p->p; args.p_bs = p->p_bs; args.p_value = p->p_value;
+        args.o_chunks = o_chunks;
+        args.a_vec = vec_ok(p->a, p->a_ld, p->a_bs, 0, p->flags);
+        args.b_vec = vec_ok(p->b, p->b_ld, p->b_bs, 0, p->flags);
+        args.c_vec = vec_ok(args.c, p->c_ld, p->c_bs, 0, p->flags);
+        args.e_vec = vec_ok(args.e, p->e_ld_n, p->e_ld_o, p->e_bs, p->flags);
+
+        const dim3 grid(tiles_m, tiles_n, static_cast<unsigned>(grid_z));
+        hipError_t e = launch_norm_gradient(p->norm_type, run.tile, args, grid, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return fail_hip(e, "norm_kernel_gradient launch");
+    }
     return KMC_OK;
 }

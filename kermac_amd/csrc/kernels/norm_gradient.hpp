@@ -194,6 +194,11 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
             }
     };
     auto read_c = [&](float (&fc)[O_TILE], const float *src) {
+        if (O_TILE < 4) {
+#pragma unroll
+            for (int o = 0; o < O_TILE; o++) fc[o] = src[o];
+            return;
+        }
 #pragma unroll
         for (int q = 0; q < O_TILE / 4; q++) {
             const float4 v = *reinterpret_cast<const float4 *>(src + 4 * q);

@@ -1,5 +1,5 @@
 // Ahead-of-time instantiations of the kernel-gradient contraction: 3 norm types
-// x (vector-ALU kernel with 4 or 8 outputs per lane tile, matrix-core kernel with
+// x (vector-ALU kernel with 1, 2, 4 or 8 outputs per lane tile, matrix-core kernel with
 // 16 or 32 output columns, with and without a partial last K slice).
 #include <hip/hip_runtime.h>
 
@@ -13,6 +13,8 @@ static hipError_t launch_norm(int o_tile, const kmc::NormGradientArgs &args, dim
     const dim3 block(kmc::NG_THREADS);
     const bool k_tail = args.k % kmc::NGM_TILE_K != 0;
     switch (o_tile) {
+    case 1: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 1>), grid, block, 0, stream, args); break;
+    case 2: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 2>), grid, block, 0, stream, args); break;
     case 4: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 4>), grid, block, 0, stream, args); break;
     case 8: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 8>), grid, block, 0, stream, args); break;
     case 16:

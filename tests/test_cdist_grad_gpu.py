@@ -58,7 +58,9 @@ def test_gradient_reference_test_case(device):
 
 @pytest.mark.parametrize("p", [1.0, 2.0, 1.3, 0.7])
 @pytest.mark.parametrize("M,N,O,K", [(1, 1, 1, 1), (70, 33, 3, 17), (64, 32, 16, 16), (65, 31, 5, 50), (200, 40, 20, 35),
-                                     (130, 64, 8, 100)])
+                                     (130, 64, 8, 100), (129, 66, 1, 48), (256, 64, 2, 64), (67, 35, 2, 19),
+                                     # output counts that are cut into runs for kernels of different width
+                                     (96, 24, 17, 20), (80, 20, 33, 33), (70, 18, 49, 16), (66, 17, 57, 21), (64, 16, 90, 16)])
 def test_gradient_ragged_shapes(device, p, M, N, O, K):
     g = torch.Generator().manual_seed(M + 2 * N + 3 * O + 5 * K)
     a = torch.rand(K, M, generator=g).to(device)
@@ -107,7 +109,7 @@ def test_gradient_sign_convention_and_linearity(device):
     assert_close_to_truth(f(c1 + c2), f(c1) + f(c2), rtol=1e-4, atol=1e-4, what="linearity in c")
 
 
-@pytest.mark.parametrize("O", [1, 8, 16, 32])
+@pytest.mark.parametrize("O", [1, 2, 8, 16, 32])
 @pytest.mark.parametrize("K", [3, 16, 35])
 def test_gradient_l1_sign_of_zero_differences(device, O, K):
     """copysign(1, d - b) for the four combinations of signed zeros, equal non-zero
