@@ -14,8 +14,11 @@ hipError_t launch_gram_coefficients(int load_a, int load_b, const kmc::KernelCoe
 
 namespace {
 
-int prepare(const kmc_kernel_coefficients_params *p, kmc::KernelCoefficientsArgs *kc, int *load_a, int *load_b,
-            dim3 *grid, bool *empty)
+// `wide_allowed`: the launch goes to an ahead-of-time instantiation of the vector kernel,
+// which exists for 32 and for 64 coefficient columns per workgroup; the matrix-core
+// variant and run-time compiled functions hold 32.
+int prepare(const kmc_kernel_coefficients_params *p, bool wide_allowed, kmc::KernelCoefficientsArgs *kc, int *load_a,
+            int *load_b, dim3 *grid, bool *empty)
 {
     if (!p) return fail(KMC_ERR_INVALID_ARGUMENT, "null parameter block");
     int status = prepare_build_kernel(&p->kernel, false, &kc->kernel, load_a, load_b);
@@ -30,7 +33,8 @@ int prepare(const kmc_kernel_coefficients_params *p, kmc::KernelCoefficientsArgs
     if (p->coef_ld < 0 || p->coef_bs < 0 || p->out_ld < 0 || p->out_bs < 0)
         return fail(KMC_ERR_INVALID_ARGUMENT, "negative stride");
     kc->o = p->o;
-    kc->o_chunks = ceil_div(p->o, kmc::KC_COLUMNS);
+    kc->columns = wide_allowed && p->o > kmc::KC_COLUMNS ? 64 : kmc::KC_COLUMNS;
+    kc->o_chunks = ceil_div(p->o, kc->columns);
     kc->coef = p->coef; kc->coef_ld = p->coef_ld; kc->coef_bs = p->coef_bs;
     kc->out = p->out; kc->out_ld = p->out_ld; kc->out_bs = p->out_bs;
     kc->coef_vec = !(p->kernel.flags & KMC_FLAG_FORCE_SCALAR_ACCESS) && aligned16(p->coef) && p->coef_ld % 4 == 0 &&
@@ -66,7 +70,8 @@ int kmc_kernel_times_coefficients(const kmc_kernel_coefficients_params *params, 
     int load_a = 0, load_b = 0;
     dim3 grid;
     bool empty = false;
-    int status = prepare(params, &kc, &load_a, &load_b, &grid, &empty);
+    const bool matrix_core = params && (params->kernel.flags & KMC_FLAG_L2_GRAM);
+    int status = prepare(params, !matrix_core, &kc, &load_a, &load_b, &grid, &empty);
     if (status != KMC_OK) return status;
     kmc_host::coef_launcher_fn launch = find_launcher(params->kernel.inner_operator, params->kernel.inner_power);
     if (params->kernel.flags & KMC_FLAG_L2_GRAM) {
@@ -94,7 +99,7 @@ int kmc_kernel_times_coefficients_jit(void *function, const kmc_kernel_coefficie
     int load_a = 0, load_b = 0;
     dim3 grid;
     bool empty = false;
-    int status = prepare(params, &kc, &load_a, &load_b, &grid, &empty);
+    int status = prepare(params, false, &kc, &load_a, &load_b, &grid, &empty);
     if (status != KMC_OK) return status;
     if (empty) return KMC_OK;
     status = require_gfx950();

@@ -30,27 +30,33 @@ typedef float kc_float4 __attribute__((ext_vector_type(4)));
 struct KernelCoefficientsArgs {
     BuildKernelArgs kernel;        // c / c_ld / c_bs unused
     int o;                         // coefficient columns in total
-    int o_chunks;                  // ceil(o / 32); blockIdx.y = batch * o_chunks + chunk
+    int o_chunks;                  // ceil(o / columns); blockIdx.y = batch * o_chunks + chunk
     const float *coef; i64 coef_ld, coef_bs;   // [n, o], o contiguous
     float *out; i64 out_ld, out_bs;            // [m, o], o contiguous
     int coef_vec;                  // coef, coef_ld, coef_bs multiples of 16 bytes
+    int columns;                   // coefficient columns per workgroup: the COLUMNS the launched kernel was built with
 };
 
-constexpr int KC_COLUMNS = 32;      // coefficient columns per workgroup
+constexpr int KC_COLUMNS = 32;      // coefficient columns per workgroup (64 in the wide instantiations)
 constexpr int KC_PASS_N = 32;       // n per contraction pass
 // [n][m] pitch of the kernel values in LDS: the 4 n-rows an MFMA operand read
 // touches land in 4 disjoint groups of 16 banks.
 constexpr int KC_KV_PITCH = BK_TILE_M + 16;
 constexpr int KC_STAGE_FLOATS = 2 * (2 * BK_LDS_SLICE + BK_LDS_PITCH);
 
-template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
+// COLUMNS: 32, or 64 for more than 32 coefficient columns (every chunk of columns
+// rebuilds the whole kernel matrix, so O = 64 in two chunks of 32 costs twice O = 32;
+// 64 columns per workgroup still leave LDS for two workgroups per CU).
+template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B, int COLUMNS = KC_COLUMNS>
 __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const KernelCoefficientsArgs kc)
 {
+    static_assert(COLUMNS % 32 == 0, "whole pairs of 16-column blocks");
+    constexpr int COLUMN_BLOCKS = COLUMNS / 16;
     static_assert(KC_PASS_N * KC_KV_PITCH <= KC_STAGE_FLOATS, "kernel values must fit in the staging buffers");
     // Staging buffers of the K walk; between two K walks the same memory holds
     // one pass of kernel values.
     __shared__ __attribute__((aligned(16))) float lds_stage[KC_STAGE_FLOATS];
-    __shared__ __attribute__((aligned(16))) float lds_coef[BK_TILE_N * KC_COLUMNS];   // [n][o]
+    __shared__ __attribute__((aligned(16))) float lds_coef[BK_TILE_N * COLUMNS];   // [n][o]
     float *lds_a = lds_stage;
     float *lds_b = lds_stage + KC_STAGE_FLOATS / 2;
     float *lds_kv = lds_stage;
@@ -60,7 +66,7 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
     const int tx = tid & 15;
     const int ty = tid >> 4;
     const int batch = blockIdx.y / kc.o_chunks;
-    const int o_base = (blockIdx.y % kc.o_chunks) * KC_COLUMNS;
+    const int o_base = (blockIdx.y % kc.o_chunks) * COLUMNS;
     const int m0 = blockIdx.x * BK_TILE_M;
     const int m_valid = args.m - m0;
 
@@ -70,7 +76,7 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
     }
 
     // Contraction role (v_mfma_f32_16x16x4_f32, lane = 16 q + r): wave w owns rows
-    // 32 w .. 32 w + 31 as two row blocks of 16, times two column blocks of 16.
+    // 32 w .. 32 w + 31 as two row blocks of 16, times COLUMNS / 16 column blocks of 16.
     // Operand A: lane supplies Kv[m = r][n = q]; operand B: coef[n = q][o = r];
     // result: lane holds rows 4 q .. 4 q + 3 of column r.
     const int lane = tid & 63;
@@ -79,30 +85,30 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
     const int r = lane & 15;
     const float *coef_batch = kc.coef + batch * kc.coef_bs;
     const bool coef_vec = kc.coef_vec;
-    kc_float4 out_acc[2][2];   // [row block][column block]
+    kc_float4 out_acc[2][COLUMN_BLOCKS];   // [row block][column block]
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-        for (int ob = 0; ob < 2; ob++) out_acc[mb][ob] = kc_float4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int ob = 0; ob < COLUMN_BLOCKS; ob++) out_acc[mb][ob] = kc_float4{0.0f, 0.0f, 0.0f, 0.0f};
 
     for (int n0 = 0; n0 < args.n; n0 += BK_TILE_N) {
         const int n_valid = args.n - n0;
 
         // 1. coefficients of this n tile -> LDS, zero filled past N and past O.
-        //    Lane t stages row t/2, columns 16*(t&1) .. +15.  The barrier that ends
+        //    Lane t stages row t/2, half t&1 of the columns.  The barrier that ends
         //    the previous tile's last pass protects lds_coef; the barriers inside
         //    the K walk below publish it.
         {
             const int n_local = tid >> 1;
-            const int c0 = (tid & 1) * 16;
+            const int c0 = (tid & 1) * (COLUMNS / 2);
             const bool row_live = n_local < n_valid;
             const float *src = coef_batch + (i64)(n0 + n_local) * kc.coef_ld + o_base + c0;
 #pragma unroll
-            for (int v4 = 0; v4 < 4; v4++) {
+            for (int v4 = 0; v4 < COLUMNS / 8; v4++) {
                 const int cols_left = kc.o - (o_base + c0 + 4 * v4);
                 float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 if (row_live) v = load4_guarded(src + 4 * v4, cols_left, coef_vec);
-                *reinterpret_cast<float4 *>(lds_coef + n_local * KC_COLUMNS + c0 + 4 * v4) = v;
+                *reinterpret_cast<float4 *>(lds_coef + n_local * COLUMNS + c0 + 4 * v4) = v;
             }
         }
 
@@ -147,29 +153,27 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
             }
             __syncthreads();
             const float *kv_src = lds_kv + q * KC_KV_PITCH + wave * 32 + r;
-            const float *coef_src = lds_coef + (pass * KC_PASS_N + q) * KC_COLUMNS + r;
+            const float *coef_src = lds_coef + (pass * KC_PASS_N + q) * COLUMNS + r;
             // Operand double buffer: reads of chunk c+1 go out before the MFMAs of chunk c.
-            float fa[2][2], fb[2][2];
+            float fa[2][2], fb[2][COLUMN_BLOCKS];
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                fa[0][t] = kv_src[t * 16];
-                fb[0][t] = coef_src[t * 16];
-            }
+            for (int t = 0; t < 2; t++) fa[0][t] = kv_src[t * 16];
+#pragma unroll
+            for (int t = 0; t < COLUMN_BLOCKS; t++) fb[0][t] = coef_src[t * 16];
 #pragma unroll
             for (int chunk = 0; chunk < KC_PASS_N / 4; chunk++) {
                 const int use = chunk & 1;
                 if (chunk + 1 < KC_PASS_N / 4) {
 #pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        fa[use ^ 1][t] = kv_src[(chunk + 1) * 4 * KC_KV_PITCH + t * 16];
-                        fb[use ^ 1][t] = coef_src[(chunk + 1) * 4 * KC_COLUMNS + t * 16];
-                    }
+                    for (int t = 0; t < 2; t++) fa[use ^ 1][t] = kv_src[(chunk + 1) * 4 * KC_KV_PITCH + t * 16];
+#pragma unroll
+                    for (int t = 0; t < COLUMN_BLOCKS; t++) fb[use ^ 1][t] = coef_src[(chunk + 1) * 4 * COLUMNS + t * 16];
                 }
                 __builtin_amdgcn_sched_barrier(0);   // keep those reads above the MFMAs
 #pragma unroll
                 for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-                    for (int ob = 0; ob < 2; ob++)
+                    for (int ob = 0; ob < COLUMN_BLOCKS; ob++)
                         out_acc[mb][ob] =
                             __builtin_amdgcn_mfma_f32_16x16x4f32(fa[use][mb], fb[use][ob], out_acc[mb][ob], 0, 0, 0);
             }
@@ -182,7 +186,7 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-        for (int ob = 0; ob < 2; ob++) {
+        for (int ob = 0; ob < COLUMN_BLOCKS; ob++) {
             const int o = o_base + ob * 16 + r;
             if (o >= kc.o) continue;
 #pragma unroll

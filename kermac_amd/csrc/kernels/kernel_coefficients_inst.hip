@@ -1,5 +1,6 @@
 // One (inner operator, inner power) pair of the fused kernel-matrix x
-// coefficients kernel, instantiated for all 16 (A loader, B loader) pairs.
+// coefficients kernel, instantiated for all 16 (A loader, B loader) pairs and for 32
+// and 64 coefficient columns per workgroup.
 // Compiled several times with different -DKMC_INNER_OP / -DKMC_INNER_POW.
 #include <hip/hip_runtime.h>
 
@@ -18,8 +19,15 @@ namespace kmc_host {
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::KernelCoefficientsArgs &args, dim3 grid, hipStream_t stream)
 {
-    hipLaunchKernelGGL((kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>), grid,
-                       dim3(kmc::BK_THREADS), 0, stream, args);
+    if (args.columns == 64) {
+        hipLaunchKernelGGL((kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B, 64>), grid,
+                           dim3(kmc::BK_THREADS), 0, stream, args);
+    } else if (args.columns == kmc::KC_COLUMNS) {
+        hipLaunchKernelGGL((kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>), grid,
+                           dim3(kmc::BK_THREADS), 0, stream, args);
+    } else {
+        return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

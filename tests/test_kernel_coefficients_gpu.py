@@ -29,7 +29,7 @@ def test_golden_vector(device):
 
 
 @pytest.mark.parametrize("M,N,K,O", [(1, 1, 1, 1), (130, 200, 17, 5), (128, 128, 16, 32), (257, 129, 40, 33),
-                                     (90, 300, 6, 70), (64, 31, 33, 16)])
+                                     (90, 300, 6, 70), (64, 31, 33, 16), (200, 150, 24, 64), (140, 260, 19, 129)])
 @pytest.mark.parametrize("layout", ["cc", "rr", "cr"])
 def test_shapes_and_layouts(device, M, N, K, O, layout):
     g = torch.Generator().manual_seed(M + N + K + O)
