@@ -422,7 +422,13 @@ __device__ __forceinline__ void finish_tile(
 // band; the padding workgroups get `false` and exit at once.
 __device__ __forceinline__ bool tile_of_workgroup(const BuildKernelArgs &args, int &tile_m, int &tile_n)
 {
-    const int linear = blockIdx.x;
+    // Batches rotate the order by one: the hardware derives the XCD from the launch-wide
+    // workgroup id, which is blockIdx.x modulo 8 for every batch (the grid width is a
+    // multiple of 8), so without the rotation a batch of problems of one tile each would
+    // run on a single XCD.  The residue classes modulo 8, and with them the ownership
+    // described above, survive the rotation.
+    const int rotated = blockIdx.x + blockIdx.y % gridDim.x;
+    const int linear = rotated >= (int)gridDim.x ? rotated - (int)gridDim.x : rotated;
     const int band_tiles = BK_BAND_N * args.tiles_m;
     const int band = linear / band_tiles;
     const int band_height = min(BK_BAND_N, args.tiles_n_padded - band * BK_BAND_N);
