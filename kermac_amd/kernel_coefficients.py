@@ -96,7 +96,7 @@ def _plan_run_kernel_coefficients(
 def run_kernel_coefficients(
     kernel_descriptor, a, b, coefficients, out: Optional[torch.Tensor] = None, p=None, inner_p=None, outer_p=None,
     bandwidth=None, epsilon=None, regularization=None, regularization_offset_x: int = 0,
-    regularization_offset_y: int = 0, debug=False,
+    regularization_offset_y: int = 0, debug=False, _may_split=True,
 ):
     """``out[l, m, o] = sum_n run_kernel(descriptor, a, b, ...)[l, m, n] * coefficients[l, n, o]``.
 
@@ -109,6 +109,11 @@ def run_kernel_coefficients(
     plan = _plan_run_kernel_coefficients(
         kernel_descriptor, a, b, coefficients, out, p, inner_p, outer_p, bandwidth, epsilon, regularization,
         regularization_offset_x, regularization_offset_y)
+    split = _split_over_centres(plan, a, b, coefficients, regularization) if _may_split else None
+    if split is not None:
+        _run_split_over_centres(split, plan, kernel_descriptor, a, b, coefficients, p, inner_p, outer_p, bandwidth,
+                                epsilon, debug)
+        return plan.out
     stream = _current_stream_for(a.device)
     params = plan.params
     kernel = params.kernel
@@ -125,3 +130,57 @@ def run_kernel_coefficients(
                 print(f"(Kermac Debug) Launching kernel: {name}")
             _backend.kernel_times_coefficients_jit(function, params, stream)
     return plan.out
+
+
+# A workgroup of the fused kernel owns 128 rows of ``a`` and walks every centre, so a
+# launch has ceil(M / 128) x L x ceil(O / 64) workgroups: few rows against many centres
+# (prediction for a small batch of points) would leave most of the 256 CUs idle.  Such a
+# call is cut over the centres instead: slices of ``b`` and ``coefficients`` become the
+# batch of one launch (``a`` broadcasts), each slice writes its own partial result, and
+# the partial results are summed in a fixed order.
+_SPLIT_BELOW_WORKGROUPS = 192
+_SPLIT_TARGET_WORKGROUPS = 512
+_SPLIT_MIN_CENTRES = 512
+
+
+def _split_over_centres(plan, a, b, coefficients, regularization):
+    """(slices, rows per slice, leftover rows), or None when the call is launched as it is."""
+    if plan.L != 1:
+        return None                      # batched calls fill the grid with their batches
+    if regularization is not None and not (isinstance(regularization, (int, float)) and regularization == 0):
+        return None                      # the regularised diagonal is addressed by the global centre index
+    M, N, O = plan.M, plan.N, plan.O
+    workgroups = -(-M // 128) * max(1, -(-O // 64))
+    if M == 0 or O == 0 or workgroups >= _SPLIT_BELOW_WORKGROUPS or N < 2 * _SPLIT_MIN_CENTRES:
+        return None
+    # Slices of a whole number of tiles each (a 16-byte aligned operand then stays aligned in every
+    # slice); the rows that remain go into a second launch.  Two workgroups fit on a CU, so a launch
+    # costs its centres per workgroup times its rounds of 512 workgroups: take the cheapest cut.
+    best = None
+    for slices in range(2, min(_SPLIT_TARGET_WORKGROUPS // workgroups, N // _SPLIT_MIN_CENTRES) + 1):
+        for rows in (N // slices // 128 * 128, -(-N // slices // 128) * 128):
+            if rows < _SPLIT_MIN_CENTRES:
+                continue
+            full = N // rows
+            leftover = N - full * rows
+            cost = rows * -(-full * workgroups // _SPLIT_TARGET_WORKGROUPS) + leftover
+            if full >= 2 and (best is None or cost < best[0]):
+                best = (cost, full, rows, leftover)
+    return best[1:] if best else None
+
+
+def _run_split_over_centres(split, plan, kernel_descriptor, a, b, coefficients, p, inner_p, outer_p, bandwidth, epsilon,
+                            debug):
+    full, rows, leftover = split
+    a2, b2, c2 = (t[0] if t.dim() == 3 else t for t in (a, b, coefficients))
+    M, K, O = plan.M, plan.K, plan.O
+    partial = torch.empty((full + (1 if leftover else 0), M, O), dtype=torch.float32, device=a.device)
+    b_slices = b2.as_strided((full, rows, K), (rows * b2.stride(0), b2.stride(0), b2.stride(1)), b2.storage_offset())
+    c_slices = c2.as_strided((full, rows, O), (rows * c2.stride(0), c2.stride(0), c2.stride(1)), c2.storage_offset())
+    hyper = dict(p=p, inner_p=inner_p, outer_p=outer_p, bandwidth=bandwidth, epsilon=epsilon, debug=debug,
+                 _may_split=False)
+    run_kernel_coefficients(kernel_descriptor, a2, b_slices, c_slices, partial[:full], **hyper)
+    if leftover:
+        run_kernel_coefficients(kernel_descriptor, a2, b2[full * rows:], c2[full * rows:], partial[full:], **hyper)
+    target = plan.out[0] if plan.out.dim() == 3 else plan.out
+    torch.sum(partial, dim=0, out=target)

@@ -112,3 +112,30 @@ def test_no_centres_gives_zeros(device):
     got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, torch.zeros(0, 6, device=device), bandwidth=2.0,
                             coefficients=torch.zeros(0, 7, device=device))
     assert got.shape == (1, 200, 7) and torch.all(got == 0)
+
+
+@pytest.mark.parametrize("M,N,K,O,layout", [(130, 5077, 24, 3, "cc"), (1000, 20000, 16, 1, "rr"), (64, 4096, 33, 70, "cr"),
+                                            (300, 1024, 8, 5, "rc")])
+def test_few_rows_many_centres_are_cut_over_the_centres(device, M, N, K, O, layout):
+    """Few rows against many centres: the call becomes one batched launch over slices of the
+    centres plus a fixed-order sum of the partial results (kermac_amd/kernel_coefficients.py);
+    same values as the composition, into a caller's strided out as well."""
+    from kermac_amd import kernel_coefficients as kc
+    g = torch.Generator().manual_seed(M + N + K + O)
+    a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False, dist="rand")
+    b = make_operand(1, N, K, layout[1] == "c", device, g, batch=False, dist="rand")
+    coef = torch.randn(N, O, generator=g).to(device)
+    plan = kc._plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l1, a, b, coef, None, None, None, None, 2.0,
+                                            None, None, 0, 0)
+    assert kc._split_over_centres(plan, a, b, coef, None) is not None
+    assert kc._split_over_centres(plan, a, b, coef, 0.5) is None        # the regularised diagonal needs global indices
+    got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, bandwidth=2.0)
+    assert got.shape == (1, M, O)
+    truth = oracle.kernel_times_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", a.cpu(), b.cpu(), coef.cpu(), bandwidth=2.0)
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="split over centres")
+    unsplit = kc.run_kernel_coefficients(kermac.kernel_descriptor_laplace_l1, a, b, coef, bandwidth=2.0, _may_split=False)
+    torch.testing.assert_close(got, unsplit, rtol=1e-5, atol=atol_for(truth, 1e-5))
+    wide = torch.full((M, O + 3), -7.0, device=device)
+    out = wide[:, :O]
+    assert kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, bandwidth=2.0, out=out) is out
+    assert torch.equal(out, got[0]) and torch.all(wide[:, O:] == -7.0)
