@@ -140,6 +140,7 @@ def cdist_grad(
     out: torch.Tensor = None,  # [O,N,M] m contiguous   grad
     p: Union[float, torch.Tensor] = 2.0,
     debug=False,
+    _may_split=True,
 ):
     """Gradient of the p-norm kernel contracted with coefficients::
 
@@ -154,9 +155,56 @@ def cdist_grad(
         ValueError: bad shapes, strides, batch sizes or devices.
     """
     plan = _plan_cdist_grad(a, b, c, d, out, p)
+    split = _split_over_contraction(plan) if _may_split else None
+    if split is not None:
+        _run_split_over_contraction(split, plan, a, b, c, d, p, debug)
+        return plan.out
     stream = _current_stream_for(a.device)
     if debug:
         print(f"(Kermac Debug) Launching kernel: norm_kernel_gradient<{('L1', 'L2', 'P')[plan.params.norm_type]}>")
     with torch.cuda.device(a.device):
         _backend.norm_kernel_gradient(plan.params, stream)
     return plan.out
+
+
+# A workgroup owns 64 (m) x 32 or 16 (n) results and walks the whole contraction index k,
+# so few samples and features against many centres (M = 2000, N = 100, K = 10000) launch a
+# hundred workgroups on 256 CUs.  Such an unbatched call is cut over k: slices of a, b and
+# c become the batch of one launch through strided views (d broadcasts), every slice writes
+# a partial result, and the partial results are summed in a fixed order.
+_SPLIT_BELOW_WORKGROUPS = 256
+_SPLIT_TARGET_WORKGROUPS = 768
+_SPLIT_MIN_DEPTH = 1024
+
+
+def _split_over_contraction(plan):
+    """(slices, k per slice, leftover k), or None when the call is launched as it is."""
+    if plan.L != 1 or plan.M == 0 or plan.N == 0 or plan.O == 0:
+        return None
+    M, N, O, K = plan.M, plan.N, plan.O, plan.K
+    n_tile = 32 if O <= 8 else 16
+    workgroups = -(-M // 64) * -(-N // n_tile) * max(1, -(-O // 32))
+    if workgroups >= _SPLIT_BELOW_WORKGROUPS or K < 2 * _SPLIT_MIN_DEPTH:
+        return None
+    slices = min(_SPLIT_TARGET_WORKGROUPS // workgroups, K // _SPLIT_MIN_DEPTH)
+    if slices < 2:
+        return None
+    depth = K // slices // 64 * 64       # whole K slices of the kernels; 16-byte alignment survives
+    slices = K // depth
+    return slices, depth, K - slices * depth
+
+
+def _run_split_over_contraction(split, plan, a, b, c, d, p, debug):
+    slices, depth, leftover = split
+    a2, b2, c2, d2 = (t[0] if t.dim() == 3 else t for t in (a, b, c, d))
+    M, N, O = plan.M, plan.N, plan.O
+    partial = torch.empty((slices + (1 if leftover else 0), O, N, M), dtype=torch.float32, device=a.device)
+    a_slices = a2.as_strided((slices, depth, M), (depth * a2.stride(0), a2.stride(0), a2.stride(1)), a2.storage_offset())
+    b_slices = b2.as_strided((slices, N, depth), (depth * b2.stride(1), b2.stride(0), b2.stride(1)), b2.storage_offset())
+    c_slices = c2.as_strided((slices, O, depth), (depth * c2.stride(1), c2.stride(0), c2.stride(1)), c2.storage_offset())
+    cdist_grad(a_slices, b_slices, c_slices, d2, out=partial[:slices], p=p, debug=debug, _may_split=False)
+    if leftover:
+        done = slices * depth
+        cdist_grad(a2[done:], b2[:, done:], c2[:, done:], d2, out=partial[slices:], p=p, debug=debug, _may_split=False)
+    target = plan.out[0] if plan.out.dim() == 4 else plan.out
+    torch.sum(partial, dim=0, out=target)

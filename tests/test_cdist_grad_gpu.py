@@ -160,3 +160,27 @@ def test_gradient_empty_contraction_writes_zeros(device):
     got = kermac.cdist_grad(torch.zeros(0, 70, device=device), torch.zeros(9, 0, device=device),
                             torch.zeros(5, 0, device=device), torch.randn(9, 70, device=device), p=1.0)
     assert got.shape == (1, 5, 9, 70) and torch.all(got == 0)
+
+
+@pytest.mark.parametrize("p", [1.0, 2.0, 1.3])
+@pytest.mark.parametrize("M,N,O,K", [(200, 40, 1, 4100), (130, 10, 3, 2048), (64, 100, 16, 5000)])
+def test_few_results_deep_contraction_is_cut_over_k(device, p, M, N, O, K):
+    """Few (m, n) results against a long contraction: one batched launch over slices of k plus a
+    fixed-order sum of the partial results (kermac_amd/cdist_grad.py); same values as one walk."""
+    import importlib
+    module = importlib.import_module("kermac_amd.cdist_grad")    # the package attribute of that name is the function
+    g = torch.Generator().manual_seed(M + N + O + K)
+    a = torch.rand(K, M, generator=g).to(device)
+    b = torch.randn(N, K, generator=g).to(device)
+    c = torch.randn(O, K, generator=g).to(device)
+    d = torch.randn(N, M, generator=g).to(device)
+    assert module._split_over_contraction(module._plan_cdist_grad(a, b, c, d, None, p)) is not None
+    got = kermac.cdist_grad(a, b, c, d, p=p)
+    assert got.shape == (1, O, N, M)
+    truth = oracle.cdist_grad(a.cpu(), b.cpu(), c.cpu(), d.cpu(), p=p)
+    rtol, atol = tolerances(p, truth)
+    assert_close_to_truth(got, truth, rtol=rtol, atol=atol, what=f"grad cut over k {M}x{N}x{O}x{K} p={p}")
+    wide = torch.full((O, N, M + 4), -7.0, device=device)
+    out = wide[:, :, :M]
+    assert kermac.cdist_grad(a, b, c, d, out=out, p=p) is out
+    assert torch.equal(out, got[0]) and torch.all(wide[:, :, M:] == -7.0)
