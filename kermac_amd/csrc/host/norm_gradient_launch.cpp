@@ -38,7 +38,7 @@ extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void 
     // The outputs are cut into at most three runs, each with the kernel that suits its
     // width: whole groups of 32 (and a remainder of 25..31) on the matrix-core kernel with
     // 32 output columns, a remainder of 9..24 as 16 columns on the matrix-core kernel with
-    // 16 plus, above 16, the rest on the vector-ALU kernel, which holds 1, 2, 4 or 8
+    // 16 plus, above 16, the rest on the vector-ALU kernel, which holds 1 to 6 or 8
     // accumulators per (m, n).  O = 17 therefore costs a 16-wide and a 1-wide launch
     // instead of one 32-wide launch that is half padding (18.5 -> 12.4 ms at M = K = 8192,
     // N = 512 for the L1 norm; O = 48: 36.6 -> 28.0 ms).
@@ -46,7 +46,9 @@ extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void 
     Run runs[3];
     int run_count = 0;
     {
-        auto small_tile = [](int o) { return o <= 1 ? 1 : o <= 2 ? 2 : o <= 4 ? 4 : 8; };
+        // the vector-ALU kernel exists for the widths 1..6 and 8 (7 accumulators per (m, n) measured
+        // slower than 8 with one padded: 7.8 against 7.3 ms)
+        auto small_tile = [](int o) { return o == 7 ? 8 : o; };
         int begin = 0, left = p->o;
         const int wide = left % 32 >= 25 ? left : left - left % 32;     // columns for the 32-wide kernel
         if (wide > 0) { runs[run_count++] = {begin, wide, 32}; begin += wide; left -= wide; }

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(NG_THREADS) void norm_kernel_gradient(const NormGra
             }
     };
     auto read_c = [&](float (&fc)[O_TILE], const float *src) {
-        if (O_TILE < 4) {
+        if (O_TILE % 4 != 0) {     // rows of O_TILE floats are not 16-byte aligned: scalar (broadcast) reads
 #pragma unroll
             for (int o = 0; o < O_TILE; o++) fc[o] = src[o];
             return;

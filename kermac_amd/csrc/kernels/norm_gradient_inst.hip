@@ -1,5 +1,5 @@
 // Ahead-of-time instantiations of the kernel-gradient contraction: 3 norm types
-// x (vector-ALU kernel with 1, 2, 4 or 8 outputs per lane tile, matrix-core kernel with
+// x (vector-ALU kernel with 1 to 6 or 8 outputs per lane tile, matrix-core kernel with
 // 16 or 32 output columns, with and without a partial last K slice).
 #include <hip/hip_runtime.h>
 
@@ -15,7 +15,10 @@ static hipError_t launch_norm(int o_tile, const kmc::NormGradientArgs &args, dim
     switch (o_tile) {
     case 1: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 1>), grid, block, 0, stream, args); break;
     case 2: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 2>), grid, block, 0, stream, args); break;
+    case 3: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 3>), grid, block, 0, stream, args); break;
     case 4: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 4>), grid, block, 0, stream, args); break;
+    case 5: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 5>), grid, block, 0, stream, args); break;
+    case 6: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 6>), grid, block, 0, stream, args); break;
     case 8: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 8>), grid, block, 0, stream, args); break;
     case 16:
         if (k_tail) hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 1, true>), grid, block, 0, stream, args);

@@ -58,7 +58,7 @@ def test_gradient_reference_test_case(device):
 
 @pytest.mark.parametrize("p", [1.0, 2.0, 1.3, 0.7])
 @pytest.mark.parametrize("M,N,O,K", [(1, 1, 1, 1), (70, 33, 3, 17), (64, 32, 16, 16), (65, 31, 5, 50), (200, 40, 20, 35),
-                                     (130, 64, 8, 100), (129, 66, 1, 48), (256, 64, 2, 64), (67, 35, 2, 19),
+                                     (130, 64, 8, 100), (129, 66, 1, 48), (256, 64, 2, 64), (67, 35, 2, 19), (128, 64, 7, 32), (90, 40, 6, 21),
                                      # output counts that are cut into runs for kernels of different width
                                      (96, 24, 17, 20), (80, 20, 33, 33), (70, 18, 49, 16), (66, 17, 57, 21), (64, 16, 90, 16)])
 def test_gradient_ragged_shapes(device, p, M, N, O, K):
