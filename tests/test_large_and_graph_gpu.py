@@ -174,3 +174,53 @@ def test_operators_replay_from_a_hip_graph(device):
             assert torch.equal(e, o), f"replay {replay}: {name} differs from the eager result"
     truth = oracle.cdist(a_store.t().cpu(), b_store.t().cpu(), p=1.0)[0]
     assert_close_to_truth(out_p1.t(), truth, rtol=1e-5, what="graph replay vs oracle")
+
+
+def test_concurrent_host_threads_on_their_own_streams(device):
+    """Four host threads, each with its own stream, call the three operators at the same
+    time; ctypes releases the interpreter lock during the launches, so this exercises the
+    thread-local error state and the absence of shared mutable state on the launch path."""
+    import threading
+    g = torch.Generator().manual_seed(99)
+    problems = []
+    for t in range(4):
+        M, N, K, O = 200 + 37 * t, 150 + 11 * t, 48 + 5 * t, 3 + t
+        a = torch.rand(M, K, generator=g).to(device)
+        b = torch.rand(N, K, generator=g).to(device)
+        grad = [torch.rand(K, M, generator=g).to(device), torch.randn(N, K, generator=g).to(device),
+                torch.randn(O, K, generator=g).to(device), torch.randn(N, M, generator=g).to(device)]
+        coef = torch.randn(N, O, generator=g).to(device)
+        problems.append((a, b, grad, coef))
+    results, errors = [None] * 4, []
+    torch.cuda.synchronize()
+
+    def work(t):
+        try:
+            a, b, grad, coef = problems[t]
+            stream = torch.cuda.Stream(device=device)
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    d1 = kermac.cdist(a, b, p=1.0)
+                    d13 = kermac.cdist(a, b, p=1.3)
+                    e = kermac.cdist_grad(*grad, p=1.0)
+                    f = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, bandwidth=2.0)
+            stream.synchronize()
+            results[t] = (d1, d13, e, f)
+        except Exception as exc:       # reported by the main thread
+            errors.append((t, exc))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for t, (a, b, grad, coef) in enumerate(problems):
+        d1, d13, e, f = results[t]
+        cpu = [x.cpu() for x in (a, b)]
+        assert_close_to_truth(d1, oracle.cdist(*cpu, p=1.0), rtol=1e-5, what=f"thread {t} p=1")
+        assert_close_to_truth(d13, oracle.cdist(*cpu, p=1.3), rtol=1e-4, what=f"thread {t} p=1.3")
+        truth = oracle.cdist_grad(*[x.cpu() for x in grad], p=1.0)
+        assert_close_to_truth(e, truth, rtol=1e-5, atol=1e-5 * truth.abs().max().item(), what=f"thread {t} grad")
+        truth = oracle.kernel_times_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", *cpu, coef.cpu(), bandwidth=2.0)
+        assert_close_to_truth(f, truth, rtol=1e-5, atol=1e-5 * truth.abs().max().item(), what=f"thread {t} fused")
