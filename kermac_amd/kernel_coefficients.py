@@ -133,40 +133,55 @@ def run_kernel_coefficients(
 
 
 # A workgroup of the fused kernel owns 128 rows of ``a`` and walks every centre, so a
-# launch has ceil(M / 128) x L x ceil(O / 64) workgroups: few rows against many centres
-# (prediction for a small batch of points) would leave most of the 256 CUs idle.  Such a
-# call is cut over the centres instead: slices of ``b`` and ``coefficients`` become the
-# batch of one launch (``a`` broadcasts), each slice writes its own partial result, and
-# the partial results are summed in a fixed order.
-_SPLIT_BELOW_WORKGROUPS = 192
-_SPLIT_TARGET_WORKGROUPS = 512
+# launch has ceil(M / 128) x L x ceil(O / 64) long-running workgroups, of which 512 run at
+# a time (two per CU).  Few rows against many centres (prediction for a small batch of
+# points) would leave most of the chip idle, and a count just above a multiple of 512
+# leaves it idle for most of the last round.  Such an unbatched call is cut over the
+# centres: slices of ``b`` and ``coefficients`` become the batch of one launch (``a``
+# broadcasts), each slice writes its own partial result, and the partial results are summed
+# in a fixed order.
+_SPLIT_CONCURRENT_WORKGROUPS = 512
 _SPLIT_MIN_CENTRES = 512
+_SPLIT_WORKGROUP_OVERHEAD = 64           # start-up and store of a workgroup, in centres walked
+_SPLIT_MAX_PARTIAL_BYTES = 256 << 20
+_SPLIT_WORTH = 0.85                      # cut only for at least 15 % less modelled time
 
 
 def _split_over_centres(plan, a, b, coefficients, regularization):
     """(slices, rows per slice, leftover rows), or None when the call is launched as it is."""
     if plan.L != 1:
-        return None                      # batched calls fill the grid with their batches
+        return None                      # the batch index of the launch is taken by the caller's batches
     if regularization is not None and not (isinstance(regularization, (int, float)) and regularization == 0):
         return None                      # the regularised diagonal is addressed by the global centre index
     M, N, O = plan.M, plan.N, plan.O
-    workgroups = -(-M // 128) * max(1, -(-O // 64))
-    if M == 0 or O == 0 or workgroups >= _SPLIT_BELOW_WORKGROUPS or N < 2 * _SPLIT_MIN_CENTRES:
+    if M == 0 or O == 0 or N < 2 * _SPLIT_MIN_CENTRES:
         return None
-    # Slices of a whole number of tiles each (a 16-byte aligned operand then stays aligned in every
-    # slice); the rows that remain go into a second launch.  Two workgroups fit on a CU, so a launch
-    # costs its centres per workgroup times its rounds of 512 workgroups: take the cheapest cut.
+    workgroups = -(-M // 128) * max(1, -(-O // 64))
+
+    def rounds(count):
+        return -(-count // _SPLIT_CONCURRENT_WORKGROUPS)
+
+    # Modelled time of a launch: centres walked per workgroup (plus its fixed cost) times rounds of
+    # workgroups.  Slices are a whole number of tiles each, so a 16-byte aligned operand stays
+    # aligned in every slice; the rows that remain go into a second launch.
+    unsplit = (N + _SPLIT_WORKGROUP_OVERHEAD) * rounds(workgroups)
+    most = min(N // _SPLIT_MIN_CENTRES, _SPLIT_MAX_PARTIAL_BYTES // (4 * M * O) - 1,
+               max(16, _SPLIT_CONCURRENT_WORKGROUPS // workgroups))
     best = None
-    for slices in range(2, min(_SPLIT_TARGET_WORKGROUPS // workgroups, N // _SPLIT_MIN_CENTRES) + 1):
+    for slices in range(2, most + 1):
         for rows in (N // slices // 128 * 128, -(-N // slices // 128) * 128):
             if rows < _SPLIT_MIN_CENTRES:
                 continue
             full = N // rows
             leftover = N - full * rows
-            cost = rows * -(-full * workgroups // _SPLIT_TARGET_WORKGROUPS) + leftover
+            cost = (rows + _SPLIT_WORKGROUP_OVERHEAD) * rounds(full * workgroups)
+            if leftover:
+                cost += (leftover + _SPLIT_WORKGROUP_OVERHEAD) * rounds(workgroups)
             if full >= 2 and (best is None or cost < best[0]):
                 best = (cost, full, rows, leftover)
-    return best[1:] if best else None
+    if best is None or best[0] > _SPLIT_WORTH * unsplit:
+        return None
+    return best[1:]
 
 
 def _run_split_over_centres(split, plan, kernel_descriptor, a, b, coefficients, p, inner_p, outer_p, bandwidth, epsilon,
