@@ -176,6 +176,62 @@ def test_operators_replay_from_a_hip_graph(device):
     assert_close_to_truth(out_p1.t(), truth, rtol=1e-5, what="graph replay vs oracle")
 
 
+def test_cut_launches_replay_from_a_hip_graph(device):
+    """The calls that the Python layer cuts into a batched launch plus a sum of partial results
+    (few rows against many centres; few results with a deep contraction) allocate a buffer and
+    call a library reduction: captured, every replay must equal the eager result bit for bit."""
+    import importlib
+    grad_module = importlib.import_module("kermac_amd.cdist_grad")
+    from kermac_amd import kernel_coefficients as coef_module
+    g = torch.Generator().manual_seed(2035)
+    M, N, K, O = 200, 5077, 40, 3
+    x = torch.rand(M, K, generator=g).to(device)
+    z = torch.rand(N, K, generator=g).to(device)
+    coef = torch.randn(N, O, generator=g).to(device)
+    out_fused = torch.empty(1, M, O, device=device)
+    plan = coef_module._plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l1, x, z, coef, None, None, None,
+                                                     None, 2.0, None, None, 0, 0)
+    assert coef_module._split_over_centres(plan, x, z, coef, None) is not None
+    weights = torch.rand(4100, 150, generator=g).to(device)     # cdist_grad's a[K', M']
+    centres = torch.randn(30, 4100, generator=g).to(device)     # b[N', K']
+    classes = torch.randn(2, 4100, generator=g).to(device)      # c[O', K']
+    samples = torch.randn(30, 150, generator=g).to(device)      # d[N', M']
+    out_grad = torch.empty(2, 30, 150, device=device)
+    assert grad_module._split_over_contraction(
+        grad_module._plan_cdist_grad(weights, centres, classes, samples, None, 1.0)) is not None
+
+    def run_all():
+        kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, z, out=out_fused, bandwidth=2.0, coefficients=coef)
+        kermac.cdist_grad(weights, centres, classes, samples, out=out_grad, p=1.0)
+
+    outs = (out_fused, out_grad)
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run_all()                                               # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run_all()
+    for replay in range(4):
+        x.copy_(torch.rand(M, K, generator=g))                  # new values, same addresses
+        samples.mul_(1.25)
+        run_all()
+        torch.cuda.synchronize()
+        eager = [o.clone() for o in outs]
+        for o in outs:
+            o.fill_(float("nan"))
+        scratch = torch.randn(256, 256, device=device) @ torch.randn(256, 256, device=device)   # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        del scratch
+        for name, e, o in zip(("fused", "grad"), eager, outs):
+            assert torch.equal(e, o), f"replay {replay}: {name} differs from the eager result"
+    truth = oracle.kernel_times_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu(), z.cpu(), coef.cpu(), bandwidth=2.0)
+    assert_close_to_truth(out_fused, truth, rtol=1e-5, atol=1e-5 * truth.abs().max().item(), what="cut fused replay")
+
+
 def test_concurrent_host_threads_on_their_own_streams(device):
     """Four host threads, each with its own stream, call the three operators at the same
     time; ctypes releases the interpreter lock during the launches, so this exercises the
