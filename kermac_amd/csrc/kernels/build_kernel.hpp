@@ -516,24 +516,59 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
         }
     }
 
-    // Symmetric result: the same values also belong at C(n, m).  There the four
-    // consecutive n of a lane are the contiguous ones: 16 pieces of 4 again.
+    // Symmetric result: the same values also belong at C(n, m).
     if (args.symmetric && tile_m != tile_n) {
+        if (args.c_vec && m_valid >= BK_TILE_M && n_valid >= BK_TILE_N) {
+            // Through LDS (idle after the K walk, which ends with a barrier), a quarter of 32 rows m
+            // at a time and the two staging arrays in turn, so that every store instruction of a
+            // wave writes two whole 512-byte rows of the mirrored tile; written straight from the
+            // registers, where a lane's four consecutive n are the contiguous ones, an instruction
+            // covers 16 rows with 64 bytes each, and the mirrored half costs 2 of 16.5 ms.
+            static_assert(32 * BK_LDS_PITCH <= 2 * BK_LDS_SLICE + BK_LDS_PITCH, "a quarter fits one staging array");
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int m_local = tx * 4 + (i & 3) + (i >> 2) * 64;
-            if (m_local >= m_valid) continue;
+            for (int quarter = 0; quarter < 4; quarter++) {
+                float *stage = (quarter & 1) ? lds_b : lds_a;
+                // rows 32 quarter .. + 31 are held by the lanes with (tx >> 3) == (quarter & 1) in
+                // registers i = 4 (quarter >> 1) .. + 3
+                if ((tx >> 3) == (quarter & 1)) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int n_local = ty * 4 + h * 64;
-                float *dst = c_tile + (i64)(m0 + m_local) * args.c_ld + n0 + n_local;
-                if (args.c_vec && n_local + 3 < n_valid) {
-                    *reinterpret_cast<float4 *>(dst) =
-                        make_float4(acc[4 * h][i], acc[4 * h + 1][i], acc[4 * h + 2][i], acc[4 * h + 3][i]);
-                } else {
+                    for (int ii = 0; ii < 4; ii++) {
+                        const int i = (quarter >> 1) * 4 + ii;
+                        const int row = (tx & 7) * 4 + ii;
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        if (n_local + j < n_valid) dst[j] = acc[4 * h + j][i];
+                        for (int h = 0; h < 2; h++)
+                            *reinterpret_cast<float4 *>(stage + row * BK_LDS_PITCH + ty * 4 + h * 64) =
+                                make_float4(acc[4 * h][i], acc[4 * h + 1][i], acc[4 * h + 2][i], acc[4 * h + 3][i]);
+                    }
+                }
+                __syncthreads();
+#pragma unroll
+                for (int pass = 0; pass < 4; pass++) {
+                    const int row = pass * 8 + (tid >> 5);
+                    const int column = (tid & 31) * 4;
+                    const float4 v = *reinterpret_cast<const float4 *>(stage + row * BK_LDS_PITCH + column);
+                    *reinterpret_cast<float4 *>(c_tile + (i64)(m0 + quarter * 32 + row) * args.c_ld + n0 + column) = v;
+                }
+                // the next quarter uses the other array; the one after next waits at that quarter's barrier
+            }
+        } else {
+            // edge tiles and unaligned results: straight from the registers
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int m_local = tx * 4 + (i & 3) + (i >> 2) * 64;
+                if (m_local >= m_valid) continue;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int n_local = ty * 4 + h * 64;
+                    float *dst = c_tile + (i64)(m0 + m_local) * args.c_ld + n0 + n_local;
+                    if (args.c_vec && n_local + 3 < n_valid) {
+                        *reinterpret_cast<float4 *>(dst) =
+                            make_float4(acc[4 * h][i], acc[4 * h + 1][i], acc[4 * h + 2][i], acc[4 * h + 3][i]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            if (n_local + j < n_valid) dst[j] = acc[4 * h + j][i];
+                    }
                 }
             }
         }
