@@ -28,7 +28,7 @@ CASES = (
 
 @pytest.fixture
 def gram_mode():
-    kermac.set_l2_mode("gram")
+    kermac.set_l2_mode("gram", min_k=0)
     yield
     kermac.set_l2_mode("direct")
 
@@ -82,7 +82,7 @@ def test_distrusted_tiles_take_the_direct_arithmetic(device):
     coef = torch.randn(400, 20, generator=g).to(device)
     kermac.set_l2_mode("direct")
     direct = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, z, bandwidth=3.0, coefficients=coef)
-    kermac.set_l2_mode("gram")
+    kermac.set_l2_mode("gram", min_k=0)
     try:
         gram = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, z, bandwidth=3.0, coefficients=coef)
     finally:
@@ -94,7 +94,7 @@ def test_distrusted_tiles_take_the_direct_arithmetic(device):
     # a mix: only the first 128 centres are near-duplicates of samples
     z2 = torch.randn(400, 32, generator=g).to(device) + 40.0
     z2[:100] = x[:100] + 1e-4
-    kermac.set_l2_mode("gram")
+    kermac.set_l2_mode("gram", min_k=0)
     try:
         mixed = kermac.run_kernel(GAUSSIAN, x, z2, bandwidth=4.0, coefficients=coef)
     finally:

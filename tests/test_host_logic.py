@@ -295,6 +295,9 @@ def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
         kermac.set_l2_mode("gram", trust=0.5)
         assert flags(kermac.kernel_descriptor_l2_norm)[1] == pytest.approx(0.5)
         assert flags(kermac.kernel_descriptor_l2_norm)[0] & _backend.FLAG_L2_GRAM_BF16 == 0
+        # short contractions stay on the direct kernel unless min_k says otherwise (K = 64 here)
+        kermac.set_l2_mode("gram", min_k=65)
+        assert flags(kermac.kernel_descriptor_l2_norm)[0] & _backend.FLAG_L2_GRAM == 0
         kermac.set_l2_mode("gram_bf16")
         f, trust = flags(kermac.kernel_descriptor_l2_norm)
         assert f & _backend.FLAG_L2_GRAM and f & _backend.FLAG_L2_GRAM_BF16 and trust == pytest.approx(0.25)

@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(params=["gram", "gram_bf16"])
 def gram_mode(request):
-    kermac.set_l2_mode(request.param)
+    kermac.set_l2_mode(request.param, min_k=0)      # also the short contractions, which would stay direct
     yield
     kermac.set_l2_mode("direct")
 
@@ -29,6 +29,8 @@ def test_mode_switch_validation():
         kermac.set_l2_mode("fast")
     with pytest.raises(ValueError):
         kermac.set_l2_mode("gram", trust=0.0)
+    with pytest.raises(ValueError):
+        kermac.set_l2_mode("gram", min_k=-1)
     assert kermac.get_l2_mode() == "direct"
 
 
@@ -124,7 +126,7 @@ def test_bf16_flag_alone_through_the_c_abi(device):
     plan.params.gram_trust = 0.25
     _backend.build_kernel(plan.params, torch.cuda.current_stream(device).cuda_stream)
     assert_close_to_truth(out, oracle.cdist(a.cpu(), b.cpu(), p=2.0), rtol=1e-5, what="bf16 flag alone")
-    kermac.set_l2_mode("gram_bf16")
+    kermac.set_l2_mode("gram_bf16", min_k=0)
     try:
         assert torch.equal(out, kermac.cdist(a, b, p=2.0))
     finally:

@@ -29,7 +29,7 @@ DESCRIPTORS = {
 
 @pytest.fixture(params=["direct", "gram", "gram_bf16"])
 def l2_mode(request):
-    kermac.set_l2_mode(request.param)
+    kermac.set_l2_mode(request.param, min_k=0)
     yield request.param
     kermac.set_l2_mode("direct")
 
