@@ -99,16 +99,24 @@ struct RowOwnerLoader {
     }
     // Load number `which` (0 .. LOADS - 1) of the current slice into r.  With EDGE, rows
     // >= rows_valid and k >= k_valid read as 0 (adds 0 to norms and dot products).
-    template <bool EDGE>
+    // QUADS (row-major operands with 128-bit loads, kernels built for a ragged K, where every
+    // tile comes through here): a predicated 128-bit load wherever all four k exist.
+    template <bool EDGE, bool QUADS = false>
     __device__ __forceinline__ void load_part(float (&r)[8], int which, int rows_valid, int k_valid) const
     {
         if (MODE == LOAD_ROW_VEC && !EDGE) {
             const gram_float4 v = *(global_quad_pointer)element(4 * which);
             r[4 * which] = v.x; r[4 * which + 1] = v.y; r[4 * which + 2] = v.z; r[4 * which + 3] = v.w;
         } else if (MODE == LOAD_ROW_VEC) {
+            if (QUADS && k_valid == BK_TILE_K) {      // uniform: every slice but the last of a ragged K
+                gram_float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (row < rows_valid) v = *(global_quad_pointer)element(4 * which);
+                r[4 * which] = v.x; r[4 * which + 1] = v.y; r[4 * which + 2] = v.z; r[4 * which + 3] = v.w;
+            } else {
 #pragma unroll
-            for (int e = 4 * which; e < 4 * which + 4; e++)
-                r[e] = (row < rows_valid && 8 * half + e < k_valid) ? *element(e) : 0.0f;
+                for (int e = 4 * which; e < 4 * which + 4; e++)
+                    r[e] = (row < rows_valid && 8 * half + e < k_valid) ? *element(e) : 0.0f;
+            }
         } else if (EDGE) {
             r[which] = (row < rows_valid && 8 * half + which < k_valid) ? *element(which) : 0.0f;
         } else {
@@ -132,7 +140,7 @@ struct GramStep {
     static constexpr int value = N;
 };
 
-template <int LOAD_A, int LOAD_B, bool FULL>
+template <int LOAD_A, int LOAD_B, bool FULL, bool QUADS = false>
 __device__ __forceinline__ void gram_bf16_walk(
     gram_float16 (&acc)[2][2], float &square_a, float &square_b, RowOwnerLoader<LOAD_A> &load_a,
     RowOwnerLoader<LOAD_B> &load_b, gram_chunk *lds_a, gram_chunk *lds_b, int k_total, int m_valid, int n_valid,
@@ -150,10 +158,10 @@ __device__ __forceinline__ void gram_bf16_walk(
             const int kv = slice + 1 == k_slices ? k_tail : BK_TILE_K;
 #pragma unroll
             for (int which = 0; which < RowOwnerLoader<LOAD_A>::LOADS; which++)
-                load_a.template load_part<!FULL>(stage[S][0], which, m_valid, kv);
+                load_a.template load_part<!FULL, QUADS>(stage[S][0], which, m_valid, kv);
 #pragma unroll
             for (int which = 0; which < RowOwnerLoader<LOAD_B>::LOADS; which++)
-                load_b.template load_part<!FULL>(stage[S][1], which, n_valid, kv);
+                load_b.template load_part<!FULL, QUADS>(stage[S][1], which, n_valid, kv);
             load_a.advance();
             load_b.advance();
         } else {
@@ -249,8 +257,14 @@ __device__ __forceinline__ void gram_bf16_walk(
     }
 }
 
-template <int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(BK_THREADS, GB_WAVES) void gram_bf16_l2_kernel(const BuildKernelArgs args)
+// RAGGED_K: built for K that is not a multiple of 16, where no tile can take the unpredicated
+// walk; instantiated for the loader pairs with 128-bit row-major loads, which otherwise fall
+// back to eight predicated scalar loads per slice (M = N = 16384, K = 1000: 6.8 -> 3.4 ms).
+// A kernel of its own because the two kinds of predicated loads side by side cost the
+// unpredicated walk of the same kernel 20 % (register allocation), and with a register
+// budget for two waves per SIMD: within the budget for three the compiler spills 180.
+template <int LOAD_A, int LOAD_B, bool RAGGED_K = false>
+__global__ __launch_bounds__(BK_THREADS, RAGGED_K ? 2 : GB_WAVES) void gram_bf16_l2_kernel(const BuildKernelArgs args)
 {
     __shared__ gram_chunk lds_a[2 * GB_PANEL_CHUNKS];
     __shared__ gram_chunk lds_b[2 * GB_PANEL_CHUNKS];
@@ -287,7 +301,10 @@ __global__ __launch_bounds__(BK_THREADS, GB_WAVES) void gram_bf16_l2_kernel(cons
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[mt][nt][v] = 0.0f;
 
-    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
+    if (RAGGED_K) {
+        gram_bf16_walk<LOAD_A, LOAD_B, false, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k,
+                                                    m_valid, n_valid, wave_m, wave_n, h, i);
+    } else if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
         gram_bf16_walk<LOAD_A, LOAD_B, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
                                              n_valid, wave_m, wave_n, h, i);
     } else {

@@ -1,5 +1,5 @@
 // Ahead-of-time instantiations of the split-bf16 matrix-core L2 kernel for all 16
-// (A loader, B loader) pairs.
+// (A loader, B loader) pairs, plus the ragged-K variants of the pairs with 128-bit row-major loads.
 #include <hip/hip_runtime.h>
 
 #include "gram_bf16_kernel.hpp"
@@ -9,7 +9,13 @@ namespace kmc_host {
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)
 {
-    hipLaunchKernelGGL((kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B>), grid, dim3(kmc::BK_THREADS), 0, stream, args);
+    constexpr bool has_ragged_variant = LOAD_A == kmc::LOAD_ROW_VEC || LOAD_B == kmc::LOAD_ROW_VEC;
+    if (has_ragged_variant && args.k % kmc::BK_TILE_K != 0) {
+        hipLaunchKernelGGL((kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B, has_ragged_variant>), grid, dim3(kmc::BK_THREADS), 0,
+                           stream, args);
+    } else {
+        hipLaunchKernelGGL((kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B>), grid, dim3(kmc::BK_THREADS), 0, stream, args);
+    }
     return hipGetLastError();
 }
 

@@ -35,7 +35,10 @@ def test_mode_switch_validation():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (128, 128, 16), (129, 127, 17), (300, 515, 70), (1000, 1000, 64),
-                                   (257, 64, 1024)])
+                                   (257, 64, 1024),
+                                   # K ragged but a multiple of 4: row-major operands keep their 128-bit loads
+                                   # and take the kernels built for a ragged K
+                                   (260, 300, 100), (384, 130, 36), (128, 256, 20)])
 @pytest.mark.parametrize("layout", ["cc", "rr", "cr", "rc"])
 def test_random_data_matches_truth(device, gram_mode, M, N, K, layout):
     g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
