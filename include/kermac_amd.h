@@ -143,6 +143,21 @@ typedef struct kmc_build_kernel_params {
 int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream);
 
 /*
+ * Second step of a contraction that the caller cut over k (no counterpart in the
+ * reference, whose kernel walks all of k in one workgroup per tile: a 100 x 100
+ * result over k = 100000 is a single workgroup there and here).  The caller launches
+ * kmc_build_kernel on `slices` ranges of k with outer_power = KMC_POW_NOOP and
+ * kernel_type = KMC_KERNEL_NONE into partial results
+ *   partials[m + n*partial_ld + l*partial_bs + s*partial_slice]
+ * (a batched launch over strided views does all slices at once); this entry point
+ * adds the partial results in slice order and applies outer power, epsilon mask,
+ * kernel function and regularised diagonal of `params` exactly like
+ * kmc_build_kernel, writing C.  `a`, `b` and `k` of `params` are not read.
+ */
+int kmc_build_kernel_finish(const kmc_build_kernel_params *params, const float *partials, int64_t partial_ld,
+                            int64_t partial_bs, int64_t partial_slice, int32_t slices, void *stream);
+
+/*
  * Arguments of the fused kernel-gradient contraction; mirrors the 24 launch
  * arguments of cute_norm_kernel_gradient (include/p_norm_gradient.cuh:413-422,
  * marshalled at src/kermac/cdist_grad.py:226-235).

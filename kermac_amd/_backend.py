@@ -90,6 +90,8 @@ SIGNATURES = {
     "kmc_build_kernel_has_variant": (ctypes.c_int, [c_int32, c_int32]),
     "kmc_build_kernel": (ctypes.c_int, [POINTER(BuildKernelParams), c_void_p]),
     "kmc_build_kernel_jit": (ctypes.c_int, [c_void_p, POINTER(BuildKernelParams), c_void_p]),
+    "kmc_build_kernel_finish": (ctypes.c_int, [POINTER(BuildKernelParams), c_void_p, c_int64, c_int64, c_int64, c_int32,
+                                               c_void_p]),
     "kmc_build_kernel_load_modes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int32), POINTER(c_int32)]),
     "kmc_norm_kernel_gradient": (ctypes.c_int, [POINTER(NormGradientParams), c_void_p]),
     "kmc_kernel_times_coefficients": (ctypes.c_int, [POINTER(KernelCoefficientsParams), c_void_p]),
@@ -163,6 +165,12 @@ def check(status: int) -> None:
 
 def build_kernel(params: BuildKernelParams, stream: int) -> None:
     check(library().kmc_build_kernel(byref(params), c_void_p(stream)))
+
+
+def build_kernel_finish(params: BuildKernelParams, partials: int, partial_ld: int, partial_bs: int, partial_slice: int,
+                        slices: int, stream: int) -> None:
+    check(library().kmc_build_kernel_finish(byref(params), c_void_p(partials), partial_ld, partial_bs, partial_slice,
+                                            slices, c_void_p(stream)))
 
 
 def build_kernel_jit(function: int, params: BuildKernelParams, stream: int) -> None:

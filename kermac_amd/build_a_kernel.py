@@ -449,16 +449,77 @@ def run_kernel(
         regularization_offset_x, regularization_offset_y, try_to_align)
     stream = _current_stream_for(a.device)
     params = plan.params
-    with torch.cuda.device(a.device):
-        if _backend.build_kernel_has_variant(params.inner_operator, params.inner_power):
+
+    def launch(block):
+        if _backend.build_kernel_has_variant(block.inner_operator, block.inner_power):
             if debug:
                 print(f"(Kermac Debug) Launching ahead-of-time kernel for {kernel_descriptor!r}")
-            _backend.build_kernel(params, stream)
+            _backend.build_kernel(block, stream)
         else:
-            load_a, load_b = _backend.build_kernel_load_modes(params)
-            function_name = build_kernel_function_name(params.inner_operator, params.inner_power, load_a, load_b)
+            load_a, load_b = _backend.build_kernel_load_modes(block)
+            function_name = build_kernel_function_name(block.inner_operator, block.inner_power, load_a, load_b)
             function = ModuleCache(debug).get_function(a.device, function_name, debug=debug)
             if debug:
                 print(f"(Kermac Debug) Launching kernel: {function_name}")
-            _backend.build_kernel_jit(function, params, stream)
+            _backend.build_kernel_jit(function, block, stream)
+
+    with torch.cuda.device(a.device):
+        cut = _cut_over_contraction(params)
+        if cut is None:
+            launch(params)
+        else:
+            _run_cut_over_contraction(cut, params, launch, stream, a.device)
     return plan.out
+
+
+# A workgroup owns one 128 x 128 tile of the result and walks the whole contraction index, so
+# a small result over a long contraction (100 x 100 over k = 100000 is one tile) leaves the
+# chip idle.  Such an unbatched call is cut over k: ranges of k become the batch of one launch
+# that stores plain sums (no outer power, no kernel function) into a buffer, and a second,
+# element-wise kernel adds the partial sums in slice order and applies the epilogue.
+_CUT_BELOW_TILES = 385          # up to 384 tiles two slices still fit the target
+_CUT_TARGET_TILES = 768
+_CUT_MIN_DEPTH = 256
+
+
+def _cut_over_contraction(params):
+    """(slices, k per slice, leftover k), or None when the launch goes out as it is."""
+    if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
+        return None
+    tiles = -(-params.m // 128) * -(-params.n // 128)
+    if tiles == 0 or tiles >= _CUT_BELOW_TILES or params.k < 2 * _CUT_MIN_DEPTH:
+        return None
+    slices = min(_CUT_TARGET_TILES // tiles, params.k // _CUT_MIN_DEPTH)
+    if slices < 2:
+        return None
+    depth = params.k // slices // 16 * 16        # whole K slices of the kernel; 16-byte alignment survives
+    slices = params.k // depth
+    return slices, depth, params.k - slices * depth
+
+
+def _run_cut_over_contraction(cut, params, launch, stream, device):
+    slices, depth, leftover = cut
+    count = slices + (1 if leftover else 0)
+    ld = -(-params.m // 4) * 4
+    plane = ld * params.n
+    partial = torch.empty(count * plane, dtype=torch.float32, device=device)
+
+    def k_stride(majorness, leading):
+        return leading if majorness == _backend.COL_MAJOR else 1
+
+    step_a = depth * k_stride(params.a_majorness, params.a_ld)
+    step_b = depth * k_stride(params.b_majorness, params.b_ld)
+    first = _backend.BuildKernelParams.from_buffer_copy(params)
+    first.outer_power, first.kernel_type = _POWER_TYPE_ABI[PowerType.NOOP], _KERNEL_TYPE_ABI[KernelType.NONE]
+    first.k, first.l = depth, slices
+    first.a_bs, first.b_bs = step_a, step_b
+    first.c, first.c_ld, first.c_bs = partial.data_ptr(), ld, plane
+    launch(first)
+    if leftover:
+        last = _backend.BuildKernelParams.from_buffer_copy(first)
+        last.k, last.l = leftover, 1
+        last.a = params.a + 4 * slices * step_a
+        last.b = params.b + 4 * slices * step_b
+        last.c = partial.data_ptr() + 4 * slices * plane
+        launch(last)
+    _backend.build_kernel_finish(params, partial.data_ptr(), ld, 0, plane, count, stream)

@@ -114,6 +114,8 @@ kmc_host::build_launcher_fn find_launcher(int inner_operator, int inner_power)
 namespace kmc_host {
 hipError_t launch_gram_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
 hipError_t launch_gram_bf16_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
+hipError_t launch_finish_partials(const kmc::BuildKernelArgs &kernel, const float *partials, int64_t partial_ld,
+                                  int64_t partial_bs, int64_t partial_slice, int slices, int vec, hipStream_t stream);
 }
 
 namespace kmc_host {
@@ -179,6 +181,30 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
     }
     hipError_t e = launch(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail_hip(e, "build_kernel launch");
+    return KMC_OK;
+}
+
+int kmc_build_kernel_finish(const kmc_build_kernel_params *params, const float *partials, int64_t partial_ld,
+                            int64_t partial_bs, int64_t partial_slice, int32_t slices, void *stream)
+{
+    kmc::BuildKernelArgs args;
+    int load_a = 0, load_b = 0;
+    int status = prepare(params, true, &args, &load_a, &load_b);
+    if (status != KMC_OK) return status;
+    if (slices < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "negative slice count %d", slices);
+    if (args.m == 0 || args.n == 0 || args.l == 0) return KMC_OK;
+    if (slices > 0 && !partials) return fail(KMC_ERR_INVALID_ARGUMENT, "partials: null pointer");
+    if (partial_ld < args.m && args.n > 1)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "partials: leading dimension %lld is smaller than m=%d",
+                    static_cast<long long>(partial_ld), args.m);
+    if (partial_ld < 0 || partial_bs < 0 || partial_slice < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "partials: negative stride");
+    if (args.n > 65535 || args.l > 65535) return fail(KMC_ERR_INVALID_ARGUMENT, "n=%d or l=%d exceeds 65535", args.n, args.l);
+    status = require_gfx950();
+    if (status != KMC_OK) return status;
+    const int vec = args.c_vec && aligned16(partials) && partial_ld % 4 == 0 && partial_bs % 4 == 0 && partial_slice % 4 == 0;
+    hipError_t e = launch_finish_partials(args, partials, partial_ld, partial_bs, partial_slice, slices, vec,
+                                          static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail_hip(e, "finish_partials launch");
     return KMC_OK;
 }
 

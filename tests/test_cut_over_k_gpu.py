@@ -1,0 +1,83 @@
+"""GPU tests of run_kernel / cdist calls with a small result over a long contraction, which the
+Python layer cuts over k: one batched launch of plain partial sums plus the element-wise kernel
+behind kmc_build_kernel_finish, which adds them and applies the epilogue."""
+import pytest
+import torch
+
+import kermac_amd as kermac
+from kermac_amd import build_a_kernel as module
+from oracle import oracle
+from tests.helpers import assert_close_to_truth, make_operand
+
+pytestmark = pytest.mark.gpu
+
+
+def is_cut(descriptor, a, b, out=None, **kw):
+    plan = module._plan_run_kernel(descriptor, a, b, out, kw.get("p"), None, None, kw.get("bandwidth"), None,
+                                   kw.get("regularization"), 0, 0, False)
+    return module._cut_over_contraction(plan.params) is not None
+
+
+@pytest.mark.parametrize("p", [1.0, 2.0, 1.3])
+@pytest.mark.parametrize("M,N,K,layout", [(100, 90, 5000, "cc"), (300, 17, 2049, "rr"), (64, 130, 4096, "cr"),
+                                          (1, 1, 1000, "rc")])
+def test_cdist_small_result_long_contraction(device, p, M, N, K, layout):
+    g = torch.Generator().manual_seed(M + N + K)
+    a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False)
+    b = make_operand(1, N, K, layout[1] == "c", device, g, batch=False)
+    assert is_cut(kermac.kernel_descriptor_p_norm if p == 1.3 else kermac.kernel_descriptor_l1_norm, a, b, p=p if p == 1.3 else None)
+    truth = oracle.cdist(a.cpu(), b.cpu(), p=p)
+    for c_col in (False, True):
+        out = torch.full((N, M + 4), -7.0, device=device).t()[:M] if c_col else torch.full((M, N + 4), -7.0, device=device)[:, :N]
+        got = kermac.cdist(a, b, out=out, p=p)
+        assert got is out
+        assert_close_to_truth(got, truth[0], rtol=1e-5 if p != 1.3 else 1e-4, what=f"cut over k p={p} {layout} col={c_col}")
+        padding = out.t().untyped_storage() if False else None     # noqa: F841 (kept simple: padding checked below)
+    wide = torch.full((M, N + 4), -7.0, device=device)
+    kermac.cdist(a, b, out=wide[:, :N], p=p)
+    assert torch.all(wide[:, N:] == -7.0), "the padding of a strided out was written"
+    skipped = kermac.cdist(a, b, p=p, skip_epilogue=True)
+    assert_close_to_truth(skipped, oracle.cdist(a.cpu(), b.cpu(), p=p, skip_epilogue=True), rtol=2e-5 if p != 1.3 else 2e-4,
+                          what="cut over k, skip_epilogue")
+
+
+def test_kernels_regularised_diagonal_and_the_symmetric_shortcut(device):
+    g = torch.Generator().manual_seed(31)
+    x = torch.rand(257, 3000, generator=g).to(device)
+    assert is_cut(kermac.kernel_descriptor_laplace_l1, x, x, bandwidth=40.0, regularization=0.25)
+    got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, x, bandwidth=40.0, regularization=0.25,
+                            regularization_offset_x=3, regularization_offset_y=0)
+    truth = oracle.build_kernel("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu(), x.cpu(), bandwidth=40.0, regularization=0.25,
+                                regularization_offset_x=3, regularization_offset_y=0)
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-9, what="cut laplace with offset diagonal")
+    plain = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, x, bandwidth=torch.tensor([7.0], device=device),
+                              regularization=1e-3)
+    assert torch.equal(plain, plain.transpose(1, 2))
+    assert torch.all(torch.diagonal(plain[0]) == 1.0 + 1e-3)
+    truth = oracle.build_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", x.cpu(), x.cpu(), bandwidth=7.0, regularization=1e-3)
+    assert_close_to_truth(plain, truth, rtol=1e-5, atol=1e-9, what="cut laplace l2, symmetric")
+
+
+def test_dot_products_and_a_run_time_compiled_descriptor(device, tmp_path, monkeypatch):
+    monkeypatch.setenv("KERMAC_AMD_CACHE_DIR", str(tmp_path))
+    g = torch.Generator().manual_seed(32)
+    a = torch.rand(120, 2600, generator=g).to(device)
+    b = torch.rand(77, 2600, generator=g).to(device)
+    got = kermac.run_kernel(kermac.kernel_descriptor_mma, a, b)
+    assert_close_to_truth(got[0], a.double().cpu() @ b.double().cpu().t(), rtol=1e-5, what="cut dot")
+    odd = kermac.KernelDescriptor(kermac.InnerOperator.DOT, kermac.PowerType.SQRT, kermac.PowerType.SQUARE,
+                                  kermac.KernelType.NONE)
+    assert is_cut(odd, a, b)
+    got = kermac.run_kernel(odd, a, b)
+    truth = torch.sqrt(a.double().cpu()[:, None, :] * b.double().cpu()[None, :, :]).sum(-1) ** 2
+    assert_close_to_truth(got[0], truth, rtol=2e-5, what="cut, run-time compiled")
+
+
+def test_batched_and_large_results_are_not_cut(device):
+    a = torch.rand(3, 100, 3000, device=device)
+    b = torch.rand(3, 90, 3000, device=device)
+    assert not is_cut(kermac.kernel_descriptor_l1_norm, a, b)
+    a = torch.rand(3000, 600, device=device)
+    assert not is_cut(kermac.kernel_descriptor_l1_norm, a, a)          # 576 tiles: the chip is full
+    a = torch.rand(100, 400, device=device)
+    assert not is_cut(kermac.kernel_descriptor_l1_norm, a, a)          # contraction too short
