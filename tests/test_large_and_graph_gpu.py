@@ -200,11 +200,20 @@ def test_cut_launches_replay_from_a_hip_graph(device):
     assert grad_module._split_over_contraction(
         grad_module._plan_cdist_grad(weights, centres, classes, samples, None, 1.0)) is not None
 
+    long_a = torch.rand(150, 3000, generator=g).to(device)      # a small distance matrix over a long contraction
+    long_b = torch.rand(90, 3000, generator=g).to(device)
+    out_long = torch.empty(150, 90, device=device)
+    from kermac_amd import build_a_kernel as kernel_module
+    assert kernel_module._cut_over_contraction(
+        kernel_module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, long_a, long_b, out_long, None, None, None, None,
+                                       None, None, 0, 0, False).params) is not None
+
     def run_all():
         kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, z, out=out_fused, bandwidth=2.0, coefficients=coef)
         kermac.cdist_grad(weights, centres, classes, samples, out=out_grad, p=1.0)
+        kermac.cdist(long_a, long_b, out=out_long, p=2.0)
 
-    outs = (out_fused, out_grad)
+    outs = (out_fused, out_grad, out_long)
     side = torch.cuda.Stream(device=device)
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -217,6 +226,7 @@ def test_cut_launches_replay_from_a_hip_graph(device):
     for replay in range(4):
         x.copy_(torch.rand(M, K, generator=g))                  # new values, same addresses
         samples.mul_(1.25)
+        long_a.mul_(0.9)
         run_all()
         torch.cuda.synchronize()
         eager = [o.clone() for o in outs]
@@ -226,7 +236,7 @@ def test_cut_launches_replay_from_a_hip_graph(device):
         graph.replay()
         torch.cuda.synchronize()
         del scratch
-        for name, e, o in zip(("fused", "grad"), eager, outs):
+        for name, e, o in zip(("fused", "grad", "long contraction"), eager, outs):
             assert torch.equal(e, o), f"replay {replay}: {name} differs from the eager result"
     truth = oracle.kernel_times_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu(), z.cpu(), coef.cpu(), bandwidth=2.0)
     assert_close_to_truth(out_fused, truth, rtol=1e-5, atol=1e-5 * truth.abs().max().item(), what="cut fused replay")
