@@ -46,9 +46,10 @@ __device__ __forceinline__ float gradient_weight(float diff, float p_minus_1)
 {
     // include/p_norm_gradient.cuh:377-387
     if (NORM == NORM_L2) return diff;
-    const float sign = signum(diff);
-    if (NORM == NORM_L1) return sign;
-    return fast_pow_abs(__builtin_fabsf(diff), p_minus_1) * sign;
+    if (NORM == NORM_L1) return signum(diff);
+    // |diff|^(p-1) is never negative, so multiplying by copysign(1, diff) is a sign transfer:
+    // one instruction instead of two
+    return __builtin_copysignf(fast_pow_abs(__builtin_fabsf(diff), p_minus_1), diff);
 }
 
 // For the L1 norm only the sign of d - b is needed, and copysign(1, d - b) is
