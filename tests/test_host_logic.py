@@ -416,6 +416,21 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     grad.norm_type = 9
     with pytest.raises(_backend.BackendError):
         _backend.norm_kernel_gradient(grad, 0)
+    # the finishing step of a contraction cut over k: host pointers are never dereferenced, so
+    # fake non-null addresses are enough to reach the checks of the partial-sum arguments
+    fake = 4096
+    params = _backend.BuildKernelParams()
+    params.inner_power = 1
+    params.m = params.n = params.k = 8
+    params.l = 1
+    params.a = params.b = params.c = fake
+    params.a_ld = params.b_ld = params.c_ld = 8
+    for partials, ld, slices, word in ((0, 8, 3, "null"), (fake, 4, 3, "leading dimension"), (fake, 8, -1, "slice count")):
+        with pytest.raises(_backend.BackendError) as info:
+            _backend.build_kernel_finish(params, partials, ld, 0, 64, slices, 0)
+        assert info.value.status == _backend.ERR_INVALID_ARGUMENT and word in str(info.value), str(info.value)
+    params.m = 0
+    _backend.build_kernel_finish(params, 0, 0, 0, 0, 0, 0)      # empty result: accepted, nothing launched
     # a device that is not a gfx950 is a ValueError, as an unsupported compute capability is in
     # the reference (src/kermac/module_cache/module_cache.py:166-167), and still a BackendError
     with pytest.raises(ValueError) as info:
