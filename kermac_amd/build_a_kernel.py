@@ -394,11 +394,20 @@ def _plan_run_kernel(
     return plan
 
 
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _current_stream_for(device: torch.device) -> int:
-    stream = torch.cuda.current_stream()
-    if stream.device != device:
-        raise ValueError(f"cuda stream must be on the same device as the tensors: got {stream.device}, expected {device}")
-    return PyTorchStreamWrapper(stream).handle
+    """The hipStream_t of torch's current stream, which must be on the tensors' device
+    (reference: build_a_kernel.py:314-321).  The raw-handle accessor saves the construction of
+    a Stream object on every call; a launch costs about 10 microseconds of host time."""
+    current = torch.cuda.current_device()
+    index = current if device.index is None else device.index
+    if current != index:
+        raise ValueError(f"cuda stream must be on the same device as the tensors: got cuda:{current}, expected {device}")
+    if _raw_current_stream is not None:
+        return _raw_current_stream(index)
+    return PyTorchStreamWrapper(torch.cuda.current_stream()).handle
 
 
 def run_kernel(
@@ -463,12 +472,11 @@ def run_kernel(
                 print(f"(Kermac Debug) Launching kernel: {function_name}")
             _backend.build_kernel_jit(function, block, stream)
 
-    with torch.cuda.device(a.device):
-        cut = _cut_over_contraction(params)
-        if cut is None:
-            launch(params)
-        else:
-            _run_cut_over_contraction(cut, params, launch, stream, a.device)
+    cut = _cut_over_contraction(params)
+    if cut is None:
+        launch(params)
+    else:
+        _run_cut_over_contraction(cut, params, launch, stream, a.device)
     return plan.out
 
 

@@ -162,8 +162,7 @@ def cdist_grad(
     stream = _current_stream_for(a.device)
     if debug:
         print(f"(Kermac Debug) Launching kernel: norm_kernel_gradient<{('L1', 'L2', 'P')[plan.params.norm_type]}>")
-    with torch.cuda.device(a.device):
-        _backend.norm_kernel_gradient(plan.params, stream)
+    _backend.norm_kernel_gradient(plan.params, stream)
     return plan.out
 
 

@@ -117,18 +117,17 @@ def run_kernel_coefficients(
     stream = _current_stream_for(a.device)
     params = plan.params
     kernel = params.kernel
-    with torch.cuda.device(a.device):
-        if _backend.kernel_times_coefficients_has_variant(kernel.inner_operator, kernel.inner_power):
-            if debug:
-                print(f"(Kermac Debug) Launching ahead-of-time fused coefficient kernel for {kernel_descriptor!r}")
-            _backend.kernel_times_coefficients(params, stream)
-        else:
-            load_a, load_b = _backend.build_kernel_load_modes(kernel)
-            name = kernel_coefficients_function_name(kernel.inner_operator, kernel.inner_power, load_a, load_b)
-            function = ModuleCache(debug).get_function(a.device, name, debug=debug)
-            if debug:
-                print(f"(Kermac Debug) Launching kernel: {name}")
-            _backend.kernel_times_coefficients_jit(function, params, stream)
+    if _backend.kernel_times_coefficients_has_variant(kernel.inner_operator, kernel.inner_power):
+        if debug:
+            print(f"(Kermac Debug) Launching ahead-of-time fused coefficient kernel for {kernel_descriptor!r}")
+        _backend.kernel_times_coefficients(params, stream)
+    else:
+        load_a, load_b = _backend.build_kernel_load_modes(kernel)
+        name = kernel_coefficients_function_name(kernel.inner_operator, kernel.inner_power, load_a, load_b)
+        function = ModuleCache(debug).get_function(a.device, name, debug=debug)
+        if debug:
+            print(f"(Kermac Debug) Launching kernel: {name}")
+        _backend.kernel_times_coefficients_jit(function, params, stream)
     return plan.out
 
 
