@@ -485,9 +485,11 @@ def run_kernel(
 # chip idle.  Such an unbatched call is cut over k: ranges of k become the batch of one launch
 # that stores plain sums (no outer power, no kernel function) into a buffer, and a second,
 # element-wise kernel adds the partial sums in slice order and applies the epilogue.
-_CUT_BELOW_TILES = 385          # up to 384 tiles two slices still fit the target
-_CUT_TARGET_TILES = 768
-_CUT_MIN_DEPTH = 256
+_CUT_BELOW_TILES = 385          # up to 384 tiles two slices still fit one round
+_CUT_CONCURRENT_TILES = 768     # three workgroups per CU
+_CUT_MIN_DEPTH = 128
+_CUT_WORKGROUP_OVERHEAD = 128   # start-up, first loads and stores of a workgroup, in k walked
+_CUT_WORTH = 0.8                # cut only for at least 20 % less modelled time
 
 
 def _cut_over_contraction(params):
@@ -495,14 +497,33 @@ def _cut_over_contraction(params):
     if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
         return None
     tiles = -(-params.m // 128) * -(-params.n // 128)
-    if tiles == 0 or tiles >= _CUT_BELOW_TILES or params.k < 2 * _CUT_MIN_DEPTH:
+    K = params.k
+    if tiles == 0 or tiles >= _CUT_BELOW_TILES or K < 4 * _CUT_MIN_DEPTH:
         return None
-    slices = min(_CUT_TARGET_TILES // tiles, params.k // _CUT_MIN_DEPTH)
-    if slices < 2:
+
+    def rounds(count):
+        return -(-count // _CUT_CONCURRENT_TILES)
+
+    # Modelled time of a launch: k walked per workgroup (plus its fixed cost) times rounds of
+    # workgroups; a leftover range of k is a second launch.  Depths are whole K slices of the
+    # kernel (16), so 16-byte alignment survives; a few depths from the one that fills one round
+    # upwards are tried, which finds the cuts without (or with a small) leftover.
+    unsplit = (K + _CUT_WORKGROUP_OVERHEAD) * rounds(tiles)
+    first = max(_CUT_MIN_DEPTH, -(-K * tiles // _CUT_CONCURRENT_TILES // 16) * 16)
+    best = None
+    for depth in range(first, first + 16 * 24, 16):
+        slices = K // depth
+        if slices < 2:
+            break
+        leftover = K - slices * depth
+        cost = (depth + _CUT_WORKGROUP_OVERHEAD) * rounds(slices * tiles)
+        if leftover:
+            cost += (leftover + 2 * _CUT_WORKGROUP_OVERHEAD) * rounds(tiles)
+        if best is None or cost < best[0]:
+            best = (cost, slices, depth, leftover)
+    if best is None or best[0] > _CUT_WORTH * unsplit:
         return None
-    depth = params.k // slices // 16 * 16        # whole K slices of the kernel; 16-byte alignment survives
-    slices = params.k // depth
-    return slices, depth, params.k - slices * depth
+    return best[1:]
 
 
 def _run_cut_over_contraction(cut, params, launch, stream, device):
