@@ -62,7 +62,15 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
     }
     const int64_t tiles_m = ceil_div(p->m, kmc::BK_TILE_M);
     const int64_t tiles_n = ceil_div(p->n, kmc::BK_TILE_N);
-    const int64_t tiles_n_padded = (tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
+    // Rounding the n tiles up to a multiple of 8 keeps every n tile on one XCD (see
+    // tile_of_workgroup).  The padding workgroups exit at once but still take their turn
+    // in the dispatch order, so the rounding is dropped where it would add more than one
+    // workgroup in eight: those problems are small enough for every L2 to hold the panels.
+    // (Measured: 16 tiles padded to 32 per batch entry, as a batch of 32, left half the CUs
+    // idle: 0.255 ms against 0.167 ms without the padding; 1000 problems of one tile each,
+    // padded to 8: 0.283 against 0.099 ms.)
+    int64_t tiles_n_padded = (tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
+    if ((tiles_n_padded - tiles_n) * 8 > tiles_n) tiles_n_padded = tiles_n;
     if (tiles_m * tiles_n_padded > INT_MAX) return fail(KMC_ERR_INVALID_ARGUMENT, "m x n needs more than 2^31 tiles");
 
     args->m = p->m; args->n = p->n; args->k = p->k; args->l = p->l;

@@ -43,7 +43,7 @@ struct BuildKernelArgs {
     int outer_power, kernel_type;
     int c_vec;     // c, c_ld and c_bs are multiples of 16 bytes: 128-bit stores allowed
     int tiles_m, tiles_n;
-    int tiles_n_padded;  // tiles_n rounded up to a multiple of 8; grid.x = tiles_m * tiles_n_padded
+    int tiles_n_padded;  // tiles_n, rounded up to a multiple of 8 where that adds little; grid.x = tiles_m * tiles_n_padded
     int repair_only;     // recompute only the tiles that carry BK_REPAIR_MARKER (see gram_kernel.hpp)
     int symmetric;       // A and B are the same panel and the result is symmetric: only tiles with
                          // tile_m >= tile_n are computed, each is also stored mirrored
@@ -419,13 +419,14 @@ __device__ __forceinline__ void finish_tile(
 // tiles and share their A and B panels through that XCD's L2, while ids are
 // still handed out in one global order (no XCD can run dry early).  Band
 // heights are rounded up to a multiple of 8 to keep that ownership in the last
-// band; the padding workgroups get `false` and exit at once.
+// band; the padding workgroups get `false` and exit at once.  The host drops the
+// rounding for problems of few n tiles, where it would add many such workgroups.
 __device__ __forceinline__ bool tile_of_workgroup(const BuildKernelArgs &args, int &tile_m, int &tile_n)
 {
     // Batches rotate the order by one: the hardware derives the XCD from the launch-wide
-    // workgroup id, which is blockIdx.x modulo 8 for every batch (the grid width is a
-    // multiple of 8), so without the rotation a batch of problems of one tile each would
-    // run on a single XCD.  The residue classes modulo 8, and with them the ownership
+    // workgroup id, which is blockIdx.x modulo 8 for every batch when the grid width is a
+    // multiple of 8, so without the rotation a batch of problems of 8 tiles each would
+    // run every tile n on a single XCD.  The residue classes modulo 8, and with them the ownership
     // described above, survive the rotation.
     const int rotated = blockIdx.x + blockIdx.y % gridDim.x;
     const int linear = rotated >= (int)gridDim.x ? rotated - (int)gridDim.x : rotated;
