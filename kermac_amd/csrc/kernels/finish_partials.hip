@@ -2,7 +2,10 @@
 // are added in slice order and the result goes through the epilogue of the fused
 // pairwise-reduction kernel (outer power, epsilon mask, kernel function, regularised
 // diagonal: include/build_a_kernel.cuh:374-447 of the reference).  Element-wise, one
-// lane per four consecutive m.
+// lane per four consecutive m; where one row of the result has fewer than 128 such
+// lanes, the lanes of a workgroup also divide the slices among themselves (lane group g
+// adds slices g, g + G, g + 2 G, ... in that order, then group 0 adds the groups' sums in
+// group order: a fixed order for a given shape, so results repeat bit for bit).
 #include <hip/hip_runtime.h>
 
 #include "build_kernel.hpp"
@@ -15,34 +18,55 @@ struct FinishArgs {
     i64 partial_ld, partial_bs, partial_slice;
     int slices;
     int vec;                    // partials and c allow 128-bit access
+    int quad_lanes;             // lanes along m per workgroup: 256 / groups, a power of two
+    int groups;                 // lane groups that share the slices of one quad of m
 };
 
 __global__ __launch_bounds__(256) void finish_partials(const FinishArgs fa)
 {
     const BuildKernelArgs &args = fa.kernel;
+    __shared__ float4 group_sums[256];
     const int batch = blockIdx.z;
     const int n = blockIdx.y;
-    const int m = (blockIdx.x * 256 + threadIdx.x) * 4;
-    if (m >= args.m) return;
-    const int valid = min(4, args.m - m);
+    const int quad = threadIdx.x & (fa.quad_lanes - 1);
+    const int group = threadIdx.x / fa.quad_lanes;
+    const int m = (blockIdx.x * fa.quad_lanes + quad) * 4;
+    const bool live = m < args.m;
+    const int valid = live ? min(4, args.m - m) : 0;
 
     float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const float *src = fa.partials + batch * fa.partial_bs + (i64)n * fa.partial_ld + m;
-    // Eight loads in flight, added in slice order (the order of the sum is fixed).
-    int s = 0;
-    for (; s + 8 <= fa.slices; s += 8) {
-        float4 v[8];
+    if (live) {
+        // Eight loads in flight, added in slice order (the order of the sum is fixed).
+        const i64 step = fa.groups * fa.partial_slice;
+        const float *at = src + group * fa.partial_slice;
+        const int mine = (fa.slices - group + fa.groups - 1) / fa.groups;   // slices group, group + G, ...
+        int s = 0;
+        for (; s + 8 <= mine; s += 8) {
+            float4 v[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = load4_guarded(src + (s + u) * fa.partial_slice, valid, fa.vec);
+            for (int u = 0; u < 8; u++) v[u] = load4_guarded(at + (s + u) * step, valid, fa.vec);
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            sum[0] += v[u].x; sum[1] += v[u].y; sum[2] += v[u].z; sum[3] += v[u].w;
+            for (int u = 0; u < 8; u++) {
+                sum[0] += v[u].x; sum[1] += v[u].y; sum[2] += v[u].z; sum[3] += v[u].w;
+            }
+        }
+        for (; s < mine; s++) {
+            const float4 v = load4_guarded(at + s * step, valid, fa.vec);
+            sum[0] += v.x; sum[1] += v.y; sum[2] += v.z; sum[3] += v.w;
         }
     }
-    for (; s < fa.slices; s++) {
-        const float4 v = load4_guarded(src + s * fa.partial_slice, valid, fa.vec);
-        sum[0] += v.x; sum[1] += v.y; sum[2] += v.z; sum[3] += v.w;
+    if (fa.groups > 1) {   // uniform over the launch
+        group_sums[threadIdx.x] = make_float4(sum[0], sum[1], sum[2], sum[3]);
+        __syncthreads();
+        if (group == 0) {
+            for (int g = 1; g < fa.groups; g++) {
+                const float4 v = group_sums[g * fa.quad_lanes + quad];
+                sum[0] += v.x; sum[1] += v.y; sum[2] += v.z; sum[3] += v.w;
+            }
+        }
     }
+    if (!live || group != 0) return;
 
     const int outer_power = args.outer_power;
     const int kernel_type = args.kernel_type;
@@ -84,7 +108,12 @@ hipError_t launch_finish_partials(const kmc::BuildKernelArgs &kernel, const floa
     fa.partial_ld = partial_ld; fa.partial_bs = partial_bs; fa.partial_slice = partial_slice;
     fa.slices = slices;
     fa.vec = vec;
-    const dim3 grid((kernel.m + 1023) / 1024, kernel.n, kernel.l);
+    // A row of fewer than 128 quads of m leaves lanes for sharing the slices (at least 8 each).
+    const int quads = (kernel.m + 3) / 4;
+    fa.quad_lanes = 256;
+    while (fa.quad_lanes > 1 && fa.quad_lanes / 2 >= quads && slices >= 8 * (512 / fa.quad_lanes)) fa.quad_lanes /= 2;
+    fa.groups = 256 / fa.quad_lanes;
+    const dim3 grid((quads + fa.quad_lanes - 1) / fa.quad_lanes, kernel.n, kernel.l);
     hipLaunchKernelGGL(kmc::finish_partials, grid, dim3(256), 0, stream, fa);
     return hipGetLastError();
 }

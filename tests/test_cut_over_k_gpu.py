@@ -81,3 +81,35 @@ def test_batched_and_large_results_are_not_cut(device):
     assert not is_cut(kermac.kernel_descriptor_l1_norm, a, a)          # 576 tiles: the chip is full
     a = torch.rand(100, 400, device=device)
     assert not is_cut(kermac.kernel_descriptor_l1_norm, a, a)          # contraction too short
+
+
+@pytest.mark.parametrize("m,n,slices", [(1, 3, 5000), (5, 7, 300), (100, 100, 768), (130, 4, 100), (511, 2, 17),
+                                        (600, 3, 9), (1030, 2, 40), (64, 5, 15), (64, 5, 16)])
+def test_finish_entry_point_adds_slices_and_applies_the_epilogue(device, m, n, slices):
+    """kmc_build_kernel_finish through the C ABI on its own: rows of few m share the slices among
+    lane groups, so every split of the lanes is compared with a float64 sum."""
+    from kermac_amd import _backend
+    g = torch.Generator().manual_seed(m * 31 + slices)
+    ld = (m + 3) // 4 * 4
+    partial = torch.zeros(slices, n, ld, device=device)
+    partial[:, :, :m] = torch.rand(slices, n, m, generator=g).to(device)
+    out = torch.full((n, ld), -3.0, device=device)
+    params = _backend.BuildKernelParams()
+    params.inner_operator = 0
+    params.inner_power = 2          # squared differences ...
+    params.outer_power = 3          # ... and their square root, as cdist(p=2) asks for
+    params.m, params.n, params.k, params.l = m, n, 8, 1
+    params.a = params.b = partial.data_ptr()       # checked for null only: the finishing step reads no operand
+    params.a_ld = params.b_ld = max(m, n, 8)
+    params.c, params.c_ld = out.data_ptr(), ld
+    stream = torch.cuda.current_stream(device).cuda_stream
+    _backend.build_kernel_finish(params, partial.data_ptr(), ld, 0, n * ld, slices, stream)
+    torch.cuda.synchronize()
+    truth = partial[:, :, :m].double().sum(0).sqrt()
+    assert_close_to_truth(out[:, :m], truth, rtol=1e-5, what=f"finish m={m} n={n} slices={slices}")
+    assert torch.all(out[:, m:] == -3.0), "columns past m were written"
+    again = torch.full((n, ld), -3.0, device=device)
+    params.c = again.data_ptr()
+    _backend.build_kernel_finish(params, partial.data_ptr(), ld, 0, n * ld, slices, stream)
+    torch.cuda.synchronize()
+    assert torch.equal(out, again), "the order of the sum is fixed: two runs agree bit for bit"
