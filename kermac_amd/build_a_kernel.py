@@ -490,6 +490,18 @@ _CUT_CONCURRENT_TILES = 768     # three workgroups per CU
 _CUT_MIN_DEPTH = 128
 _CUT_WORKGROUP_OVERHEAD = 128   # start-up, first loads and stores of a workgroup, in k walked
 _CUT_WORTH = 0.8                # cut only for at least 20 % less modelled time
+# From 385 to 2047 tiles the launch is a few workgroups per CU, all started together: the CUs
+# that got one more set the time, and workgroups in lockstep share a CU worse than staggered
+# ones (576 tiles at K = 4096 run at 62 TFLOP/s, 1024 tiles at 90).  Cutting k into 2 to 8
+# ranges makes more, shorter workgroups that the dispatcher balances (576 tiles: 93 TFLOP/s).
+_CUT_MID_BELOW_TILES = 2048
+_CUT_MID_SLICES = (2, 3, 4, 6, 8)
+_CUT_MID_OVERHEAD = 40          # fixed cost of a workgroup among many, in k walked
+_CUT_MID_LOCKSTEP = 0.46        # cost of a one-round launch per workgroup on the fullest CU (1/3 if staggered)
+_CUT_MID_TAIL = 0.64            # rounds of 768 added for the last workgroups of a balanced launch
+_CUT_MID_FINISH = 0.07          # storing and adding one partial tile, in k walked
+_CUT_MID_WORTH = 0.86
+_CUT_MID_MAX_PARTIAL_BYTES = 512 << 20
 
 
 def _cut_over_contraction(params):
@@ -498,8 +510,15 @@ def _cut_over_contraction(params):
         return None
     tiles = -(-params.m // 128) * -(-params.n // 128)
     K = params.k
-    if tiles == 0 or tiles >= _CUT_BELOW_TILES or K < 4 * _CUT_MIN_DEPTH:
+    if tiles == 0 or K < 4 * _CUT_MIN_DEPTH:
         return None
+    mirrored = (params.a == params.b and params.m == params.n and params.a_ld == params.b_ld
+                and params.a_majorness == params.b_majorness and not params.flags & _backend.FLAG_NO_SYMMETRY)
+    if mirrored:
+        side = -(-params.m // 128)
+        tiles = side * (side + 1) // 2      # the kernel computes one triangle and mirrors it
+    if tiles >= _CUT_BELOW_TILES:
+        return _cut_mid_size(params, tiles, mirrored)
 
     def rounds(count):
         return -(-count // _CUT_CONCURRENT_TILES)
@@ -522,6 +541,34 @@ def _cut_over_contraction(params):
         if best is None or cost < best[0]:
             best = (cost, slices, depth, leftover)
     if best is None or best[0] > _CUT_WORTH * unsplit:
+        return None
+    return best[1:]
+
+
+def _cut_mid_size(params, tiles, mirrored):
+    """The cut for 385 to 2047 tiles to compute: a few ranges of k, several rounds of workgroups."""
+    K = params.k
+    working = tiles
+    if working >= _CUT_MID_BELOW_TILES:
+        return None
+    fullest_cu = -(-working // 256)
+    finish = _CUT_MID_FINISH * (2 if mirrored else 1)     # a mirrored tile is stored and added twice
+    unsplit = (K + _CUT_MID_OVERHEAD) * _CUT_MID_LOCKSTEP * fullest_cu
+    plane_bytes = 4 * -(-params.m // 4) * 4 * params.n
+    best = None
+    for wanted in _CUT_MID_SLICES:
+        depth = -(-K // (16 * wanted)) * 16
+        slices = K // depth
+        leftover = K - slices * depth
+        if depth < _CUT_MIN_DEPTH or slices < 2 or (slices + 1) * plane_bytes > _CUT_MID_MAX_PARTIAL_BYTES:
+            continue
+        cost = ((depth + _CUT_MID_OVERHEAD) * (slices * working / _CUT_CONCURRENT_TILES + _CUT_MID_TAIL)
+                + finish * slices * working)
+        if leftover:
+            cost += (leftover + _CUT_MID_OVERHEAD) * _CUT_MID_LOCKSTEP * fullest_cu + finish * working
+        if best is None or cost < best[0]:
+            best = (cost, slices, depth, leftover)
+    if best is None or best[0] > _CUT_MID_WORTH * unsplit:
         return None
     return best[1:]
 

@@ -113,3 +113,37 @@ def test_finish_entry_point_adds_slices_and_applies_the_epilogue(device, m, n, s
     _backend.build_kernel_finish(params, partial.data_ptr(), ld, 0, n * ld, slices, stream)
     torch.cuda.synchronize()
     assert torch.equal(out, again), "the order of the sum is fixed: two runs agree bit for bit"
+
+
+@pytest.mark.parametrize("p,M,N,K,col_major", [(1.0, 3000, 2900, 2048, True), (2.0, 3000, 3100, 1024 + 512, False),
+                                              (1.3, 2560, 2560, 2048, True)])
+def test_a_result_of_a_few_hundred_tiles_is_cut_into_a_few_ranges(device, monkeypatch, p, M, N, K, col_major):
+    """385 to 2047 tiles: k is cut into 2 to 8 ranges, several rounds of shorter workgroups.  Checked
+    against the oracle on slabs of rows and against the uncut launch everywhere."""
+    g = torch.Generator().manual_seed(int(p * 10) + M)
+    a = make_operand(1, M, K, col_major, device, g, batch=False)
+    b = make_operand(1, N, K, col_major, device, g, batch=False)
+    descriptor = {1.0: kermac.kernel_descriptor_l1_norm, 2.0: kermac.kernel_descriptor_l2_norm,
+                  1.3: kermac.kernel_descriptor_p_norm}[p]
+    plan = module._plan_run_kernel(descriptor, a, b, None, p if p == 1.3 else None, None, None, None, None, None, 0, 0, False)
+    cut = module._cut_over_contraction(plan.params)
+    assert cut is not None and 2 <= cut[0] <= 8, cut
+    got = kermac.cdist(a, b, p=p)[0]             # unbatched operands, out=None: the result is [1, M, N]
+    rtol = 1e-4 if p == 1.3 else 1e-5
+    for rows in (slice(0, 48), slice(M - 48, M)):
+        assert_close_to_truth(got[rows], oracle.cdist(a[rows].cpu(), b.cpu(), p=p)[0], rtol=rtol, what=f"mid-size cut p={p}")
+    monkeypatch.setattr(module, "_cut_over_contraction", lambda params: None)
+    uncut = kermac.cdist(a, b, p=p)[0]
+    assert_close_to_truth(got, uncut, rtol=rtol / 2, what="cut against uncut")
+
+
+def test_a_set_against_itself_is_cut_by_the_tiles_of_one_triangle(device):
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(2048, 4096, generator=g).to(device).t()       # K-major, 32 x 32 tiles, 528 to compute
+    plan = module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, x, x, None, None, None, None, None, None, None, 0, 0, False)
+    assert module._cut_over_contraction(plan.params) is not None
+    got = kermac.cdist(x, x, p=2.0)[0]
+    assert torch.equal(got, got.t())
+    assert torch.all(torch.diagonal(got) == 0.0)
+    rows = slice(1000, 1040)
+    assert_close_to_truth(got[rows], oracle.cdist(x[rows].cpu(), x.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30, what="x against x, cut")
