@@ -168,12 +168,18 @@ def cdist_grad(
 
 # A workgroup owns 64 (m) x 32 or 16 (n) results and walks the whole contraction index k,
 # so few samples and features against many centres (M = 2000, N = 100, K = 10000) launch a
-# hundred workgroups on 256 CUs.  Such an unbatched call is cut over k: slices of a, b and
-# c become the batch of one launch through strided views (d broadcasts), every slice writes
-# a partial result, and the partial results are summed in a fixed order.
-_SPLIT_BELOW_WORKGROUPS = 256
-_SPLIT_TARGET_WORKGROUPS = 768
-_SPLIT_MIN_DEPTH = 1024
+# hundred workgroups on 256 CUs, and a few hundred workgroups, all started together, leave
+# the CUs unevenly loaded (256 workgroups at O = 16: 65 TFLOP/s where 4096 reach 120).  Such
+# an unbatched call is cut over k: slices of a, b and c become the batch of one launch
+# through strided views (d broadcasts), every slice writes a partial result, and the
+# partial results are summed in a fixed order.  Measured at N = 128, K = 4096, cut in 8:
+# O = 16, M = 2048: 65 -> 96 TFLOP/s; O = 1, M = 4096: 24 -> 60; nothing from 1536
+# workgroups on.
+_SPLIT_BELOW_WORKGROUPS = 1536
+_SPLIT_TARGET_WORKGROUPS = 3072
+_SPLIT_MIN_DEPTH = 512                      # from 512 workgroups on: 1024, and 2048 for the matrix-core kernels
+_SPLIT_MAX_SLICES = 24
+_SPLIT_MAX_PARTIAL_BYTES = 512 << 20
 
 
 def _split_over_contraction(plan):
@@ -183,9 +189,11 @@ def _split_over_contraction(plan):
     M, N, O, K = plan.M, plan.N, plan.O, plan.K
     n_tile = 32 if O <= 8 else 16
     workgroups = -(-M // 64) * -(-N // n_tile) * max(1, -(-O // 32))
-    if workgroups >= _SPLIT_BELOW_WORKGROUPS or K < 2 * _SPLIT_MIN_DEPTH:
+    min_depth = _SPLIT_MIN_DEPTH * (1 if workgroups < 512 else 2 if O <= 8 else 4)
+    if workgroups >= _SPLIT_BELOW_WORKGROUPS or K < 2 * min_depth:
         return None
-    slices = min(_SPLIT_TARGET_WORKGROUPS // workgroups, K // _SPLIT_MIN_DEPTH)
+    slices = min(max(2, round(_SPLIT_TARGET_WORKGROUPS / workgroups)), K // min_depth, _SPLIT_MAX_SLICES,
+                 _SPLIT_MAX_PARTIAL_BYTES // (4 * O * N * M) - 1)
     if slices < 2:
         return None
     depth = K // slices // 64 * 64       # whole K slices of the kernels; 16-byte alignment survives

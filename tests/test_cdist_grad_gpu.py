@@ -163,7 +163,8 @@ def test_gradient_empty_contraction_writes_zeros(device):
 
 
 @pytest.mark.parametrize("p", [1.0, 2.0, 1.3])
-@pytest.mark.parametrize("M,N,O,K", [(200, 40, 1, 4100), (130, 10, 3, 2048), (64, 100, 16, 5000)])
+@pytest.mark.parametrize("M,N,O,K", [(200, 40, 1, 4100), (130, 10, 3, 2048), (64, 100, 16, 5000),
+                                     (2048, 128, 16, 1100), (4100, 250, 2, 2100)])      # 256 and 520 workgroups
 def test_few_results_deep_contraction_is_cut_over_k(device, p, M, N, O, K):
     """Few (m, n) results against a long contraction: one batched launch over slices of k plus a
     fixed-order sum of the partial results (kermac_amd/cdist_grad.py); same values as one walk."""
