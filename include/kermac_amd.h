@@ -134,6 +134,12 @@ typedef struct kmc_build_kernel_params {
     int32_t regularization_offset_y;
     float epsilon;
     float gram_trust;           /* used with KMC_FLAG_L2_GRAM; <= 0 selects 0.25 */
+    /* 0, or the length of one contraction whose consecutive ranges are the batch
+     * entries of this launch (see kmc_build_kernel_finish): entry l then walks the k
+     * terms from l*k on, the last entry only the k_total - (l-1)*k that are left
+     * (1 .. k of them; l must be ceil(k_total / k)).  kmc_build_kernel only, not with
+     * the matrix-core flags.  No counterpart in the reference. */
+    int32_t k_total;
 } kmc_build_kernel_params;
 
 /* Stands in for launch(stream, config, cute_build_kernel<...>, *args)
@@ -149,7 +155,8 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream);
  * kmc_build_kernel on `slices` ranges of k with outer_power = KMC_POW_NOOP and
  * kernel_type = KMC_KERNEL_NONE into partial results
  *   partials[m + n*partial_ld + l*partial_bs + s*partial_slice]
- * (a batched launch over strided views does all slices at once); this entry point
+ * (a batched launch over strided views does all slices at once, with k_total for a
+ * shorter last range); this entry point
  * adds the partial results in slice order and applies outer power, epsilon mask,
  * kernel function and regularised diagonal of `params` exactly like
  * kmc_build_kernel, writing C.  `a`, `b` and `k` of `params` are not read.

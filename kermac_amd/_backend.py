@@ -55,6 +55,7 @@ class BuildKernelParams(Structure):
         ("regularization_offset_x", c_int32), ("regularization_offset_y", c_int32),
         ("epsilon", c_float),
         ("gram_trust", c_float),
+        ("k_total", c_int32),
     ]
 
 

@@ -13,6 +13,7 @@ View convention (torch.cdist's): ``a`` is ``[L?, M, K]``, ``b`` is ``[L?, N, K]`
 """
 from __future__ import annotations
 
+import functools
 import os
 from enum import Enum, auto
 from itertools import product
@@ -482,35 +483,62 @@ def run_kernel(
 
 # A workgroup owns one 128 x 128 tile of the result and walks the whole contraction index, so
 # a small result over a long contraction (100 x 100 over k = 100000 is one tile) leaves the
-# chip idle.  Such an unbatched call is cut over k: ranges of k become the batch of one launch
-# that stores plain sums (no outer power, no kernel function) into a buffer, and a second,
-# element-wise kernel adds the partial sums in slice order and applies the epilogue.
-_CUT_BELOW_TILES = 385          # up to 384 tiles two slices still fit one round
-_CUT_CONCURRENT_TILES = 768     # three workgroups per CU
+# chip idle, and a few hundred tiles are a few workgroups per CU, all started together: the
+# CUs that got one more set the time, and workgroups in lockstep share a CU worse than
+# staggered ones (576 tiles at K = 4096 run at 62 TFLOP/s, 1024 tiles at 90).  Such an
+# unbatched call is cut over k: ranges of k become the batch of one launch that stores plain
+# sums (no outer power, no kernel function) into a buffer, and a second, element-wise kernel
+# adds the partial sums in range order and applies the epilogue.  The number of ranges comes
+# from a model of the launch time fitted to sweeps of M = N = 512 ... 5760, K = 1024 ... 16384.
+_CUT_BELOW_TILES = 2048
+_CUT_MIN_K = 512
 _CUT_MIN_DEPTH = 128
-_CUT_WORKGROUP_OVERHEAD = 128   # start-up, first loads and stores of a workgroup, in k walked
-_CUT_WORTH = 0.8                # cut only for at least 20 % less modelled time
-# From 385 to 2047 tiles the launch is a few workgroups per CU, all started together: the CUs
-# that got one more set the time, and workgroups in lockstep share a CU worse than staggered
-# ones (576 tiles at K = 4096 run at 62 TFLOP/s, 1024 tiles at 90).  Cutting k into 2 to 8
-# ranges makes more, shorter workgroups that the dispatcher balances (576 tiles: 93 TFLOP/s).
-_CUT_MID_BELOW_TILES = 2048
-_CUT_MID_SLICES = (2, 3, 4, 6, 8)
-_CUT_MID_OVERHEAD = 40          # fixed cost of a workgroup among many, in k walked
-_CUT_MID_LOCKSTEP = 0.46        # cost of a one-round launch per workgroup on the fullest CU (1/3 if staggered)
-_CUT_MID_TAIL = 0.64            # rounds of 768 added for the last workgroups of a balanced launch
-_CUT_MID_FINISH = 0.07          # storing and adding one partial tile, in k walked
-_CUT_MID_WORTH = 0.86
-_CUT_MID_MAX_PARTIAL_BYTES = 512 << 20
+_CUT_RANGES = (2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768)
+_CUT_WORTH = 0.9                # cut only for at least 10 % less modelled time
+_CUT_MAX_PARTIAL_BYTES = 512 << 20
+
+
+def _launch_ms(workgroups, depth):
+    """Modelled time of `workgroups` tiles that walk `depth` terms each, in milliseconds."""
+    per_cu = workgroups / 256
+    if per_cu <= 1:
+        return (depth + 128) / 3900             # one wave per SIMD: latency bound
+    if per_cu <= 3:
+        return -(-workgroups // 256) * (depth + 128) / 7300      # one round, in lockstep
+    return (per_cu + 1.92) * (depth + 40) / 10000                # rounds that the dispatcher balances
+
+
+@functools.lru_cache(maxsize=256)
+def _choose_cut(tiles, K, mirrored, plane_bytes):
+    # A mirrored launch has as many empty workgroups as working ones, and the working ones
+    # end up unevenly spread over the CUs; its workgroups also store every tile twice.
+    unsplit = _launch_ms(tiles * (1.3 if mirrored else 1.0), K)
+    best = None
+    seen = 0
+    for wanted in _CUT_RANGES:
+        depth = -(-K // (16 * wanted)) * 16
+        if depth < _CUT_MIN_DEPTH:
+            break
+        ranges = -(-K // depth)
+        if ranges < 2 or ranges == seen or ranges * plane_bytes > _CUT_MAX_PARTIAL_BYTES:
+            continue
+        seen = ranges
+        workgroups = ranges * tiles
+        cost = (_launch_ms(workgroups, depth) * (1.35 if mirrored else 1.0)
+                + 2.1e-5 * workgroups * (2 if mirrored else 1) + 0.01)      # partial sums stored and added, second launch
+        if best is None or cost < best[0]:
+            best = (cost, ranges, depth)
+    if best is None or best[0] > _CUT_WORTH * unsplit:
+        return None
+    return best[1:]
 
 
 def _cut_over_contraction(params):
-    """(slices, k per slice, leftover k), or None when the launch goes out as it is."""
+    """(ranges of k, k per range), or None when the launch goes out as it is."""
     if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
         return None
     tiles = -(-params.m // 128) * -(-params.n // 128)
-    K = params.k
-    if tiles == 0 or K < 4 * _CUT_MIN_DEPTH:
+    if tiles == 0 or params.k < _CUT_MIN_K:
         return None
     mirrored = (params.a == params.b and params.m == params.n and params.a_ld == params.b_ld
                 and params.a_majorness == params.b_majorness and not params.flags & _backend.FLAG_NO_SYMMETRY)
@@ -518,84 +546,24 @@ def _cut_over_contraction(params):
         side = -(-params.m // 128)
         tiles = side * (side + 1) // 2      # the kernel computes one triangle and mirrors it
     if tiles >= _CUT_BELOW_TILES:
-        return _cut_mid_size(params, tiles, mirrored)
-
-    def rounds(count):
-        return -(-count // _CUT_CONCURRENT_TILES)
-
-    # Modelled time of a launch: k walked per workgroup (plus its fixed cost) times rounds of
-    # workgroups; a leftover range of k is a second launch.  Depths are whole K slices of the
-    # kernel (16), so 16-byte alignment survives; a few depths from the one that fills one round
-    # upwards are tried, which finds the cuts without (or with a small) leftover.
-    unsplit = (K + _CUT_WORKGROUP_OVERHEAD) * rounds(tiles)
-    first = max(_CUT_MIN_DEPTH, -(-K * tiles // _CUT_CONCURRENT_TILES // 16) * 16)
-    best = None
-    for depth in range(first, first + 16 * 24, 16):
-        slices = K // depth
-        if slices < 2:
-            break
-        leftover = K - slices * depth
-        cost = (depth + _CUT_WORKGROUP_OVERHEAD) * rounds(slices * tiles)
-        if leftover:
-            cost += (leftover + 2 * _CUT_WORKGROUP_OVERHEAD) * rounds(tiles)
-        if best is None or cost < best[0]:
-            best = (cost, slices, depth, leftover)
-    if best is None or best[0] > _CUT_WORTH * unsplit:
         return None
-    return best[1:]
-
-
-def _cut_mid_size(params, tiles, mirrored):
-    """The cut for 385 to 2047 tiles to compute: a few ranges of k, several rounds of workgroups."""
-    K = params.k
-    working = tiles
-    if working >= _CUT_MID_BELOW_TILES:
-        return None
-    fullest_cu = -(-working // 256)
-    finish = _CUT_MID_FINISH * (2 if mirrored else 1)     # a mirrored tile is stored and added twice
-    unsplit = (K + _CUT_MID_OVERHEAD) * _CUT_MID_LOCKSTEP * fullest_cu
-    plane_bytes = 4 * -(-params.m // 4) * 4 * params.n
-    best = None
-    for wanted in _CUT_MID_SLICES:
-        depth = -(-K // (16 * wanted)) * 16
-        slices = K // depth
-        leftover = K - slices * depth
-        if depth < _CUT_MIN_DEPTH or slices < 2 or (slices + 1) * plane_bytes > _CUT_MID_MAX_PARTIAL_BYTES:
-            continue
-        cost = ((depth + _CUT_MID_OVERHEAD) * (slices * working / _CUT_CONCURRENT_TILES + _CUT_MID_TAIL)
-                + finish * slices * working)
-        if leftover:
-            cost += (leftover + _CUT_MID_OVERHEAD) * _CUT_MID_LOCKSTEP * fullest_cu + finish * working
-        if best is None or cost < best[0]:
-            best = (cost, slices, depth, leftover)
-    if best is None or best[0] > _CUT_MID_WORTH * unsplit:
-        return None
-    return best[1:]
+    return _choose_cut(tiles, params.k, bool(mirrored), 4 * -(-params.m // 4) * 4 * params.n)
 
 
 def _run_cut_over_contraction(cut, params, launch, stream, device):
-    slices, depth, leftover = cut
-    count = slices + (1 if leftover else 0)
+    slices, depth = cut
     ld = -(-params.m // 4) * 4
     plane = ld * params.n
-    partial = torch.empty(count * plane, dtype=torch.float32, device=device)
+    partial = torch.empty(slices * plane, dtype=torch.float32, device=device)
 
     def k_stride(majorness, leading):
         return leading if majorness == _backend.COL_MAJOR else 1
 
-    step_a = depth * k_stride(params.a_majorness, params.a_ld)
-    step_b = depth * k_stride(params.b_majorness, params.b_ld)
-    first = _backend.BuildKernelParams.from_buffer_copy(params)
-    first.outer_power, first.kernel_type = _POWER_TYPE_ABI[PowerType.NOOP], _KERNEL_TYPE_ABI[KernelType.NONE]
-    first.k, first.l = depth, slices
-    first.a_bs, first.b_bs = step_a, step_b
-    first.c, first.c_ld, first.c_bs = partial.data_ptr(), ld, plane
-    launch(first)
-    if leftover:
-        last = _backend.BuildKernelParams.from_buffer_copy(first)
-        last.k, last.l = leftover, 1
-        last.a = params.a + 4 * slices * step_a
-        last.b = params.b + 4 * slices * step_b
-        last.c = partial.data_ptr() + 4 * slices * plane
-        launch(last)
-    _backend.build_kernel_finish(params, partial.data_ptr(), ld, 0, plane, count, stream)
+    ranges = _backend.BuildKernelParams.from_buffer_copy(params)
+    ranges.outer_power, ranges.kernel_type = _POWER_TYPE_ABI[PowerType.NOOP], _KERNEL_TYPE_ABI[KernelType.NONE]
+    ranges.k, ranges.l, ranges.k_total = depth, slices, params.k      # the last range is what is left of k
+    ranges.a_bs = depth * k_stride(params.a_majorness, params.a_ld)
+    ranges.b_bs = depth * k_stride(params.b_majorness, params.b_ld)
+    ranges.c, ranges.c_ld, ranges.c_bs = partial.data_ptr(), ld, plane
+    launch(ranges)
+    _backend.build_kernel_finish(params, partial.data_ptr(), ld, 0, plane, slices, stream)

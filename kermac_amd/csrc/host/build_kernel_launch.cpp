@@ -96,6 +96,17 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
                       p->a_ld == p->b_ld && p->a_bs == p->b_bs && p->a_majorness == p->b_majorness &&
                       p->regularization_offset_x == p->regularization_offset_y && tiles_m > 1;
     args->gram_trust = p->gram_trust > 0.0f ? p->gram_trust : 0.25f;
+    if (p->k_total < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "negative k_total %d", p->k_total);
+    if (p->k_total > 0) {
+        // the batch entries are ranges of one contraction: all but the last are full
+        const int64_t before_last = static_cast<int64_t>(p->l - 1) * p->k;
+        if (p->l < 1 || p->k < 1 || before_last >= p->k_total || before_last + p->k < p->k_total)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "k_total=%d is not covered by l=%d ranges of k=%d, the last one not empty",
+                        p->k_total, p->l, p->k);
+        if (p->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16))
+            return fail(KMC_ERR_INVALID_ARGUMENT, "k_total cannot be combined with the matrix-core flags");
+    }
+    args->k_total = p->k_total;
     args->outer_power = p->outer_power;
     args->kernel_type = p->kernel_type;
     args->c_vec = need_c && !(p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) && aligned16(p->c) && p->c_ld % 4 == 0 &&

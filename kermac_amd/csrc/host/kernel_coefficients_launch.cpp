@@ -24,6 +24,7 @@ int prepare(const kmc_kernel_coefficients_params *p, bool wide_allowed, kmc::Ker
     int status = prepare_build_kernel(&p->kernel, false, &kc->kernel, load_a, load_b);
     if (status != KMC_OK) return status;
     if (p->o < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "negative coefficient column count %d", p->o);
+    if (p->kernel.k_total != 0) return fail(KMC_ERR_INVALID_ARGUMENT, "k_total is for kmc_build_kernel only");
     const kmc::BuildKernelArgs &k = kc->kernel;
     *empty = k.m == 0 || k.l == 0 || p->o == 0;
     if (*empty) return KMC_OK;

@@ -48,6 +48,8 @@ struct BuildKernelArgs {
     int symmetric;       // A and B are the same panel and the result is symmetric: only tiles with
                          // tile_m >= tile_n are computed, each is also stored mirrored
     float gram_trust;    // gram_kernel.hpp: distrust d^2 below gram_trust * (|a|^2 + |b|^2)
+    int k_total;         // 0, or: the batch entries are consecutive ranges of k terms of one contraction of
+                         // k_total terms, and the last entry walks only what is left
 };
 
 constexpr int BK_TILE_M = 128;
@@ -486,12 +488,13 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
 #pragma unroll
         for (int i = 0; i < 8; i++) acc[j][i] = 0.0f;
 
-    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
+    const int k_here = args.k_total > 0 ? min(args.k, args.k_total - batch * args.k) : args.k;
+    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && k_here % BK_TILE_K == 0) {
         accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, true>(
-            acc, load_a, load_b, lds_a, lds_b, args.k, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
+            acc, load_a, load_b, lds_a, lds_b, k_here, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
     } else {
         accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, false>(
-            acc, load_a, load_b, lds_a, lds_b, args.k, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
+            acc, load_a, load_b, lds_a, lds_b, k_here, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
     }
 
     finish_tile(acc, args, batch, m0, n0, tx, ty);

@@ -77,8 +77,10 @@ def test_batched_and_large_results_are_not_cut(device):
     a = torch.rand(3, 100, 3000, device=device)
     b = torch.rand(3, 90, 3000, device=device)
     assert not is_cut(kermac.kernel_descriptor_l1_norm, a, b)
-    a = torch.rand(3000, 600, device=device)
-    assert not is_cut(kermac.kernel_descriptor_l1_norm, a, a)          # 576 tiles: the chip is full
+    a = torch.rand(6000, 600, device=device)
+    assert not is_cut(kermac.kernel_descriptor_l1_norm, a, a)          # 1128 tiles to compute: the chip is full
+    b = torch.rand(17000, 2048, device=device)
+    assert not is_cut(kermac.kernel_descriptor_l1_norm, b, a.new_empty(16400, 2048))     # 2048 tiles and more: never
     a = torch.rand(100, 400, device=device)
     assert not is_cut(kermac.kernel_descriptor_l1_norm, a, a)          # contraction too short
 
@@ -115,7 +117,7 @@ def test_finish_entry_point_adds_slices_and_applies_the_epilogue(device, m, n, s
     assert torch.equal(out, again), "the order of the sum is fixed: two runs agree bit for bit"
 
 
-@pytest.mark.parametrize("p,M,N,K,col_major", [(1.0, 3000, 2900, 2048, True), (2.0, 3000, 3100, 1024 + 512, False),
+@pytest.mark.parametrize("p,M,N,K,col_major", [(1.0, 3000, 2900, 2048, True), (2.0, 3000, 3100, 1024 + 512, False), (2.0, 3072, 3000, 1000, False),
                                               (1.3, 2560, 2560, 2048, True)])
 def test_a_result_of_a_few_hundred_tiles_is_cut_into_a_few_ranges(device, monkeypatch, p, M, N, K, col_major):
     """385 to 2047 tiles: k is cut into 2 to 8 ranges, several rounds of shorter workgroups.  Checked
@@ -139,7 +141,7 @@ def test_a_result_of_a_few_hundred_tiles_is_cut_into_a_few_ranges(device, monkey
 
 def test_a_set_against_itself_is_cut_by_the_tiles_of_one_triangle(device):
     g = torch.Generator().manual_seed(77)
-    x = torch.randn(2048, 4096, generator=g).to(device).t()       # K-major, 32 x 32 tiles, 528 to compute
+    x = torch.randn(2048, 3584, generator=g).to(device).t()       # K-major, 28 x 28 tiles, 406 to compute
     plan = module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, x, x, None, None, None, None, None, None, None, 0, 0, False)
     assert module._cut_over_contraction(plan.params) is not None
     got = kermac.cdist(x, x, p=2.0)[0]

@@ -429,6 +429,21 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
         with pytest.raises(_backend.BackendError) as info:
             _backend.build_kernel_finish(params, partials, ld, 0, 64, slices, 0)
         assert info.value.status == _backend.ERR_INVALID_ARGUMENT and word in str(info.value), str(info.value)
+    # ranges of one contraction as batch entries: k_total must be covered by l ranges of k, the last not empty
+    for l, k, k_total, flags, word in ((3, 8, -1, 0, "k_total"), (3, 8, 30, 0, "not covered"), (3, 8, 16, 0, "not covered"),
+                                       (3, 8, 20, _backend.FLAG_L2_GRAM, "matrix-core")):
+        ranged = _backend.BuildKernelParams.from_buffer_copy(params)
+        ranged.inner_power = 2
+        ranged.l, ranged.k, ranged.k_total, ranged.flags = l, k, k_total, flags
+        with pytest.raises(_backend.BackendError) as info:
+            _backend.build_kernel(ranged, 0)
+        assert info.value.status == _backend.ERR_INVALID_ARGUMENT and word in str(info.value), str(info.value)
+    fused = _backend.KernelCoefficientsParams()
+    fused.kernel = _backend.BuildKernelParams.from_buffer_copy(params)
+    fused.kernel.k_total = 8
+    with pytest.raises(_backend.BackendError) as info:
+        _backend.kernel_times_coefficients(fused, 0)
+    assert "k_total" in str(info.value)
     params.m = 0
     _backend.build_kernel_finish(params, 0, 0, 0, 0, 0, 0)      # empty result: accepted, nothing launched
     # a device that is not a gfx950 is a ValueError, as an unsupported compute capability is in
