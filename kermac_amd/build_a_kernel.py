@@ -510,9 +510,9 @@ def _launch_ms(workgroups, depth):
 
 @functools.lru_cache(maxsize=256)
 def _choose_cut(tiles, K, mirrored, plane_bytes):
-    # A mirrored launch has as many empty workgroups as working ones, and the working ones
-    # end up unevenly spread over the CUs; its workgroups also store every tile twice.
-    unsplit = _launch_ms(tiles * (1.3 if mirrored else 1.0), K)
+    # A mirrored launch of so few tiles has one workgroup per tile of the triangle (no empty
+    # ones); its workgroups store every tile twice.
+    unsplit = _launch_ms(tiles, K)
     best = None
     seen = 0
     for wanted in _CUT_RANGES:
@@ -524,7 +524,7 @@ def _choose_cut(tiles, K, mirrored, plane_bytes):
             continue
         seen = ranges
         workgroups = ranges * tiles
-        cost = (_launch_ms(workgroups, depth) * (1.35 if mirrored else 1.0)
+        cost = (_launch_ms(workgroups, depth)
                 + 2.1e-5 * workgroups * (2 if mirrored else 1) + 0.01)      # partial sums stored and added, second launch
         if best is None or cost < best[0]:
             best = (cost, ranges, depth)

@@ -114,6 +114,7 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
     args->tiles_m = static_cast<int>(tiles_m);
     args->tiles_n = static_cast<int>(tiles_n);
     args->tiles_n_padded = static_cast<int>(tiles_n_padded);
+    args->grid_width = static_cast<int>(args->symmetric ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n_padded);
     *load_a = pick_load_mode(p->a, p->a_ld, p->a_bs, p->a_majorness, p->flags);
     *load_b = pick_load_mode(p->b, p->b_ld, p->b_bs, p->b_majorness, p->flags);
     return KMC_OK;
@@ -187,7 +188,7 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
     if (args.m == 0 || args.n == 0 || args.l == 0) return KMC_OK;
     status = require_gfx950();
     if (status != KMC_OK) return status;
-    const dim3 grid(static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n_padded), args.l, 1);
+    const dim3 grid(static_cast<unsigned>(args.grid_width), args.l, 1);
     if (params->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16)) {
         if (params->inner_operator != KMC_OP_DIFF || params->inner_power != KMC_POW_SQUARE)
             return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L2_GRAM needs inner_operator DIFF and inner_power SQUARE");
@@ -240,7 +241,7 @@ int kmc_build_kernel_jit(void *function, const kmc_build_kernel_params *params, 
     size_t size = sizeof(args);
     void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
     hipError_t e = hipModuleLaunchKernel(static_cast<hipFunction_t>(function),
-                                         static_cast<unsigned>(args.tiles_m) * static_cast<unsigned>(args.tiles_n_padded),
+                                         static_cast<unsigned>(args.grid_width),
                                          args.l, 1, kmc::BK_THREADS, 1, 1, 0, static_cast<hipStream_t>(stream), nullptr,
                                          config);
     if (e != hipSuccess) return fail_hip(e, "build_kernel (run-time compiled) launch");

@@ -50,6 +50,7 @@ struct BuildKernelArgs {
     float gram_trust;    // gram_kernel.hpp: distrust d^2 below gram_trust * (|a|^2 + |b|^2)
     int k_total;         // 0, or: the batch entries are consecutive ranges of k terms of one contraction of
                          // k_total terms, and the last entry walks only what is left
+    int grid_width;      // gridDim.x: tiles_m * tiles_n_padded, or (symmetric) the tiles of one triangle
 };
 
 constexpr int BK_TILE_M = 128;
@@ -432,14 +433,25 @@ __device__ __forceinline__ bool tile_of_workgroup(const BuildKernelArgs &args, i
     // described above, survive the rotation.
     const int rotated = blockIdx.x + blockIdx.y % gridDim.x;
     const int linear = rotated >= (int)gridDim.x ? rotated - (int)gridDim.x : rotated;
+    if (args.symmetric) {
+        // Symmetric result: the ids count through the tiles on and below the diagonal, row r
+        // of the triangle starting at id r (r + 1) / 2.  (In the band order half the
+        // workgroups would be empty and XCD x would own the tile rows n = x mod 8, which have
+        // different lengths: 80 tiles for XCD 0 and 52 for XCD 7 at 32 x 32 tiles, which then
+        // took as long as computing every tile; at 235 x 235 tiles the band order cost 10 %.)
+        int row = (int)((sqrtf(8.0f * (float)linear + 1.0f) - 1.0f) * 0.5f);
+        while (row * (row + 1) / 2 > linear) row--;
+        while ((row + 1) * (row + 2) / 2 <= linear) row++;
+        tile_m = row;
+        tile_n = linear - row * (row + 1) / 2;
+        return true;
+    }
     const int band_tiles = BK_BAND_N * args.tiles_m;
     const int band = linear / band_tiles;
     const int band_height = min(BK_BAND_N, args.tiles_n_padded - band * BK_BAND_N);
     const int in_band = linear - band * band_tiles;
     tile_m = in_band / band_height;
     tile_n = band * BK_BAND_N + in_band % band_height;
-    // Symmetric result: the workgroups of the upper triangle have nothing to do.
-    if (args.symmetric && tile_n > tile_m) return false;
     return tile_n < args.tiles_n;
 }
 
