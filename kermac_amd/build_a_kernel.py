@@ -484,8 +484,8 @@ def run_kernel(
 # A workgroup owns one 128 x 128 tile of the result and walks the whole contraction index, so
 # a small result over a long contraction (100 x 100 over k = 100000 is one tile) leaves the
 # chip idle, and a few hundred tiles are a few workgroups per CU, all started together: the
-# CUs that got one more set the time, and workgroups in lockstep share a CU worse than
-# staggered ones (576 tiles at K = 4096 run at 62 TFLOP/s, 1024 tiles at 90).  Such an
+# CUs that got one more set the time, and a CU works through such a single round at 0.73 of
+# the rate it reaches on a long queue (576 tiles at K = 4096 run at 62 TFLOP/s, 1024 at 90).  Such an
 # unbatched call is cut over k: ranges of k become the batch of one launch that stores plain
 # sums (no outer power, no kernel function) into a buffer, and a second, element-wise kernel
 # adds the partial sums in range order and applies the epilogue.  The number of ranges comes
@@ -504,7 +504,7 @@ def _launch_ms(workgroups, depth):
     if per_cu <= 1:
         return (depth + 128) / 3900             # one wave per SIMD: latency bound
     if per_cu <= 3:
-        return -(-workgroups // 256) * (depth + 128) / 7300      # one round, in lockstep
+        return -(-workgroups // 256) * (depth + 128) / 7300      # one round
     return (per_cu + 1.92) * (depth + 40) / 10000                # rounds that the dispatcher balances
 
 
