@@ -4,7 +4,7 @@ outputs or a deep contraction.  Prints milliseconds and TFLOP/s in the units of 
 (3 operations per (m, n, k) for the pairwise kernels, (2 O + 3) per (m, n, k) for the gradient).
 
     python examples/shapes.py            # everything
-    python examples/shapes.py cdist      # one group: cdist, grad or fused
+    python examples/shapes.py cdist      # one group: cdist, self, grad or fused
 """
 import sys
 from pathlib import Path
@@ -31,7 +31,8 @@ def cdist_shapes(device):
     print("cdist, K-major panels: L, M, N, K -> p = 1 / p = 2")
     shapes = [(1, 30000, 30000, 1024), (1, 4096, 4096, 1024), (1, 2048, 2048, 1024), (1, 1024, 1024, 4096),
               (1, 100, 100, 100000), (1, 512, 512, 16384), (1, 128, 1000000, 64), (1, 1000, 100000, 512),
-              (1, 30000, 30000, 16), (64, 512, 512, 256), (1000, 128, 128, 128)]
+              (1, 30000, 30000, 16), (64, 512, 512, 256), (1000, 128, 128, 128), (1, 3000, 2900, 2048),
+              (1, 3072, 3072, 1000), (1, 2304, 2304, 16384)]
     for L, M, N, K in shapes:
         a = torch.randn(L, K, M, device=device).transpose(1, 2)
         b = torch.randn(L, K, N, device=device).transpose(1, 2)
@@ -42,6 +43,19 @@ def cdist_shapes(device):
             cells.append(f"{ms:8.3f} ms {3.0 * L * M * N * K / ms / 1e9:6.1f} TFLOP/s")
         print(f"  {L:5d} {M:6d} {N:8d} {K:7d}   " + "   ".join(cells), flush=True)
         del a, b, out
+
+
+def self_shapes(device):
+    print("cdist of a set against itself (one triangle of tiles computed, mirrored): M, K -> p = 1 / p = 2")
+    for M, K in ((30000, 1024), (8192, 1024), (4096, 4096), (3072, 1024), (1536, 4096)):
+        x = torch.randn(K, M, device=device).t()
+        out = torch.empty(M, M, device=device).t()
+        cells = []
+        for p in (1.0, 2.0):
+            ms = timeit(lambda: kermac.cdist(x, x, out=out, p=p))
+            cells.append(f"{ms:8.3f} ms {3.0 * M * M * K / ms / 1e9:6.1f} TFLOP/s of the full matrix")
+        print(f"  {M:6d} {K:6d}   " + "   ".join(cells), flush=True)
+        del x, out
 
 
 def grad_shapes(device):
@@ -85,7 +99,7 @@ def fused_shapes(device):
 if __name__ == "__main__":
     if not torch.cuda.is_available():
         sys.exit("examples/shapes.py needs a GPU")
-    groups = {"cdist": cdist_shapes, "grad": grad_shapes, "fused": fused_shapes}
+    groups = {"cdist": cdist_shapes, "self": self_shapes, "grad": grad_shapes, "fused": fused_shapes}
     chosen = sys.argv[1:] or list(groups)
     for name in chosen:
         if name not in groups:
