@@ -214,4 +214,9 @@ def _run_split_over_contraction(split, plan, a, b, c, d, p, debug):
         done = slices * depth
         cdist_grad(a2[done:], b2[:, done:], c2[:, done:], d2, out=partial[slices:], p=p, debug=debug, _may_split=False)
     target = plan.out[0] if plan.out.dim() == 4 else plan.out
-    torch.sum(partial, dim=0, out=target)
+    if target.is_contiguous():
+        torch.sum(partial, dim=0, out=target)
+    else:
+        # the order in which torch adds the slices depends on the layout of the result: a strided
+        # `out` gets the bits of a contiguous one
+        target.copy_(torch.sum(partial, dim=0))

@@ -9,6 +9,7 @@ matrix ever reaching memory, with exactly the per-element semantics of
 """
 from __future__ import annotations
 
+import functools
 from typing import Optional
 
 import torch
@@ -140,7 +141,7 @@ def run_kernel_coefficients(
 # broadcasts), each slice writes its own partial result, and the partial results are summed
 # in a fixed order.
 _SPLIT_CONCURRENT_WORKGROUPS = 512
-_SPLIT_MIN_CENTRES = 512
+_SPLIT_MIN_CENTRES = 128
 _SPLIT_WORKGROUP_OVERHEAD = 64           # start-up and store of a workgroup, in centres walked
 _SPLIT_MAX_PARTIAL_BYTES = 256 << 20
 _SPLIT_WORTH = 0.92                      # cut only for at least 8 % less modelled time (448 workgroups: 10 % modelled, 14 % measured)
@@ -152,9 +153,13 @@ def _split_over_centres(plan, a, b, coefficients, regularization):
         return None                      # the batch index of the launch is taken by the caller's batches
     if regularization is not None and not (isinstance(regularization, (int, float)) and regularization == 0):
         return None                      # the regularised diagonal is addressed by the global centre index
-    M, N, O = plan.M, plan.N, plan.O
-    if M == 0 or O == 0 or N < 2 * _SPLIT_MIN_CENTRES:
+    if plan.M == 0 or plan.O == 0 or plan.N < 2 * _SPLIT_MIN_CENTRES:
         return None
+    return _choose_split(plan.M, plan.N, plan.O)
+
+
+@functools.lru_cache(maxsize=256)
+def _choose_split(M, N, O):
     workgroups = -(-M // 128) * max(1, -(-O // 64))
 
     def rounds(count):
@@ -197,4 +202,9 @@ def _run_split_over_centres(split, plan, kernel_descriptor, a, b, coefficients, 
     if leftover:
         run_kernel_coefficients(kernel_descriptor, a2, b2[full * rows:], c2[full * rows:], partial[full:], **hyper)
     target = plan.out[0] if plan.out.dim() == 3 else plan.out
-    torch.sum(partial, dim=0, out=target)
+    if target.is_contiguous():
+        torch.sum(partial, dim=0, out=target)
+    else:
+        # the order in which torch adds the slices depends on the layout of the result: a strided
+        # `out` gets the bits of a contiguous one
+        target.copy_(torch.sum(partial, dim=0))
