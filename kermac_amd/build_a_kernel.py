@@ -23,8 +23,8 @@ import numpy as np
 import torch
 
 from . import _backend
-from .common import (Alignment, Majorness, PyTorchStreamWrapper, TensorStats, ceil_div, merge_batch_size,
-                     tensor_stats)
+from .common import (Alignment, Majorness, PyTorchStreamWrapper, TensorStats, ceil_div, launch_cuts_enabled,
+                     merge_batch_size, tensor_stats)
 from .module_cache.module_cache import ModuleCache, build_kernel_function_name
 
 
@@ -538,7 +538,7 @@ def _cut_over_contraction(params):
     if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
         return None
     tiles = -(-params.m // 128) * -(-params.n // 128)
-    if tiles == 0 or params.k < _CUT_MIN_K:
+    if tiles == 0 or params.k < _CUT_MIN_K or not launch_cuts_enabled():
         return None
     mirrored = (params.a == params.b and params.m == params.n and params.a_ld == params.b_ld
                 and params.a_majorness == params.b_majorness and not params.flags & _backend.FLAG_NO_SYMMETRY)

@@ -12,7 +12,7 @@ import torch
 
 from . import _backend
 from .build_a_kernel import _current_stream_for
-from .common import merge_batch_size, tensor_stats
+from .common import launch_cuts_enabled, merge_batch_size, tensor_stats
 
 _NORM_L1, _NORM_L2, _NORM_P = 0, 1, 2
 
@@ -184,7 +184,7 @@ _SPLIT_MAX_PARTIAL_BYTES = 512 << 20
 
 def _split_over_contraction(plan):
     """(slices, k per slice, leftover k), or None when the call is launched as it is."""
-    if plan.L != 1 or plan.M == 0 or plan.N == 0 or plan.O == 0:
+    if plan.L != 1 or plan.M == 0 or plan.N == 0 or plan.O == 0 or not launch_cuts_enabled():
         return None
     M, N, O, K = plan.M, plan.N, plan.O, plan.K
     n_tile = 32 if O <= 8 else 16

@@ -7,6 +7,7 @@ that code written against it keeps working: ``Majorness``, ``Alignment``,
 """
 from __future__ import annotations
 
+import os
 from enum import Enum, auto
 from typing import Optional, Tuple, Union
 
@@ -62,6 +63,13 @@ class CudaTimer:
         self.end_event.record()
         self.end_event.synchronize()
         return self.start_event.elapsed_time(self.end_event)
+
+
+def launch_cuts_enabled() -> bool:
+    """The Python layer cuts launches that would leave CUs idle into one batched launch over
+    ranges of the contracted index plus a sum of partial results, which needs a temporary
+    buffer (up to 512 MB).  KERMAC_AMD_NO_CUT=1 launches every call exactly as it was given."""
+    return os.environ.get("KERMAC_AMD_NO_CUT", "0") in ("", "0")
 
 
 def ceil_div(x, d):

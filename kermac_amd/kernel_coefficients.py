@@ -15,7 +15,7 @@ from typing import Optional
 import torch
 
 from . import _backend
-from .common import merge_batch_size
+from .common import launch_cuts_enabled, merge_batch_size
 from .module_cache.module_cache import ModuleCache, kernel_coefficients_function_name
 
 
@@ -153,7 +153,7 @@ def _split_over_centres(plan, a, b, coefficients, regularization):
         return None                      # the batch index of the launch is taken by the caller's batches
     if regularization is not None and not (isinstance(regularization, (int, float)) and regularization == 0):
         return None                      # the regularised diagonal is addressed by the global centre index
-    if plan.M == 0 or plan.O == 0 or plan.N < 2 * _SPLIT_MIN_CENTRES:
+    if plan.M == 0 or plan.O == 0 or plan.N < 2 * _SPLIT_MIN_CENTRES or not launch_cuts_enabled():
         return None
     return _choose_split(plan.M, plan.N, plan.O)
 

@@ -451,3 +451,33 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     with pytest.raises(ValueError) as info:
         _backend.check(_backend.ERR_WRONG_DEVICE)
     assert isinstance(info.value, _backend.BackendError) and info.value.status == _backend.ERR_WRONG_DEVICE
+
+
+def test_launch_cuts_follow_the_shape_and_the_environment_switch(monkeypatch):
+    """The cut over k is decided from the parameter block alone: small and middling results over a
+    long contraction are cut, batches, short contractions and large results are not, and
+    KERMAC_AMD_NO_CUT=1 switches every cut off."""
+    from kermac_amd import _backend
+    from kermac_amd import build_a_kernel as module
+
+    def block(m, n, k, l=1, same=False, flags=0):
+        params = _backend.BuildKernelParams()
+        params.m, params.n, params.k, params.l, params.flags = m, n, k, l, flags
+        params.a, params.b = 4096, 4096 if same else 8192
+        params.a_ld = params.b_ld = max(m, n)
+        return params
+
+    monkeypatch.delenv("KERMAC_AMD_NO_CUT", raising=False)
+    ranges, depth = module._cut_over_contraction(block(100, 100, 100000))
+    assert ranges * depth >= 100000 > (ranges - 1) * depth and depth % 16 == 0 and ranges > 100
+    ranges, depth = module._cut_over_contraction(block(3072, 3072, 1000))
+    assert 2 <= ranges <= 8 and ranges * depth >= 1000 > (ranges - 1) * depth
+    assert module._cut_over_contraction(block(3072, 3072, 1000, l=2)) is None                 # batched
+    assert module._cut_over_contraction(block(3072, 3072, 256)) is None                       # short contraction
+    assert module._cut_over_contraction(block(30000, 30000, 1024)) is None                    # the chip is full
+    assert module._cut_over_contraction(block(3072, 3072, 4096, flags=_backend.FLAG_L2_GRAM)) is None
+    # a set against itself counts the tiles of one triangle: 64 x 64 tiles are 2080 to compute, 2048 cut nothing
+    assert module._cut_over_contraction(block(8192, 8192, 4096, same=True)) is None
+    assert module._cut_over_contraction(block(5120, 5120, 4096, same=True)) is not None
+    monkeypatch.setenv("KERMAC_AMD_NO_CUT", "1")
+    assert module._cut_over_contraction(block(100, 100, 100000)) is None
