@@ -8,7 +8,7 @@ from pathlib import Path
 import torch
 
 sys.path.insert(0, str(Path(__file__).resolve().parents[1]))
-import kermac_amd as kermac  # noqa: E402
+import kermac  # noqa: E402
 
 device = torch.device("cuda")
 data = torch.randn(10000, 6, device=device)
@@ -18,7 +18,7 @@ laplace_l2 = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType
 out = kermac.run_kernel(laplace_l2, data, data, bandwidth=torch.tensor([10.0, 20.0], device=device),
                         regularization=10.0, regularization_offset_x=3, regularization_offset_y=1)
 print(out.shape)            # [2, 10000, 10000]: one kernel matrix per bandwidth
-print(out[:, :5, :5])       # elements with 3 + m == 1 + n hold 1 + 10
+print(out[:, :5, :5])       # elements [m, n] with 3 + n == 1 + m hold 1 + 10 (as in the reference for out=None)
 
 laplace_p = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.POW, kermac.PowerType.POW,
                                     kermac.KernelType.LAPLACE)

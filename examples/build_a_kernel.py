@@ -11,7 +11,7 @@ from pathlib import Path
 import torch
 
 sys.path.insert(0, str(Path(__file__).resolve().parents[1]))
-import kermac_amd as kermac  # noqa: E402
+import kermac  # noqa: E402
 
 
 def main():
@@ -19,7 +19,9 @@ def main():
     ap.add_argument("-m", "--M", type=int, default=4000)
     ap.add_argument("-n", "--N", type=int, default=3000)
     ap.add_argument("-k", "--K", type=int, default=64)
+    ap.add_argument("-a", "--try_align", action="store_true", help="accepted for compatibility (alignment is automatic)")
     ap.add_argument("-d", "--debug", action="store_true")
+    ap.add_argument("-s", "--skip_torch", action="store_true", help="run the kernels without the torch comparisons")
     args = ap.parse_args()
     device = torch.device("cuda")
     a = torch.randn(args.M, args.K, device=device)
@@ -35,34 +37,47 @@ def main():
     kermac.pre_compile_descriptors(device, [kermac.kernel_descriptor_l1_norm, sqrt_sum, gaussian_p], debug=args.debug)
 
     def show(title, value, expected):
-        err = (value - expected).abs().max().item()
-        print(f"{title:42s} max abs difference to torch {err:.2e}")
+        """`expected` is a function so that --skip_torch really skips the torch side."""
+        if args.skip_torch:
+            print(f"{title:42s} result {tuple(value.shape)}")
+            return
+        truth = expected()
+        err = (value - truth).abs().max().item()
+        print(f"{title:42s} max abs difference to torch {err:.2e}   relative to max |torch| {err / truth.abs().max().item():.2e}")
 
-    d1, d2 = torch.cdist(a, b, p=1.0), torch.cdist(a, b, p=2.0)
+    def d1():
+        return torch.cdist(a, b, p=1.0)
+
+    def d2():
+        return torch.cdist(a, b, p=2.0)
+
+    align = dict(try_to_align=args.try_align)
     show("laplace, L2 distance, bandwidth 10",
-         kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, a, b, out=out, bandwidth=10.0, epsilon=1e-5),
-         torch.exp(-d2 / 10.0))
+         kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, a, b, out=out, bandwidth=10.0, epsilon=1e-5, **align),
+         lambda: torch.exp(-d2() / 10.0))
     show("laplace, L1 distance, bandwidth 10",
-         kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, out=out, bandwidth=10.0), torch.exp(-d1 / 10.0))
-    show("L1 norm", kermac.run_kernel(kermac.kernel_descriptor_l1_norm, a, b, out=out), d1)
-    show("L2 norm", kermac.run_kernel(kermac.kernel_descriptor_l2_norm, a, b, out=out), d2)
+         kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, out=out, bandwidth=10.0, **align),
+         lambda: torch.exp(-d1() / 10.0))
+    show("L1 norm", kermac.run_kernel(kermac.kernel_descriptor_l1_norm, a, b, out=out, **align), d1)
+    show("L2 norm", kermac.run_kernel(kermac.kernel_descriptor_l2_norm, a, b, out=out, **align), d2)
     # the Gaussian function is applied to whatever the outer power yields: here the 1.3-norm itself
     show("gaussian of the 1.3-norm, bandwidth 10",
-         kermac.run_kernel(gaussian_p, a, b, out=out, inner_p=1.3, outer_p=1.0 / 1.3, bandwidth=10.0),
-         torch.exp(-torch.cdist(a, b, p=1.3) / 200.0))
-    show("plain a @ b.T", kermac.run_kernel(kermac.kernel_descriptor_mma, a, b, out=out), a @ b.T)
-    show("sum_k sqrt(a b) (run-time compiled)", kermac.run_kernel(sqrt_sum, a.abs(), b.abs(), out=out),
-         (a.abs()[:, None, :] * b.abs()[None, :, :]).sqrt().sum(-1) if args.M * args.N * args.K < 2e9 else out)
+         kermac.run_kernel(gaussian_p, a, b, out=out, inner_p=1.3, outer_p=1.0 / 1.3, bandwidth=10.0, **align),
+         lambda: torch.exp(-torch.cdist(a, b, p=1.3) / 200.0))
+    show("plain a @ b.T", kermac.run_kernel(kermac.kernel_descriptor_mma, a, b, out=out, **align), lambda: a @ b.T)
+    if args.M * args.N * args.K < 2e9:
+        show("sum_k sqrt(a b) (run-time compiled)", kermac.run_kernel(sqrt_sum, a.abs(), b.abs(), out=out, **align),
+             lambda: (a.abs()[:, None, :] * b.abs()[None, :, :]).sqrt().sum(-1))
 
     # per-batch hyper-parameters: 4 kernels in one launch
     p = torch.tensor([0.5, 1.0, 1.5, 2.0], device=device)
     batched = kermac.run_kernel(kermac.kernel_descriptor_p_norm, a, b, p=p)
-    show("4 p-norms in one launch", batched, torch.stack([torch.cdist(a, b, p=float(x)) for x in p]))
+    show("4 p-norms in one launch", batched, lambda: torch.stack([torch.cdist(a, b, p=float(x)) for x in p]))
 
     # fused contraction: the M x N kernel matrix is never stored
     coef = torch.randn(args.N, 8, device=device)
     fused = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, bandwidth=10.0, coefficients=coef)
-    show("laplace-L1 kernel matrix @ coefficients", fused[0], torch.exp(-d1 / 10.0) @ coef)
+    show("laplace-L1 kernel matrix @ coefficients", fused[0], lambda: torch.exp(-d1() / 10.0) @ coef)
 
 
 if __name__ == "__main__":

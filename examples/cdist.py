@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Time kermac_amd.cdist against torch.cdist on one MI355X.
+"""Time kermac.cdist against torch.cdist on one MI355X.
 
 Same switches as the reference's examples/cdist.py, so its README table can be
 reproduced one-for-one:
@@ -16,7 +16,7 @@ from pathlib import Path
 import torch
 
 sys.path.insert(0, str(Path(__file__).resolve().parents[1]))
-import kermac_amd as kermac  # noqa: E402
+import kermac  # noqa: E402
 
 
 def parse_args():
@@ -30,7 +30,7 @@ def parse_args():
     ap.add_argument("-a", "--try_align", action="store_true", help="accepted for compatibility (alignment is automatic)")
     ap.add_argument("-d", "--debug", action="store_true", help="print what is launched")
     ap.add_argument("-t", "--transposes", type=str, default=None, help="three of 'n'/'t' for a, b, out")
-    ap.add_argument("--l2_mode", choices=["direct", "gram"], default="direct", help="evaluation of p = 2 (see set_l2_mode)")
+    ap.add_argument("--l2_mode", choices=["direct", "gram", "gram_bf16"], default="direct", help="evaluation of p = 2 (see set_l2_mode)")
     ap.add_argument("--skip_numeric_compare", action="store_true", help="do not compare with torch.cdist")
     ap.add_argument("--skip_torch", action="store_true", help="do not run torch.cdist at all")
     ap.add_argument("--warmup", type=int, default=2)
@@ -70,7 +70,7 @@ def main():
     ms = timer.stop() / args.iters
     ops = 3.0 * args.L * args.M * args.N * args.K
     print(f"p={args.p} ({args.L},{args.M},{args.K}) x ({args.L},{args.N},{args.K})")
-    print(f"\tkermac_amd.cdist\t{ms:.3f} ms / iteration\t{ops / ms / 1e9:.1f} TFLOP/s (3 ops per m,n,k)")
+    print(f"\tkermac.cdist\t\t{ms:.3f} ms / iteration\t{ops / ms / 1e9:.1f} TFLOP/s (3 ops per m,n,k)")
     if args.skip_torch:
         return
     for _ in range(args.warmup):
@@ -93,7 +93,7 @@ def main():
     truth = torch.cdist(a[l, ms].double(), b[l, ns].double(), p=args.p)
     if args.skip_epilogue:
         truth = truth ** args.p
-    for name, value in (("kermac_amd", result), ("torch fp32", reference)):
+    for name, value in (("kermac", result), ("torch fp32", reference)):
         rel = ((value[l, ms, ns].double() - truth).abs() / truth.abs().clamp_min(1e-30)).max().item()
         print(f"\t{name} vs float64 torch.cdist on a 512 x 512 slab: max rel err {rel:.3e}")
 

@@ -51,9 +51,12 @@ enum kmc_flags {
     /* Use the 32-bit loaders/stores even when the operands are 16-byte aligned
      * (what the reference does without try_to_align). */
     KMC_FLAG_FORCE_SCALAR_ACCESS = 1,
-    /* Compute A(m,k) - B(n,k) instead of B(n,k) - A(m,k).  Set by callers that
-     * swapped the operands to obtain a row-major result; only matters for the
-     * sign-sensitive inner powers (NOOP, SQRT). */
+    /* Compute A(m,k) - B(n,k) instead of B(n,k) - A(m,k); only matters for the
+     * sign-sensitive inner powers (NOOP, SQRT).  The reference's run_kernel hands its
+     * operands over exchanged whenever the result is row-major (its default,
+     * src/kermac/build_a_kernel.py:259,323-336), so what its callers see there is
+     * first operand minus second; a caller that launches without that exchange sets
+     * this flag (and exchanges the regularisation offsets) to get the same values. */
     KMC_FLAG_NEGATE_DIFF = 2,
     /* Only for inner_operator DIFF + inner_power SQUARE: compute the sum of squared
      * differences as |a|^2 + |b|^2 - 2 a.b with the cross term on the matrix cores

@@ -13,8 +13,10 @@ View convention (torch.cdist's): ``a`` is ``[L?, M, K]``, ``b`` is ``[L?, N, K]`
 """
 from __future__ import annotations
 
+import contextlib
 import functools
 import os
+import threading
 from enum import Enum, auto
 from itertools import product
 from typing import Any, List, Optional, Union
@@ -70,7 +72,7 @@ class KernelDescriptor:
     """What the fused kernel computes per output element
     (reference: build_a_kernel.py:39-71):
 
-    ``kernel_type( outer_power( sum_k inner_power( b[n,k] (-|*) a[m,k] ) ) )``
+    ``kernel_type( outer_power( sum_k inner_power( a[m,k] (-|*) b[n,k] ) ) )``
     """
 
     def __init__(self, inner_operator, inner_power, outer_power, kernel_type):
@@ -196,13 +198,34 @@ def _hyper_parameter(name, value, L, device, require_device):
 #   launches are bound by the result stores, and the direct kernel has the cheaper
 #   epilogue and no repair launch (M = N = 30000, K = 16: 1.2 ms against 2.4 .. 2.6 ms).
 _L2_DEFAULT_MIN_K = 64
-_l2_mode = {"mode": os.environ.get("KERMAC_AMD_L2_MODE", "direct"), "trust": None, "min_k": _L2_DEFAULT_MIN_K}
+_L2_MODES = ("direct", "gram", "gram_bf16")
+# The process-wide setting, and per host thread what `l2_mode(...)` blocks have put on top
+# of it: two threads can evaluate squared differences in different modes at the same time.
+_l2_process = {"mode": os.environ.get("KERMAC_AMD_L2_MODE", "direct"), "trust": None, "min_k": _L2_DEFAULT_MIN_K}
+_l2_thread = threading.local()
+
+
+def _l2_setting(mode, trust, min_k):
+    if mode not in _L2_MODES:
+        raise ValueError(f"l2 mode must be 'direct', 'gram' or 'gram_bf16', got {mode!r}")
+    if trust is not None and not trust > 0.0:
+        raise ValueError("trust must be positive")
+    if min_k is not None and min_k < 0:
+        raise ValueError("min_k must not be negative")
+    return {"mode": mode, "trust": trust, "min_k": _L2_DEFAULT_MIN_K if min_k is None else int(min_k)}
+
+
+def _l2_current():
+    stack = getattr(_l2_thread, "stack", None)
+    return stack[-1] if stack else _l2_process
 
 
 def set_l2_mode(mode: str, trust: Optional[float] = None, min_k: Optional[int] = None) -> None:
-    """Choose how squared-difference descriptors are evaluated: ``"direct"`` (default),
-    ``"gram"`` (fp32 matrix cores + automatic repair of ill-conditioned tiles) or
-    ``"gram_bf16"`` (the same on the bf16 matrix instruction, three bf16 pieces per operand).
+    """Choose, for the whole process, how squared-difference descriptors are evaluated:
+    ``"direct"`` (default), ``"gram"`` (fp32 matrix cores + automatic repair of
+    ill-conditioned tiles) or ``"gram_bf16"`` (the same on the bf16 matrix instruction,
+    three bf16 pieces per operand).  A thread inside an ``l2_mode(...)`` block keeps the
+    mode of its block.
 
     ``trust`` (gram modes) is the fraction of ``|a|^2 + |b|^2`` below which a squared
     distance is recomputed directly.  The default keeps the relative error of the
@@ -210,23 +233,33 @@ def set_l2_mode(mode: str, trust: Optional[float] = None, min_k: Optional[int] =
     ``min_k`` (gram modes, default 64): contractions shorter than this use the direct
     kernel, which is the faster one there.
     """
-    if mode not in ("direct", "gram", "gram_bf16"):
-        raise ValueError(f"l2 mode must be 'direct', 'gram' or 'gram_bf16', got {mode!r}")
-    if trust is not None and not trust > 0.0:
-        raise ValueError("trust must be positive")
-    if min_k is not None and min_k < 0:
-        raise ValueError("min_k must not be negative")
-    _l2_mode["mode"], _l2_mode["trust"] = mode, trust
-    _l2_mode["min_k"] = _L2_DEFAULT_MIN_K if min_k is None else int(min_k)
+    _l2_process.update(_l2_setting(mode, trust, min_k))
+
+
+@contextlib.contextmanager
+def l2_mode(mode: str, trust: Optional[float] = None, min_k: Optional[int] = None):
+    """``with kermac.l2_mode("gram"): ...`` evaluates squared-difference descriptors in
+    ``mode`` for the calls the current host thread makes inside the block; other threads
+    and the process-wide setting (``set_l2_mode``) are not affected.  Arguments as for
+    ``set_l2_mode``; blocks nest."""
+    setting = _l2_setting(mode, trust, min_k)
+    stack = getattr(_l2_thread, "stack", None)
+    if stack is None:
+        stack = _l2_thread.stack = []
+    stack.append(setting)
+    try:
+        yield
+    finally:
+        stack.pop()
 
 
 def get_l2_mode() -> str:
-    return _l2_mode["mode"]
+    return _l2_current()["mode"]
 
 
-def _gram_trust(K: int) -> float:
-    if _l2_mode["trust"] is not None:
-        return float(_l2_mode["trust"])
+def _gram_trust(K: int, setting) -> float:
+    if setting["trust"] is not None:
+        return float(setting["trust"])
     return max(0.25, (K ** 0.5) * 2.0 ** -24 / 8e-6)
 
 
@@ -347,15 +380,21 @@ def _plan_run_kernel(
     keepalive += [pi_keep, po_keep, bw_keep, rg_keep]
 
     # The kernel writes C with m contiguous.  A row-major out is the transpose of
-    # that, so swap the operands (reference: :323-336).  Unlike the reference the
-    # swap also exchanges the regularisation offsets and keeps the sign of b - a,
-    # so the result does not depend on the layout of `out`.
+    # that, so swap the operands (reference: :323-336).  The reference swaps neither the
+    # regularisation offsets nor the sign of a signed inner term, so there the result
+    # depends on the layout of `out`.  Here it does not: every layout gives what the
+    # reference returns for `out=None` (a row-major result, the case all of its users
+    # see): the inner difference is a[m] - b[n] and the regularised elements are those
+    # with offset_x + n == offset_y + m.  The kernel itself computes B - A and tests
+    # offset_x + (row of A) == offset_y + (row of B), so the swapped launch passes
+    # through as it is and the unswapped one exchanges the offsets and negates.
     swapped = stats_c is not None and stats_c.majorness is Majorness.ROW_MAJOR
     off_x, off_y = int(regularization_offset_x), int(regularization_offset_y)
     if swapped:
         M, N = N, M
         a, b = b, a
         stats_a, stats_b = stats_b, stats_a
+    else:
         off_x, off_y = off_y, off_x
 
     params = _backend.BuildKernelParams()
@@ -365,18 +404,19 @@ def _plan_run_kernel(
     params.kernel_type = _KERNEL_TYPE_ABI[d._kernel_type]
     params.a_majorness = _MAJORNESS_ABI[stats_a.majorness]
     params.b_majorness = _MAJORNESS_ABI[stats_b.majorness]
-    params.flags = _backend.FLAG_NEGATE_DIFF if swapped else 0
+    params.flags = 0 if swapped else _backend.FLAG_NEGATE_DIFF
     if os.environ.get("KERMAC_AMD_NO_SYMMETRY", "0") not in ("", "0"):
         # the library computes x-against-x matrices from the tiles on and below the diagonal
         # (bit-identical result, about half the time); this keeps it to the full computation
         params.flags |= _backend.FLAG_NO_SYMMETRY
-    if (_l2_mode["mode"] in ("gram", "gram_bf16") and d._inner_operator is InnerOperator.DIFF
-            and d._inner_power is PowerType.SQUARE and K >= _l2_mode["min_k"]):
+    l2 = _l2_current()
+    if (l2["mode"] in ("gram", "gram_bf16") and d._inner_operator is InnerOperator.DIFF
+            and d._inner_power is PowerType.SQUARE and K >= l2["min_k"]):
         # also for the fused coefficient product (no out matrix here): it has a matrix-core variant too
         params.flags |= _backend.FLAG_L2_GRAM
-        if _l2_mode["mode"] == "gram_bf16":
+        if l2["mode"] == "gram_bf16":
             params.flags |= _backend.FLAG_L2_GRAM_BF16
-        params.gram_trust = _gram_trust(K)
+        params.gram_trust = _gram_trust(K, l2)
     params.m, params.n, params.k, params.l = M, N, K, L
     params.a, params.a_ld, params.a_bs = a.data_ptr(), stats_a.leading_dimension_stride, stats_a.batch_stride
     params.b, params.b_ld, params.b_bs = b.data_ptr(), stats_b.leading_dimension_stride, stats_b.batch_stride
@@ -430,12 +470,18 @@ def run_kernel(
 ):
     """Fused pairwise kernel matrix (reference: build_a_kernel.py:158-394).
 
-    ``out[l, m, n] = kernel_type(outer_power(sum_k inner_power(b[l,n,k] (-|*) a[l,m,k])))``
+    ``out[l, m, n] = kernel_type(outer_power(sum_k inner_power(a[l,m,k] (-|*) b[l,n,k])))``
     followed, for Laplace/Gaussian kernels with a non-zero ``regularization``,
-    by replacing every element with ``offset_x + m == offset_y + n`` by
+    by replacing every element with ``offset_x + n == offset_y + m`` by
     ``1 + regularization``.  ``a``, ``b``, ``out`` and the hyper-parameter
     tensors may each carry a leading batch dimension of 1 or L; a missing batch
-    broadcasts.  Returns ``out`` (allocated as zeros ``[L, M, N]`` when None).
+    broadcasts.  Returns ``out`` (allocated ``[L, M, N]`` when None).
+
+    The sign of the difference (it matters for the inner powers NOOP and SQRT only)
+    and the side each offset belongs to are those of the reference's result for
+    ``out=None``; the reference gives the mirrored convention when it is handed a
+    column-major ``out`` (it swaps the operands but not the offsets or the sign,
+    build_a_kernel.py:323-336), here the result is the same for every layout of ``out``.
 
     ``try_to_align`` is accepted for signature compatibility: 128-bit accesses
     are used whenever pointer, leading dimension and batch stride allow them.

@@ -218,7 +218,6 @@ int kmc_build_kernel_finish(const kmc_build_kernel_params *params, const float *
         return fail(KMC_ERR_INVALID_ARGUMENT, "partials: leading dimension %lld is smaller than m=%d",
                     static_cast<long long>(partial_ld), args.m);
     if (partial_ld < 0 || partial_bs < 0 || partial_slice < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "partials: negative stride");
-    if (args.n > 65535 || args.l > 65535) return fail(KMC_ERR_INVALID_ARGUMENT, "n=%d or l=%d exceeds 65535", args.n, args.l);
     status = require_gfx950();
     if (status != KMC_OK) return status;
     const int vec = args.c_vec && aligned16(partials) && partial_ld % 4 == 0 && partial_bs % 4 == 0 && partial_slice % 4 == 0;

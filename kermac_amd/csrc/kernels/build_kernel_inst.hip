@@ -3,6 +3,7 @@
 // Compiled several times with different -DKMC_INNER_OP / -DKMC_INNER_POW.
 #include <hip/hip_runtime.h>
 
+#include "launch.hpp"
 #include "build_kernel.hpp"
 
 #ifndef KMC_INNER_OP
@@ -18,9 +19,7 @@ namespace kmc_host {
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)
 {
-    hipLaunchKernelGGL((kmc::build_kernel<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>), grid,
-                       dim3(kmc::BK_THREADS), 0, stream, args);
-    return hipGetLastError();
+    return launch(kmc::build_kernel<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
 }
 
 hipError_t KMC_LAUNCHER_NAME(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)

@@ -8,6 +8,7 @@
 // group order: a fixed order for a given shape, so results repeat bit for bit).
 #include <hip/hip_runtime.h>
 
+#include "launch.hpp"
 #include "build_kernel.hpp"
 
 namespace kmc {
@@ -22,12 +23,11 @@ struct FinishArgs {
     int groups;                 // lane groups that share the slices of one quad of m
 };
 
-__global__ __launch_bounds__(256) void finish_partials(const FinishArgs fa)
+// One row n of the result for this workgroup's lanes.
+__device__ __forceinline__ void finish_row(const FinishArgs &fa, float4 *group_sums, int batch, int n, float p_outer,
+                                           float neg_gamma, float regularization)
 {
     const BuildKernelArgs &args = fa.kernel;
-    __shared__ float4 group_sums[256];
-    const int batch = blockIdx.z;
-    const int n = blockIdx.y;
     const int quad = threadIdx.x & (fa.quad_lanes - 1);
     const int group = threadIdx.x / fa.quad_lanes;
     const int m = (blockIdx.x * fa.quad_lanes + quad) * 4;
@@ -65,19 +65,12 @@ __global__ __launch_bounds__(256) void finish_partials(const FinishArgs fa)
                 sum[0] += v.x; sum[1] += v.y; sum[2] += v.z; sum[3] += v.w;
             }
         }
+        __syncthreads();   // the next row of this workgroup writes group_sums again
     }
     if (!live || group != 0) return;
 
     const int outer_power = args.outer_power;
     const int kernel_type = args.kernel_type;
-    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
-    if (outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
-    if (kernel_type != KERNEL_NONE) {
-        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
-        neg_gamma = kernel_neg_gamma(kernel_type, bw);
-        regularization = args.regularization ? args.regularization[batch * args.regularization_bs]
-                                             : args.regularization_value;
-    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         sum[i] = epilogue_value(sum[i], outer_power, kernel_type, p_outer, neg_gamma, args.epsilon);
@@ -93,6 +86,24 @@ __global__ __launch_bounds__(256) void finish_partials(const FinishArgs fa)
         for (int i = 0; i < 4; i++)
             if (i < valid) dst[i] = sum[i];
     }
+}
+
+// Grid: x = blocks of lanes along m, y = rows n (a workgroup strides over n by the grid
+// height, so n may exceed the 65535 a grid dimension can hold), z = batch.
+__global__ __launch_bounds__(256) void finish_partials(const FinishArgs fa)
+{
+    const BuildKernelArgs &args = fa.kernel;
+    __shared__ float4 group_sums[256];
+    const int batch = blockIdx.z;
+    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
+    if (args.outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
+    if (args.kernel_type != KERNEL_NONE) {
+        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
+        neg_gamma = kernel_neg_gamma(args.kernel_type, bw);
+        regularization = args.regularization ? args.regularization[batch * args.regularization_bs]
+                                             : args.regularization_value;
+    }
+    for (int n = blockIdx.y; n < args.n; n += gridDim.y) finish_row(fa, group_sums, batch, n, p_outer, neg_gamma, regularization);
 }
 
 }  // namespace kmc
@@ -113,9 +124,8 @@ hipError_t launch_finish_partials(const kmc::BuildKernelArgs &kernel, const floa
     fa.quad_lanes = 256;
     while (fa.quad_lanes > 1 && fa.quad_lanes / 2 >= quads && slices >= 8 * (512 / fa.quad_lanes)) fa.quad_lanes /= 2;
     fa.groups = 256 / fa.quad_lanes;
-    const dim3 grid((quads + fa.quad_lanes - 1) / fa.quad_lanes, kernel.n, kernel.l);
-    hipLaunchKernelGGL(kmc::finish_partials, grid, dim3(256), 0, stream, fa);
-    return hipGetLastError();
+    const dim3 grid((quads + fa.quad_lanes - 1) / fa.quad_lanes, kernel.n < 65535 ? kernel.n : 65535, kernel.l);
+    return launch(kmc::finish_partials, grid, dim3(256), stream, fa);
 }
 
 }  // namespace kmc_host

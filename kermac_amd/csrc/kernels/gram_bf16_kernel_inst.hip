@@ -2,6 +2,7 @@
 // (A loader, B loader) pairs, plus the ragged-K variants of the pairs with 128-bit row-major loads.
 #include <hip/hip_runtime.h>
 
+#include "launch.hpp"
 #include "gram_bf16_kernel.hpp"
 
 namespace kmc_host {
@@ -10,13 +11,13 @@ template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)
 {
     constexpr bool has_ragged_variant = LOAD_A == kmc::LOAD_ROW_VEC || LOAD_B == kmc::LOAD_ROW_VEC;
+    hipError_t status;
     if (has_ragged_variant && args.k % kmc::BK_TILE_K != 0) {
-        hipLaunchKernelGGL((kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B, has_ragged_variant>), grid, dim3(kmc::BK_THREADS), 0,
-                           stream, args);
+        status = launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B, has_ragged_variant>, grid, dim3(kmc::BK_THREADS), stream, args);
     } else {
-        hipLaunchKernelGGL((kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B>), grid, dim3(kmc::BK_THREADS), 0, stream, args);
+        status = launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
     }
-    return hipGetLastError();
+    return status;
 }
 
 hipError_t launch_gram_bf16_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)

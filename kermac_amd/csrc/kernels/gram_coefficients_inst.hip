@@ -2,6 +2,7 @@
 // coefficients kernel for all 16 (A loader, B loader) pairs.
 #include <hip/hip_runtime.h>
 
+#include "launch.hpp"
 #include "gram_coefficients.hpp"
 
 namespace kmc_host {
@@ -9,8 +10,7 @@ namespace kmc_host {
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::KernelCoefficientsArgs &args, dim3 grid, hipStream_t stream)
 {
-    hipLaunchKernelGGL((kmc::gram_times_coefficients<LOAD_A, LOAD_B>), grid, dim3(kmc::BK_THREADS), 0, stream, args);
-    return hipGetLastError();
+    return launch(kmc::gram_times_coefficients<LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
 }
 
 hipError_t launch_gram_coefficients(int load_a, int load_b, const kmc::KernelCoefficientsArgs &args, dim3 grid,

@@ -4,6 +4,7 @@
 // Compiled several times with different -DKMC_INNER_OP / -DKMC_INNER_POW.
 #include <hip/hip_runtime.h>
 
+#include "launch.hpp"
 #include "kernel_coefficients.hpp"
 
 #ifndef KMC_INNER_OP
@@ -19,16 +20,15 @@ namespace kmc_host {
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::KernelCoefficientsArgs &args, dim3 grid, hipStream_t stream)
 {
+    hipError_t status;
     if (args.columns == 64) {
-        hipLaunchKernelGGL((kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B, 64>), grid,
-                           dim3(kmc::BK_THREADS), 0, stream, args);
+        status = launch(kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B, 64>, grid, dim3(kmc::BK_THREADS), stream, args);
     } else if (args.columns == kmc::KC_COLUMNS) {
-        hipLaunchKernelGGL((kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>), grid,
-                           dim3(kmc::BK_THREADS), 0, stream, args);
+        status = launch(kmc::kernel_times_coefficients<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
     } else {
         return hipErrorInvalidValue;
     }
-    return hipGetLastError();
+    return status;
 }
 
 hipError_t KMC_LAUNCHER_NAME(int load_a, int load_b, const kmc::KernelCoefficientsArgs &args, dim3 grid,

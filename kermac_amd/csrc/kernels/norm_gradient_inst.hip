@@ -3,6 +3,7 @@
 // 16 or 32 output columns, with and without a partial last K slice).
 #include <hip/hip_runtime.h>
 
+#include "launch.hpp"
 #include "norm_gradient_mfma.hpp"
 
 namespace kmc_host {
@@ -12,25 +13,26 @@ static hipError_t launch_norm(int o_tile, const kmc::NormGradientArgs &args, dim
 {
     const dim3 block(kmc::NG_THREADS);
     const bool k_tail = args.k % kmc::NGM_TILE_K != 0;
+    hipError_t status;
     switch (o_tile) {
-    case 1: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 1>), grid, block, 0, stream, args); break;
-    case 2: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 2>), grid, block, 0, stream, args); break;
-    case 3: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 3>), grid, block, 0, stream, args); break;
-    case 4: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 4>), grid, block, 0, stream, args); break;
-    case 5: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 5>), grid, block, 0, stream, args); break;
-    case 6: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 6>), grid, block, 0, stream, args); break;
-    case 8: hipLaunchKernelGGL((kmc::norm_kernel_gradient<NORM, 8>), grid, block, 0, stream, args); break;
+    case 1: status = launch(kmc::norm_kernel_gradient<NORM, 1>, grid, block, stream, args); break;
+    case 2: status = launch(kmc::norm_kernel_gradient<NORM, 2>, grid, block, stream, args); break;
+    case 3: status = launch(kmc::norm_kernel_gradient<NORM, 3>, grid, block, stream, args); break;
+    case 4: status = launch(kmc::norm_kernel_gradient<NORM, 4>, grid, block, stream, args); break;
+    case 5: status = launch(kmc::norm_kernel_gradient<NORM, 5>, grid, block, stream, args); break;
+    case 6: status = launch(kmc::norm_kernel_gradient<NORM, 6>, grid, block, stream, args); break;
+    case 8: status = launch(kmc::norm_kernel_gradient<NORM, 8>, grid, block, stream, args); break;
     case 16:
-        if (k_tail) hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 1, true>), grid, block, 0, stream, args);
-        else hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 1, false>), grid, block, 0, stream, args);
+        if (k_tail) status = launch(kmc::norm_kernel_gradient_mfma<NORM, 1, true>, grid, block, stream, args);
+        else status = launch(kmc::norm_kernel_gradient_mfma<NORM, 1, false>, grid, block, stream, args);
         break;
     case 32:
-        if (k_tail) hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 2, true>), grid, block, 0, stream, args);
-        else hipLaunchKernelGGL((kmc::norm_kernel_gradient_mfma<NORM, 2, false>), grid, block, 0, stream, args);
+        if (k_tail) status = launch(kmc::norm_kernel_gradient_mfma<NORM, 2, true>, grid, block, stream, args);
+        else status = launch(kmc::norm_kernel_gradient_mfma<NORM, 2, false>, grid, block, stream, args);
         break;
     default: return hipErrorInvalidValue;
     }
-    return hipGetLastError();
+    return status;
 }
 
 hipError_t launch_norm_gradient(int norm_type, int o_tile, const kmc::NormGradientArgs &args, dim3 grid,

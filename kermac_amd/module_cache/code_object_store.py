@@ -111,7 +111,17 @@ class CodeObjectStore:
         return code_hash
 
     def get_code(self, code_hash: str) -> Optional[bytes]:
+        """The stored code object, or None when it is missing or its bytes no longer
+        hash to its name (a truncated or edited file): the caller then recompiles."""
+        path = self.dir / f"code-{code_hash}.hsaco"
         try:
-            return (self.dir / f"code-{code_hash}.hsaco").read_bytes()
+            code = path.read_bytes()
         except OSError:
             return None
+        if hashlib.sha256(code).hexdigest() != code_hash:
+            try:
+                path.unlink()
+            except OSError:
+                pass
+            return None
+        return code

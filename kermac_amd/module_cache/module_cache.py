@@ -158,7 +158,19 @@ class ModuleCache(metaclass=Singleton):
             if module is None:
                 code = self._store.get_code(code_hash)
                 if code is None:
-                    raise RuntimeError(f"kernel cache has no code object {code_hash}")
+                    # the stored file vanished or failed its hash check (the store has dropped it):
+                    # compile again; other functions of the lost program follow when they are asked for
+                    if debug:
+                        print(f"(Kermac Debug) Code object {code_hash} is unusable, compiling {function_name} again")
+                    self.compile_and_cache_functions(device, [function_name], debug=debug)
+                    mapping = self._store.get_function_mapping(key)
+                    if mapping is None:
+                        raise RuntimeError(f"kernel cache lost the entry for {function_name} right after compiling it")
+                    lowered_name, code_hash = mapping
+                    module_key = (device_id, code_hash)
+                    code = self._store.get_code(code_hash)
+                    if code is None:
+                        raise RuntimeError(f"kernel cache has no code object {code_hash}")
                 with torch.cuda.device(device_id):
                     module = _backend.module_load(code)
                 self._loaded_modules[module_key] = module

@@ -105,6 +105,27 @@ def build_kernel(inner_operator, inner_power, outer_power, kernel_type, a, b,
     return out
 
 
+def run_kernel(inner_operator, inner_power, outer_power, kernel_type, a, b, **kw):
+    """out[L, M, N] as the reference's ``run_kernel`` returns it for ``out=None``
+    (src/kermac/build_a_kernel.py:259 allocates a row-major ``[L, M, N]``; :323-336 then
+    swap the operands, but neither the regularisation offsets nor the sign of the
+    difference, before the kernel of ``build_kernel`` runs and writes the transpose):
+    the inner difference is ``a[m] - b[n]`` and the regularised elements are those with
+    ``offset_x + n == offset_y + m``.  For the inner powers that ignore the sign and
+    with equal offsets this is ``build_kernel(a, b)`` itself."""
+    return build_kernel(inner_operator, inner_power, outer_power, kernel_type, b, a, **kw).transpose(-1, -2)
+
+
+def run_kernel_coefficients(inner_operator, inner_power, outer_power, kernel_type, a, b, coef,
+                            regularization_offset_x=0, regularization_offset_y=0, **kw):
+    """out[L, M, O] = run_kernel(...)[L, M, N] @ coef[L?, N, O] without the matrix, in the
+    convention of ``run_kernel`` above: negating both operands turns the kernel's b - a
+    into a - b (and leaves products unchanged), and the offsets change sides."""
+    return kernel_times_coefficients(inner_operator, inner_power, outer_power, kernel_type, -a, -b, coef,
+                                     regularization_offset_x=regularization_offset_y,
+                                     regularization_offset_y=regularization_offset_x, **kw)
+
+
 def cdist(a, b, p=2.0, skip_epilogue=False, wide=True):
     """What kermac.cdist documents: (sum_k |b - a|^p)^(1/p), or the bare sum."""
     if p == 1.0:

@@ -173,8 +173,13 @@ def test_run_kernel_golden_kernel_functions(device):
         out = out.t() if c_col else out
         got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, x, out=out, bandwidth=3.0, regularization=0.25,
                                 regularization_offset_x=3, regularization_offset_y=1)
-        assert_close_to_truth(got, torch.from_numpy(GOLDEN["laplace_l1_self_bw3_reg0.25_off3_1"]), rtol=1e-5,
+        # The reference's examples/broadcast_kernel.py passes offsets (3, 1) with out=None: its
+        # row-major result has 1 + regularization where 3 + n == 1 + m, i.e. at [n + 2, n], below
+        # the diagonal (the golden vector holds the kernel-level position [m, m + 2]; x against
+        # x is symmetric elsewhere, so the expected matrix is its transpose).  Same for every out.
+        assert_close_to_truth(got, torch.from_numpy(GOLDEN["laplace_l1_self_bw3_reg0.25_off3_1"]).t(), rtol=1e-5,
                               what=f"offset diagonal, out col-major={c_col}")
+        assert got[0, 2, 0].item() == 1.25 and got[0, 0, 2].item() < 1.0
 
 
 def test_run_kernel_batched_hyper_parameters(device):
@@ -196,8 +201,8 @@ def test_run_kernel_batched_hyper_parameters(device):
     bw2 = torch.tensor([10.0, 20.0], device=device)
     out = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, data, data, bandwidth=bw2, regularization=10.0,
                             regularization_offset_x=3, regularization_offset_y=1)
-    truth = oracle.build_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", data.cpu(), data.cpu(), bandwidth=bw2.cpu(),
-                                regularization=10.0, regularization_offset_x=3, regularization_offset_y=1)
+    truth = oracle.run_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", data.cpu(), data.cpu(), bandwidth=bw2.cpu(),
+                              regularization=10.0, regularization_offset_x=3, regularization_offset_y=1)
     assert out.shape == (2, N, N)
     assert_close_to_truth(out, truth, rtol=1e-5, what="per-batch bandwidth, offset diagonal")
     # independent inner / outer powers (examples/build_a_kernel.py: Gaussian p-norm)
@@ -249,16 +254,41 @@ def test_run_kernel_epsilon_mask(device):
 
 
 def test_signed_inner_operator_with_row_major_out(device):
-    # DIFF + NOOP is sign sensitive; the operand swap for a row-major out must not flip it.
+    # DIFF + NOOP is sign sensitive: a[m] - b[n], what the reference returns for out=None
+    # (src/kermac/build_a_kernel.py:323-336 swap the operands in front of a kernel that
+    # computes B - A), here for every layout of out.
     g = torch.Generator().manual_seed(82)
     a, b = torch.randn(70, 9, generator=g).to(device), torch.randn(50, 9, generator=g).to(device)
     signed = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.NOOP, kermac.PowerType.NOOP,
                                      kermac.KernelType.NONE)
-    truth = (b.double()[None] - a.double()[:, None]).sum(-1).cpu()
+    truth = (a.double()[:, None] - b.double()[None]).sum(-1).cpu()
+    assert_close_to_truth(kermac.run_kernel(signed, a, b), truth, rtol=1e-5, atol=1e-5, what="signed diff, out=None")
     for c_col in (False, True):
         out = torch.empty(50, 70, device=device).t() if c_col else torch.empty(70, 50, device=device)
         got = kermac.run_kernel(signed, a, b, out=out)
         assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-5, what=f"signed diff, out col-major={c_col}")
+
+
+@pytest.mark.parametrize("l2_mode", ["direct", "gram", "gram_bf16"])
+def test_cdist_cpu_oracle_configuration(device, l2_mode):
+    """The reference's CPU-runnable case exactly: a_store[K=64, M=1024], b_store[64, N=1024]
+    ~ U(0,1) from torch.manual_seed(0), K-major panels, p = 2 with the square root, one
+    batch, out[N, M]; against the float64 oracle at rtol 1e-5 and against torch.cdist under
+    the reference test's criterion (tests/test_cdist.py:75-88), in every L2 mode."""
+    torch.manual_seed(0)
+    a_store = torch.rand(64, 1024)
+    b_store = torch.rand(64, 1024)
+    out_store = torch.empty(1024, 1024, device=device)
+    a, b = a_store.to(device).t(), b_store.to(device).t()
+    with kermac.l2_mode(l2_mode, min_k=0):
+        out = kermac.cdist(a, b, out=out_store.t(), p=2.0)
+    assert out.data_ptr() == out_store.data_ptr() and tuple(out.shape) == (1024, 1024)
+    truth = oracle.cdist(a_store.t(), b_store.t(), p=2.0)[0]
+    assert_close_to_truth(out, truth, rtol=1e-5, what=f"configs[0], l2 mode {l2_mode}")
+    assert_close_to_truth(out, torch.cdist(a_store.t().double(), b_store.t().double(), p=2.0), rtol=1e-5,
+                          what=f"configs[0] vs float64 torch.cdist, l2 mode {l2_mode}")
+    diff = out.cpu() - torch.cdist(a_store.t(), b_store.t(), p=2.0)
+    assert torch.sqrt(torch.mean(diff ** 2)).item() < 1e-4 and diff.abs().max().item() < 1e-4
 
 
 # ------------------------------------------------- full-size, size-independent checks
@@ -281,6 +311,16 @@ def test_cdist_full_size_properties(device, p):
     for ms, ns in ((slice(0, 300), slice(0, 2000)), (slice(29900, 30000), slice(29800, 30000))):
         truth = torch.cdist(a_store.t()[ms].double(), b_store.t()[ns].double(), p=p)
         assert_close_to_truth(out[ms, ns], truth, rtol=rtol_for(p), what=f"slab p={p}")
+    if p == 1.3:
+        # the same launch without the 1/p power (the reference raises here; its README
+        # documents the bare sum): float64 slabs of cdist ** p at the fractional tolerance
+        raw = kermac.cdist(a_store.t(), b_store.t(), out=out_store.t(), p=p, skip_epilogue=True)
+        assert raw.data_ptr() == out_store.data_ptr()
+        for ms, ns in ((slice(0, 300), slice(0, 2000)), (slice(29900, 30000), slice(29800, 30000)),
+                       (slice(14000, 14200), slice(7000, 7600))):
+            truth = torch.cdist(a_store.t()[ms].double(), b_store.t()[ns].double(), p=p) ** p
+            assert_close_to_truth(raw[ms, ns], truth, rtol=1e-4, what="slab p=1.3, skip_epilogue")
+        out = kermac.cdist(a_store.t(), b_store.t(), out=out_store.t(), p=p)
     # exchanging the operands transposes the result exactly (same sums, |b-a| = |a-b|)
     swapped = torch.empty(4000, 3000, device=device)
     kermac.cdist(b_store.t()[:3000], a_store.t()[:4000], out=swapped.t(), p=p)

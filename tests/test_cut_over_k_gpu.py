@@ -47,8 +47,8 @@ def test_kernels_regularised_diagonal_and_the_symmetric_shortcut(device):
     assert is_cut(kermac.kernel_descriptor_laplace_l1, x, x, bandwidth=40.0, regularization=0.25)
     got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, x, bandwidth=40.0, regularization=0.25,
                             regularization_offset_x=3, regularization_offset_y=0)
-    truth = oracle.build_kernel("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu(), x.cpu(), bandwidth=40.0, regularization=0.25,
-                                regularization_offset_x=3, regularization_offset_y=0)
+    truth = oracle.run_kernel("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu(), x.cpu(), bandwidth=40.0, regularization=0.25,
+                              regularization_offset_x=3, regularization_offset_y=0)
     assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-9, what="cut laplace with offset diagonal")
     plain = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, x, bandwidth=torch.tensor([7.0], device=device),
                               regularization=1e-3)
@@ -149,3 +149,25 @@ def test_a_set_against_itself_is_cut_by_the_tiles_of_one_triangle(device):
     assert torch.all(torch.diagonal(got) == 0.0)
     rows = slice(1000, 1040)
     assert_close_to_truth(got[rows], oracle.cdist(x[rows].cpu(), x.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30, what="x against x, cut")
+
+
+@pytest.mark.parametrize("out_row_major", [True, False])
+def test_a_tall_narrow_result_is_cut_beyond_65535_rows(device, monkeypatch, out_row_major):
+    """782 tiles stacked along one side, K = 2048: the call is cut over k, and the finishing
+    kernel walks more rows of the result than one grid dimension holds (70000 > 65535).  With a
+    row-major result the operands are exchanged, with a column-major one they are not: the long
+    side is n of the kernel in one case and m in the other."""
+    g = torch.Generator().manual_seed(9)
+    M, N, K = 70000, 100, 2048
+    a = torch.randn(M, K, generator=g).to(device)
+    b = torch.randn(N, K, generator=g).to(device)
+    out = torch.empty(M, N, device=device) if out_row_major else torch.empty(N, M, device=device).t()
+    plan = module._plan_run_kernel(kermac.kernel_descriptor_l1_norm, a, b, out, None, None, None, None, None, None, 0, 0, False)
+    assert plan.swapped == out_row_major and (plan.params.n if out_row_major else plan.params.m) == M
+    assert module._cut_over_contraction(plan.params) is not None
+    got = kermac.cdist(a, b, out=out, p=1.0)
+    for rows in (slice(0, 40), slice(65520, 65560), slice(M - 40, M)):
+        assert_close_to_truth(got[rows], oracle.cdist(a[rows].cpu(), b.cpu(), p=1.0)[0], rtol=1e-5, what=f"tall result rows {rows}")
+    monkeypatch.setattr(module, "_cut_over_contraction", lambda params: None)
+    uncut = kermac.cdist(a, b, p=1.0)[0]
+    assert_close_to_truth(got, uncut, rtol=5e-6, what="cut against uncut")

@@ -66,9 +66,9 @@ def test_batches_regularisation_and_unfused_composition(device, gram_mode):
     composed = torch.bmm(full.double(), coef.double())
     assert_close_to_truth(got, composed, rtol=1e-5, atol=atol_for(composed, 1e-5), what="fused vs unfused")
     assert torch.all(out[..., O] == 5.0), "wrote outside the out view"
-    truth = oracle.kernel_times_coefficients("DIFF", "SQUARE", "SQRT", "LAPLACE", x.cpu().contiguous(),
-                                             z.cpu().contiguous(), coef.cpu().contiguous(), bandwidth=bw.cpu(),
-                                             regularization=0.5, regularization_offset_x=2, regularization_offset_y=0)
+    truth = oracle.run_kernel_coefficients("DIFF", "SQUARE", "SQRT", "LAPLACE", x.cpu().contiguous(),
+                                           z.cpu().contiguous(), coef.cpu().contiguous(), bandwidth=bw.cpu(),
+                                           regularization=0.5, regularization_offset_x=2, regularization_offset_y=0)
     assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="fused vs oracle")
 
 

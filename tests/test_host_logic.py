@@ -8,6 +8,7 @@ or a wrong enum value shows up without a GPU.
 """
 import ctypes
 import re
+import sys
 from ctypes import POINTER, c_float, c_int, c_int64
 from itertools import product
 from pathlib import Path
@@ -234,14 +235,14 @@ def test_marshalling_sign_and_offsets_survive_the_swap(c_col):
     signed = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.NOOP, kermac.PowerType.NOOP,
                                      kermac.KernelType.NONE)
     got = cpu_run_kernel(signed, a, b, out=out)
-    truth = (b.double()[None, :, :] - a.double()[:, None, :]).sum(-1)        # sum_k (b - a), signed
+    truth = (a.double()[:, None, :] - b.double()[None, :, :]).sum(-1)        # sum_k (a[m] - b[n]), signed
     assert_close_to_truth(got, truth, rtol=1e-6, atol=1e-9, what="signed difference")
     got = cpu_run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, out=out, bandwidth=2.0, regularization=0.5,
                          regularization_offset_x=4, regularization_offset_y=1)
     truth = torch.exp(-torch.cdist(a.double(), b.double(), p=1.0) / 2.0)
-    for m in range(M):
-        if 0 <= m + 3 < N:
-            truth[m, m + 3] = 1.5
+    for n in range(N):                      # offset_x + n == offset_y + m: the reference's out=None result
+        if 0 <= n + 3 < M:
+            truth[n + 3, n] = 1.5
     assert_close_to_truth(got, truth, rtol=1e-6, what="offset diagonal")
 
 
@@ -306,7 +307,8 @@ def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
         kermac.set_l2_mode("direct")
     # the default trust grows with K so that very long sums fall back to the direct kernel
     from kermac_amd.build_a_kernel import _gram_trust
-    assert _gram_trust(1024) == pytest.approx(0.25) and _gram_trust(1 << 20) > 2.0
+    default = {"trust": None}
+    assert _gram_trust(1024, default) == pytest.approx(0.25) and _gram_trust(1 << 20, default) > 2.0
     # the C ABI refuses the flag for other inner powers
     params = _backend.BuildKernelParams()
     params.inner_power, params.flags, params.l = 1, _backend.FLAG_L2_GRAM, 1
@@ -481,3 +483,69 @@ def test_launch_cuts_follow_the_shape_and_the_environment_switch(monkeypatch):
     assert module._cut_over_contraction(block(5120, 5120, 4096, same=True)) is not None
     monkeypatch.setenv("KERMAC_AMD_NO_CUT", "1")
     assert module._cut_over_contraction(block(100, 100, 100000)) is None
+
+
+def test_reference_module_name_resolves_to_this_package():
+    """Callers of the reference do `import kermac` (examples/cdist.py:2, tests/test_cdist.py:3)."""
+    import kermac as by_reference_name
+    import kermac.common
+    import kermac.module_cache.module_cache
+    import kermac_amd.module_cache.module_cache
+    assert by_reference_name is kermac
+    assert kermac.common is sys.modules["kermac_amd.common"]
+    assert sys.modules["kermac.module_cache.module_cache"] is kermac_amd.module_cache.module_cache
+    from kermac.common import Majorness
+    assert Majorness is kermac.Majorness
+    for name in ("cdist", "cdist_grad", "run_kernel", "pre_compile_descriptors", "KernelDescriptor", "InnerOperator",
+                 "PowerType", "KernelType", "Symmetry", "ModuleCache", "CudaTimer", "tensor_stats", "TensorStats",
+                 "Majorness", "Alignment", "FillMode", "ceil_div", "merge_batch_size", "PyTorchStreamWrapper",
+                 "kernel_descriptor_laplace_l1", "kernel_descriptor_laplace_l2", "kernel_descriptor_p_norm",
+                 "kernel_descriptor_l1_norm", "kernel_descriptor_l2_norm", "kernel_descriptor_mma"):
+        assert hasattr(by_reference_name, name), name
+
+
+def test_l2_mode_blocks_are_per_thread():
+    import threading
+    seen = {}
+    ready, release = threading.Event(), threading.Event()
+
+    def worker():
+        with kermac.l2_mode("gram_bf16"):
+            seen["worker_inside"] = kermac.get_l2_mode()
+            ready.set()
+            release.wait(10)
+        seen["worker_after"] = kermac.get_l2_mode()
+
+    thread = threading.Thread(target=worker)
+    thread.start()
+    assert ready.wait(10)
+    assert kermac.get_l2_mode() == "direct"             # the other thread's block does not leak
+    with kermac.l2_mode("gram", trust=0.5):
+        assert kermac.get_l2_mode() == "gram"
+        plan = _plan_run_kernel(kermac.kernel_descriptor_l2_norm, torch.zeros(4, 64), torch.zeros(4, 64), None, None,
+                                None, None, None, None, None, 0, 0, False, require_device=False)
+        assert plan.params.flags & _backend.FLAG_L2_GRAM and not plan.params.flags & _backend.FLAG_L2_GRAM_BF16
+        assert plan.params.gram_trust == 0.5
+        with kermac.l2_mode("direct"):
+            assert kermac.get_l2_mode() == "direct"
+        assert kermac.get_l2_mode() == "gram"
+    release.set()
+    thread.join()
+    assert seen == {"worker_inside": "gram_bf16", "worker_after": "direct"}
+    assert kermac.get_l2_mode() == "direct"
+    with pytest.raises(ValueError):
+        with kermac.l2_mode("fast"):
+            pass
+
+
+def test_cut_decision_for_a_tall_narrow_result():
+    """cdist(a[100000, 4096], b[100, 4096]) with the default row-major result reaches the kernel as
+    m = 100, n = 100000 (operands exchanged): 782 tiles, so the cut over k is taken; the finishing
+    step strides over the rows, so there is no limit of 65535 on n."""
+    from kermac_amd import build_a_kernel as module
+    plan = _plan_run_kernel(kermac.kernel_descriptor_l1_norm, torch.empty(100000, 4096, device="meta"),
+                            torch.empty(100, 4096, device="meta"), torch.empty(100000, 100, device="meta"), None, None,
+                            None, None, None, None, 0, 0, False, require_device=False)
+    assert plan.swapped and (plan.params.m, plan.params.n) == (100, 100000)
+    cut = module._cut_over_contraction(plan.params)
+    assert cut is not None and cut[0] * cut[1] >= 4096 and cut[1] % 16 == 0

@@ -94,8 +94,8 @@ def test_kernels_batches_and_regularisation(device, gram_mode):
     bw = torch.tensor([2.0, 5.0, 9.0], device=device)
     got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, data, data, bandwidth=bw, regularization=0.125,
                             regularization_offset_x=2, regularization_offset_y=0)
-    truth = oracle.build_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", data.cpu(), data.cpu(), bandwidth=bw.cpu(),
-                                regularization=0.125, regularization_offset_x=2, regularization_offset_y=0)
+    truth = oracle.run_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", data.cpu(), data.cpu(), bandwidth=bw.cpu(),
+                              regularization=0.125, regularization_offset_x=2, regularization_offset_y=0)
     assert_close_to_truth(got, truth, rtol=1e-5, what="gram laplace-l2")
     gaussian = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP,
                                        kermac.KernelType.GAUSSIAN)

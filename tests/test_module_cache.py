@@ -66,6 +66,18 @@ def test_source_hash_change_clears_the_store(tmp_path):
     assert (tmp_path / "source_hash").read_text() == "hash-two"
 
 
+def test_damaged_code_object_is_dropped_not_returned(tmp_path):
+    store = CodeObjectStore(tmp_path, "hash-one")
+    key = FunctionKey("kermac_amd", "0.1.0", "7.0", "gfx950", "-O3", "kmc::f<1>")
+    code_hash = store.put_code(b"\x7fELFfake-code-object")
+    store.put_function_mapping(key, "_Zf1", code_hash)
+    path = tmp_path / f"code-{code_hash}.hsaco"
+    path.write_bytes(b"\x7fELFfake")                      # truncated behind the store's back
+    assert store.get_code(code_hash) is None              # bytes no longer hash to the name
+    assert not path.exists()
+    assert store.get_function_mapping(key) is None        # so the function counts as not compiled
+
+
 def test_key_covers_everything_the_binary_depends_on(tmp_path):
     store = CodeObjectStore(tmp_path, "h")
     base = dict(package_name="kermac_amd", package_version="0.1.0", toolchain_version="7.0", arch="gfx950",

@@ -184,3 +184,26 @@ def test_kernel_times_coefficients_golden_and_composition():
     km = oracle.build_kernel("DIFF", "SQUARE", "NOOP", "GAUSSIAN", a, b, bandwidth=2.0).double()
     got = oracle.kernel_times_coefficients("DIFF", "SQUARE", "NOOP", "GAUSSIAN", a, b, coef, bandwidth=2.0)
     assert_close_to_truth(got, km @ coef.double(), rtol=1e-5, atol=1e-6, what="composition")
+
+
+def test_run_kernel_wrapper_is_the_references_default_layout_result():
+    """oracle.run_kernel = the reference's run_kernel for out=None: operands exchanged in
+    front of the kernel, offsets and sign left alone (src/kermac/build_a_kernel.py:259,323-336).
+    Its examples/broadcast_kernel.py passes offsets (3, 1): 1 + regularization lands where
+    3 + n == 1 + m, at [n + 2, n]; a signed inner term reads a[m] - b[n]."""
+    g = torch.Generator().manual_seed(4)
+    a, b = torch.randn(9, 5, generator=g), torch.randn(7, 5, generator=g)
+    got = oracle.run_kernel("DIFF", "NOOP", "NOOP", "NONE", a, b)[0]
+    truth = (a.double()[:, None, :] - b.double()[None, :, :]).sum(-1)
+    assert_close_to_truth(got, truth, rtol=1e-6, atol=1e-9, what="signed difference a - b")
+    got = oracle.run_kernel("DIFF", "ABS", "NOOP", "LAPLACE", a, b, bandwidth=2.0, regularization=0.25,
+                            regularization_offset_x=3, regularization_offset_y=1)[0]
+    truth = torch.exp(-torch.cdist(a.double(), b.double(), p=1.0) / 2.0)
+    for n in range(7):
+        if n + 2 < 9:
+            truth[n + 2, n] = 1.25
+    assert_close_to_truth(got, truth, rtol=3e-7, what="offset diagonal of the default layout")
+    coef = torch.randn(7, 3, generator=g)
+    fused = oracle.run_kernel_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", a, b, coef, bandwidth=2.0,
+                                           regularization=0.25, regularization_offset_x=3, regularization_offset_y=1)[0]
+    assert_close_to_truth(fused, truth @ coef.double(), rtol=1e-6, atol=1e-6, what="fused product, same convention")

@@ -96,7 +96,7 @@ def test_run_kernel_random_descriptors_and_layouts(device, seed):
         what = f"seed {seed} case {case}: {descriptor} L={L} M={M} N={N} K={K} {kwargs.keys()}"
         print(what, flush=True)
         got = kermac.run_kernel(descriptor, a, b, out=out, **kwargs)
-        truth = oracle.build_kernel(inner_op, inner_pow, outer_pow, kernel, a_cpu, b_cpu, **okwargs)
+        truth = oracle.run_kernel(inner_op, inner_pow, outer_pow, kernel, a_cpu, b_cpu, **okwargs)
         fractional = inner_pow == "POW" or outer_pow == "POW"
         rtol = 1e-4 if fractional else 1e-5
         # signed sums and dot products cancel: measure against the sum of magnitudes

@@ -94,14 +94,14 @@ def test_lookalikes_take_the_ordinary_path(device):
     signed = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.NOOP, kermac.PowerType.NOOP,
                                      kermac.KernelType.NONE)
     got = kermac.run_kernel(signed, x, x)[0]
-    truth = (x.double()[None] - x.double()[:, None]).sum(-1)
+    truth = (x.double()[:, None] - x.double()[None]).sum(-1)          # sum_k (a[m] - b[n])
     assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-5, what="signed self differences")
     assert torch.equal(got, -got.t())
     # different regularisation offsets: the replaced diagonal is not symmetric
     got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, x, bandwidth=4.0, regularization=0.25,
                             regularization_offset_x=130, regularization_offset_y=0)[0]
-    truth = oracle.build_kernel("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu(), x.cpu(), bandwidth=4.0, regularization=0.25,
-                                regularization_offset_x=130, regularization_offset_y=0)[0]
+    truth = oracle.run_kernel("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu(), x.cpu(), bandwidth=4.0, regularization=0.25,
+                              regularization_offset_x=130, regularization_offset_y=0)[0]
     assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-7, what="offset diagonal")
     assert not torch.equal(got, got.t())
     # same pointer but another extent: rows of one panel against a prefix of it
