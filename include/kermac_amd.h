@@ -168,6 +168,25 @@ int kmc_build_kernel_finish(const kmc_build_kernel_params *params, const float *
                             int64_t partial_bs, int64_t partial_slice, int32_t slices, void *stream);
 
 /*
+ * The cut over k above as one call that allocates nothing.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  `params` describes the
+ * whole problem exactly as for kmc_build_kernel (l must be 1, k_total 0, no matrix-core
+ * flags, an ahead-of-time compiled (inner_operator, inner_power) pair); k is cut into at
+ * most `ranges` ranges of whole 16-term slices, kmc_build_kernel computes their plain sums
+ * and kmc_build_kernel_finish adds them in range order and applies the epilogue -- the same
+ * two launches, the same bits, as the two-call form with a caller-supplied buffer.  The
+ * partial sums live in a static device array of the library: KMC_STATIC_SCRATCH_BYTES on
+ * every GPU that runs the library, held until the process ends.  A call whose
+ * ceil(k / depth) * n * (m rounded up to 4) floats do not fit is rejected with
+ * KMC_ERR_INVALID_ARGUMENT before anything is launched.  No hipMalloc, hipFree or other
+ * allocating call is made.  All calls on one GPU share the array: calls on one stream are
+ * ordered, calls that overlap on one GPU (two streams, two host threads) race.
+ */
+#define KMC_STATIC_SCRATCH_BYTES (64u << 20)
+int kmc_build_kernel_cut_static(const kmc_build_kernel_params *params, int32_t ranges, void *stream);
+
+/*
  * Arguments of the fused kernel-gradient contraction; mirrors the 24 launch
  * arguments of cute_norm_kernel_gradient (include/p_norm_gradient.cuh:413-422,
  * marshalled at src/kermac/cdist_grad.py:226-235).

@@ -93,6 +93,7 @@ SIGNATURES = {
     "kmc_build_kernel_jit": (ctypes.c_int, [c_void_p, POINTER(BuildKernelParams), c_void_p]),
     "kmc_build_kernel_finish": (ctypes.c_int, [POINTER(BuildKernelParams), c_void_p, c_int64, c_int64, c_int64, c_int32,
                                                c_void_p]),
+    "kmc_build_kernel_cut_static": (ctypes.c_int, [POINTER(BuildKernelParams), c_int32, c_void_p]),
     "kmc_build_kernel_load_modes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int32), POINTER(c_int32)]),
     "kmc_norm_kernel_gradient": (ctypes.c_int, [POINTER(NormGradientParams), c_void_p]),
     "kmc_kernel_times_coefficients": (ctypes.c_int, [POINTER(KernelCoefficientsParams), c_void_p]),
@@ -172,6 +173,14 @@ def build_kernel_finish(params: BuildKernelParams, partials: int, partial_ld: in
                         slices: int, stream: int) -> None:
     check(library().kmc_build_kernel_finish(byref(params), c_void_p(partials), partial_ld, partial_bs, partial_slice,
                                             slices, c_void_p(stream)))
+
+
+STATIC_SCRATCH_BYTES = 64 << 20
+
+
+def build_kernel_cut_static(params: BuildKernelParams, ranges: int, stream: int) -> None:
+    """The cut over k with the partial sums in the library's static device array: allocates nothing."""
+    check(library().kmc_build_kernel_cut_static(byref(params), ranges, c_void_p(stream)))
 
 
 def build_kernel_jit(function: int, params: BuildKernelParams, stream: int) -> None:
