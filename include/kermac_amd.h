@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define KMC_ABI_VERSION 1
+#define KMC_ABI_VERSION 2
 
 enum kmc_status {
     KMC_OK = 0,
@@ -229,6 +229,17 @@ typedef struct kmc_kernel_coefficients_params {
     int32_t o;                                    /* coefficient columns */
     const float *coef; int64_t coef_ld; int64_t coef_bs;  /* [n, o], o contiguous */
     float *out; int64_t out_ld; int64_t out_bs;           /* [m, o], o contiguous */
+    /* 0 or 1: one launch computes the whole product.  R > 1: the n rows of b and coef (the
+     * centres) are cut into R consecutive ranges of ceil(ceil(n / 128) / R) tiles of 128, every
+     * range is walked by workgroups of its own and writes its partial product
+     *   out[m*out_ld + o + l*out_bs + r*out_range_stride],
+     * and the caller adds the R partial products (in a fixed order, for reproducible results).
+     * A workgroup owns 128 rows m and walks every centre of its range, so few rows against
+     * many centres, or a batch of problems that fills only two workgroup slots per CU, leave
+     * the chip under-used unless the centres are cut.  Everything else, the regularised
+     * diagonal included (it is addressed by the global index n), is unchanged. */
+    int32_t n_ranges;
+    int64_t out_range_stride;
 } kmc_kernel_coefficients_params;
 
 /* Coefficient columns are processed in chunks of 32 per workgroup; o > 32 works

@@ -16,7 +16,7 @@ from typing import List, Optional, Sequence, Tuple
 # KERMAC_AMD_LIBRARY points at another build of the same ABI (e.g. an experimental one).
 LIB_PATH = Path(os.environ.get("KERMAC_AMD_LIBRARY") or Path(__file__).resolve().parent / "_lib" / "libkermac_amd.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # enum kmc_status
 OK = 0
@@ -80,6 +80,7 @@ class KernelCoefficientsParams(Structure):
         ("o", c_int32),
         ("coef", _float_p), ("coef_ld", c_int64), ("coef_bs", c_int64),
         ("out", _float_p), ("out_ld", c_int64), ("out_bs", c_int64),
+        ("n_ranges", c_int32), ("out_range_stride", c_int64),
     ]
 
 

@@ -43,7 +43,13 @@ int prepare(const kmc_kernel_coefficients_params *p, bool wide_allowed, kmc::Ker
     const int64_t grid_y = static_cast<int64_t>(k.l) * kc->o_chunks;
     if (grid_y > 65535)
         return fail(KMC_ERR_INVALID_ARGUMENT, "batch x coefficient chunks = %lld exceeds 65535", static_cast<long long>(grid_y));
-    *grid = dim3(k.tiles_m, static_cast<unsigned>(grid_y), 1);
+    if (p->n_ranges < 0 || p->n_ranges > 65535)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "n_ranges = %d is outside 0 .. 65535", p->n_ranges);
+    const int ranges = p->n_ranges > 1 ? p->n_ranges : 1;
+    if (ranges > 1 && p->out_range_stride < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "negative out_range_stride");
+    kc->split_tiles = k.tiles_n > 0 ? ceil_div(k.tiles_n, ranges) : 1;
+    kc->out_split_stride = ranges > 1 ? p->out_range_stride : 0;
+    *grid = dim3(k.tiles_m, static_cast<unsigned>(grid_y), static_cast<unsigned>(ranges));
     return KMC_OK;
 }
 
@@ -107,7 +113,7 @@ int kmc_kernel_times_coefficients_jit(void *function, const kmc_kernel_coefficie
     if (status != KMC_OK) return status;
     size_t size = sizeof(kc);
     void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &kc, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-    hipError_t e = hipModuleLaunchKernel(static_cast<hipFunction_t>(function), grid.x, grid.y, 1, kmc::BK_THREADS, 1, 1,
+    hipError_t e = hipModuleLaunchKernel(static_cast<hipFunction_t>(function), grid.x, grid.y, grid.z, kmc::BK_THREADS, 1, 1,
                                          0, static_cast<hipStream_t>(stream), nullptr, config);
     if (e != hipSuccess) return fail_hip(e, "kernel_times_coefficients (run-time compiled) launch");
     return KMC_OK;

@@ -76,7 +76,9 @@ __global__ __launch_bounds__(BK_THREADS, 2) void gram_times_coefficients(const K
 #pragma unroll
         for (int ob = 0; ob < 2; ob++) out_acc[mb][ob] = kc_float4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    for (int n0 = 0; n0 < args.n; n0 += BK_TILE_N) {
+    int n_begin, n_end;
+    centre_range(kc, n_begin, n_end);
+    for (int n0 = n_begin; n0 < n_end; n0 += BK_TILE_N) {
         const int n_valid = args.n - n0;
 
         // 1. coefficients of this n tile -> LDS, zero filled past N and past O (as in
@@ -249,7 +251,7 @@ __global__ __launch_bounds__(BK_THREADS, 2) void gram_times_coefficients(const K
     }
 
     // Store: this lane holds rows 32 wave + 16 mb + 4 q + e, column 16 ob + r.
-    float *out_batch = kc.out + batch * kc.out_bs;
+    float *out_batch = kc.out + batch * kc.out_bs + blockIdx.z * kc.out_split_stride;
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
 #pragma unroll

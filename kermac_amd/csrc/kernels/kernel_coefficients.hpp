@@ -35,7 +35,21 @@ struct KernelCoefficientsArgs {
     float *out; i64 out_ld, out_bs;            // [m, o], o contiguous
     int coef_vec;                  // coef, coef_ld, coef_bs multiples of 16 bytes
     int columns;                   // coefficient columns per workgroup: the COLUMNS the launched kernel was built with
+    // The centres can be cut into consecutive ranges of whole n tiles, one per blockIdx.z: range z
+    // walks `split_tiles` tiles from tile z * split_tiles on and writes its partial product to
+    // out + z * out_split_stride; the caller adds the ranges.  One range: the whole product.
+    int split_tiles;
+    i64 out_split_stride;
 };
+
+// First centre and one past the last centre of the range this workgroup walks.
+__device__ __forceinline__ void centre_range(const KernelCoefficientsArgs &kc, int &n_begin, int &n_end)
+{
+    const i64 first = (i64)blockIdx.z * kc.split_tiles * BK_TILE_N;
+    const i64 last = first + (i64)kc.split_tiles * BK_TILE_N;
+    n_begin = (int)(first < kc.kernel.n ? first : kc.kernel.n);
+    n_end = (int)(last < kc.kernel.n ? last : kc.kernel.n);
+}
 
 constexpr int KC_COLUMNS = 32;      // coefficient columns per workgroup (64 in the wide instantiations)
 constexpr int KC_PASS_N = 32;       // n per contraction pass
@@ -47,8 +61,15 @@ constexpr int KC_STAGE_FLOATS = 2 * (2 * BK_LDS_SLICE + BK_LDS_PITCH);
 // COLUMNS: 32, or 64 for more than 32 coefficient columns (every chunk of columns
 // rebuilds the whole kernel matrix, so O = 64 in two chunks of 32 costs twice O = 32;
 // 64 columns per workgroup still leave LDS for two workgroups per CU).
+// Waves per SIMD the 32-column kernel is compiled for.  Three (168 registers; the compiler spills
+// about 20, none of them inside the K walk) let a CU hold three workgroups, which is what the K
+// walk needs to reach its rate; measured with the centres cut into ranges (so that there are
+// workgroups for every place) 9.6 against 10.4 ms at L = 4, M = N = 16384, K = 256, O = 32.
+#ifndef KC_MIN_WAVES
+#define KC_MIN_WAVES 3
+#endif
 template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B, int COLUMNS = KC_COLUMNS>
-__global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const KernelCoefficientsArgs kc)
+__global__ __launch_bounds__(BK_THREADS, COLUMNS == KC_COLUMNS ? KC_MIN_WAVES : 2) void kernel_times_coefficients(const KernelCoefficientsArgs kc)
 {
     static_assert(COLUMNS % 32 == 0, "whole pairs of 16-column blocks");
     constexpr int COLUMN_BLOCKS = COLUMNS / 16;
@@ -91,7 +112,9 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
 #pragma unroll
         for (int ob = 0; ob < COLUMN_BLOCKS; ob++) out_acc[mb][ob] = kc_float4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    for (int n0 = 0; n0 < args.n; n0 += BK_TILE_N) {
+    int n_begin, n_end;
+    centre_range(kc, n_begin, n_end);
+    for (int n0 = n_begin; n0 < n_end; n0 += BK_TILE_N) {
         const int n_valid = args.n - n0;
 
         // 1. coefficients of this n tile -> LDS, zero filled past N and past O.
@@ -182,7 +205,7 @@ __global__ __launch_bounds__(BK_THREADS) void kernel_times_coefficients(const Ke
     }
 
     // Store: this lane holds rows 32 wave + 16 mb + 4 q + i, column 16 ob + r.
-    float *out_batch = kc.out + batch * kc.out_bs;
+    float *out_batch = kc.out + batch * kc.out_bs + blockIdx.z * kc.out_split_stride;
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
 #pragma unroll

@@ -97,7 +97,7 @@ def _plan_run_kernel_coefficients(
 def run_kernel_coefficients(
     kernel_descriptor, a, b, coefficients, out: Optional[torch.Tensor] = None, p=None, inner_p=None, outer_p=None,
     bandwidth=None, epsilon=None, regularization=None, regularization_offset_x: int = 0,
-    regularization_offset_y: int = 0, debug=False, _may_split=True,
+    regularization_offset_y: int = 0, debug=False,
 ):
     """``out[l, m, o] = sum_n run_kernel(descriptor, a, b, ...)[l, m, n] * coefficients[l, n, o]``.
 
@@ -110,17 +110,22 @@ def run_kernel_coefficients(
     plan = _plan_run_kernel_coefficients(
         kernel_descriptor, a, b, coefficients, out, p, inner_p, outer_p, bandwidth, epsilon, regularization,
         regularization_offset_x, regularization_offset_y)
-    split = _split_over_centres(plan, a, b, coefficients, regularization) if _may_split else None
-    if split is not None:
-        _run_split_over_centres(split, plan, kernel_descriptor, a, b, coefficients, p, inner_p, outer_p, bandwidth,
-                                epsilon, debug)
-        return plan.out
     stream = _current_stream_for(a.device)
     params = plan.params
     kernel = params.kernel
-    if _backend.kernel_times_coefficients_has_variant(kernel.inner_operator, kernel.inner_power):
+    aot = _backend.kernel_times_coefficients_has_variant(kernel.inner_operator, kernel.inner_power)
+    matrix_core = bool(kernel.flags & _backend.FLAG_L2_GRAM)
+    ranges = _centre_ranges(plan, three_resident=aot and not matrix_core and plan.O <= 32)
+    partial = None
+    if ranges > 1:
+        # every range of centres writes its own partial product; they are added below in range order
+        partial = torch.empty((ranges, plan.L, plan.M, plan.O), dtype=torch.float32, device=a.device)
+        params.out, params.out_ld, params.out_bs = partial.data_ptr(), plan.O, plan.M * plan.O
+        params.n_ranges, params.out_range_stride = ranges, plan.L * plan.M * plan.O
+    if aot:
         if debug:
-            print(f"(Kermac Debug) Launching ahead-of-time fused coefficient kernel for {kernel_descriptor!r}")
+            print(f"(Kermac Debug) Launching ahead-of-time fused coefficient kernel for {kernel_descriptor!r}"
+                  + (f", centres in {ranges} ranges" if ranges > 1 else ""))
         _backend.kernel_times_coefficients(params, stream)
     else:
         load_a, load_b = _backend.build_kernel_load_modes(kernel)
@@ -129,82 +134,69 @@ def run_kernel_coefficients(
         if debug:
             print(f"(Kermac Debug) Launching kernel: {name}")
         _backend.kernel_times_coefficients_jit(function, params, stream)
+    if partial is not None:
+        target = plan.out if plan.out.dim() == 3 else plan.out.unsqueeze(0)
+        if target.is_contiguous():
+            torch.sum(partial, dim=0, out=target)
+        else:
+            # the order in which torch adds the ranges depends on the layout of the result: a strided
+            # `out` gets the bits of a contiguous one
+            target.copy_(torch.sum(partial, dim=0))
     return plan.out
 
 
-# A workgroup of the fused kernel owns 128 rows of ``a`` and walks every centre, so a
-# launch has ceil(M / 128) x L x ceil(O / 64) long-running workgroups, of which 512 run at
-# a time (two per CU).  Few rows against many centres (prediction for a small batch of
-# points) would leave most of the chip idle, and a count just above a multiple of 512
-# leaves it idle for most of the last round.  Such an unbatched call is cut over the
-# centres: slices of ``b`` and ``coefficients`` become the batch of one launch (``a``
-# broadcasts), each slice writes its own partial result, and the partial results are summed
-# in a fixed order.
-_SPLIT_CONCURRENT_WORKGROUPS = 512
-_SPLIT_MIN_CENTRES = 128
-_SPLIT_WORKGROUP_OVERHEAD = 64           # start-up and store of a workgroup, in centres walked
+# A workgroup of the fused kernel owns 128 rows of ``a`` (one batch entry, one chunk of up to 64
+# coefficient columns) and walks every centre, so a launch has ceil(M / 128) x L x ceil(O / 64)
+# long-running workgroups, three to a CU (two for the 64-column and matrix-core variants).  Few rows
+# against many centres (prediction for a small batch of points) would leave most of the chip idle;
+# a batch that fills two places per CU (L = 4, M = 16384: 512 workgroups) leaves a third of the
+# places empty; and a few long workgroups per CU, all started together, finish unevenly.  The
+# kernel therefore takes the centres in ranges (``n_ranges`` of the C parameter block): every range
+# is walked by workgroups of its own into a partial product of its own, and the partial products
+# are added in range order.  Measured at L = 4, M = N = 16384, K = 256, O = 32: 10.4 ms uncut,
+# 10.0 ms in 6 ranges, 9.6 ms in 12 to 43, 9.7 ms in 64 (the kernel matrix written out and
+# multiplied by torch.bmm: 10.0 ms).  The number of ranges comes from the model of the launch time
+# that the pairwise kernel uses for its cut over k (same K walk, same three regimes).
 _SPLIT_MAX_PARTIAL_BYTES = 256 << 20
-_SPLIT_WORTH = 0.92                      # cut only for at least 8 % less modelled time (448 workgroups: 10 % modelled, 14 % measured)
+_SPLIT_WORTH = 0.95                           # cut only for at least 5 % less modelled time
+_TILE_OVERHEAD_K = 24                         # coefficient staging and contraction of one tile, in k-steps
 
 
-def _split_over_centres(plan, a, b, coefficients, regularization):
-    """(slices, rows per slice, leftover rows), or None when the call is launched as it is."""
-    if plan.L != 1:
-        return None                      # the batch index of the launch is taken by the caller's batches
-    if regularization is not None and not (isinstance(regularization, (int, float)) and regularization == 0):
-        return None                      # the regularised diagonal is addressed by the global centre index
-    if plan.M == 0 or plan.O == 0 or plan.N < 2 * _SPLIT_MIN_CENTRES or not launch_cuts_enabled():
-        return None
-    return _choose_split(plan.M, plan.N, plan.O)
+def _centre_ranges(plan, three_resident):
+    """How many ranges the centres are cut into (1: the launch goes out as it is)."""
+    if plan.M == 0 or plan.O == 0 or plan.L == 0 or plan.N <= 128 or not launch_cuts_enabled():
+        return 1
+    workgroups = -(-plan.M // 128) * plan.L * max(1, -(-plan.O // 64))
+    return _choose_ranges(workgroups, -(-plan.N // 128), plan.K, 3 if three_resident else 2,
+                          4 * plan.L * plan.M * plan.O)
 
 
-@functools.lru_cache(maxsize=256)
-def _choose_split(M, N, O):
-    workgroups = -(-M // 128) * max(1, -(-O // 64))
-
-    def rounds(count):
-        return -(-count // _SPLIT_CONCURRENT_WORKGROUPS)
-
-    # Modelled time of a launch: centres walked per workgroup (plus its fixed cost) times rounds of
-    # workgroups.  Slices are a whole number of tiles each, so a 16-byte aligned operand stays
-    # aligned in every slice; the rows that remain go into a second launch.
-    unsplit = (N + _SPLIT_WORKGROUP_OVERHEAD) * rounds(workgroups)
-    most = min(N // _SPLIT_MIN_CENTRES, _SPLIT_MAX_PARTIAL_BYTES // (4 * M * O) - 1,
-               max(16, _SPLIT_CONCURRENT_WORKGROUPS // workgroups))
-    best = None
-    for slices in range(2, most + 1):
-        for rows in (N // slices // 128 * 128, -(-N // slices // 128) * 128):
-            if rows < _SPLIT_MIN_CENTRES:
-                continue
-            full = N // rows
-            leftover = N - full * rows
-            cost = (rows + _SPLIT_WORKGROUP_OVERHEAD) * rounds(full * workgroups)
-            if leftover:
-                cost += (leftover + _SPLIT_WORKGROUP_OVERHEAD) * rounds(workgroups)
-            if full >= 2 and (best is None or cost < best[0]):
-                best = (cost, full, rows, leftover)
-    if best is None or best[0] > _SPLIT_WORTH * unsplit:
-        return None
-    return best[1:]
+def _launch_ms(workgroups, depth, resident):
+    """Modelled time of `workgroups` workgroups that walk `depth` k-steps each, in milliseconds."""
+    per_cu = workgroups / 256
+    if per_cu <= 1:
+        return (depth + 128) / 3900                               # one wave per SIMD: latency bound
+    slower = 1.0 if resident == 3 else 1.0 / 0.912                # two resident workgroups deliver 0.91 of three
+    if per_cu <= resident:
+        return -(-workgroups // 256) * (depth + 128) / 7300 * slower     # one round, all started together
+    return (per_cu + 1.92) * (depth + 40) / 10000 * slower       # rounds that the dispatcher balances
 
 
-def _run_split_over_centres(split, plan, kernel_descriptor, a, b, coefficients, p, inner_p, outer_p, bandwidth, epsilon,
-                            debug):
-    full, rows, leftover = split
-    a2, b2, c2 = (t[0] if t.dim() == 3 else t for t in (a, b, coefficients))
-    M, K, O = plan.M, plan.K, plan.O
-    partial = torch.empty((full + (1 if leftover else 0), M, O), dtype=torch.float32, device=a.device)
-    b_slices = b2.as_strided((full, rows, K), (rows * b2.stride(0), b2.stride(0), b2.stride(1)), b2.storage_offset())
-    c_slices = c2.as_strided((full, rows, O), (rows * c2.stride(0), c2.stride(0), c2.stride(1)), c2.storage_offset())
-    hyper = dict(p=p, inner_p=inner_p, outer_p=outer_p, bandwidth=bandwidth, epsilon=epsilon, debug=debug,
-                 _may_split=False)
-    run_kernel_coefficients(kernel_descriptor, a2, b_slices, c_slices, partial[:full], **hyper)
-    if leftover:
-        run_kernel_coefficients(kernel_descriptor, a2, b2[full * rows:], c2[full * rows:], partial[full:], **hyper)
-    target = plan.out[0] if plan.out.dim() == 3 else plan.out
-    if target.is_contiguous():
-        torch.sum(partial, dim=0, out=target)
-    else:
-        # the order in which torch adds the slices depends on the layout of the result: a strided
-        # `out` gets the bits of a contiguous one
-        target.copy_(torch.sum(partial, dim=0))
+@functools.lru_cache(maxsize=512)
+def _choose_ranges(workgroups, tiles, K, resident, product_bytes):
+    per_tile = K + _TILE_OVERHEAD_K
+    unsplit = _launch_ms(workgroups, tiles * per_tile, resident)
+    best = (unsplit, 1)
+    most = min(tiles, _SPLIT_MAX_PARTIAL_BYTES // max(product_bytes, 1))
+    seen = tiles
+    for ranges in range(2, most + 1):
+        walk = -(-tiles // ranges)
+        if walk == seen:
+            continue                      # the same tiles per range as one range fewer: only more empty ranges
+        seen = walk
+        used = -(-tiles // walk)
+        count = workgroups * used
+        cost = _launch_ms(count, walk * per_tile, resident) + 2.1e-5 * count + 0.01     # partial products, second launch
+        if cost < best[0]:
+            best = (cost, used)
+    return best[1] if best[0] <= _SPLIT_WORTH * unsplit else 1

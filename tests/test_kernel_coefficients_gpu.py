@@ -116,10 +116,11 @@ def test_no_centres_gives_zeros(device):
 
 @pytest.mark.parametrize("M,N,K,O,layout", [(130, 5077, 24, 3, "cc"), (1000, 20000, 16, 1, "rr"), (64, 4096, 33, 70, "cr"),
                                             (300, 1024, 8, 5, "rc")])
-def test_few_rows_many_centres_are_cut_over_the_centres(device, M, N, K, O, layout):
-    """Few rows against many centres: the call becomes one batched launch over slices of the
-    centres plus a fixed-order sum of the partial results (kermac_amd/kernel_coefficients.py);
-    same values as the composition, into a caller's strided out as well."""
+def test_few_rows_many_centres_are_cut_over_the_centres(device, monkeypatch, M, N, K, O, layout):
+    """Few rows against many centres: the launch takes the centres in ranges (n_ranges of the C
+    parameter block), each with workgroups and a partial product of its own, and the partial
+    products are added in range order (kermac_amd/kernel_coefficients.py); same values as the
+    composition, with a regularised diagonal and into a caller's strided out as well."""
     from kermac_amd import kernel_coefficients as kc
     g = torch.Generator().manual_seed(M + N + K + O)
     a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False, dist="rand")
@@ -127,15 +128,41 @@ def test_few_rows_many_centres_are_cut_over_the_centres(device, M, N, K, O, layo
     coef = torch.randn(N, O, generator=g).to(device)
     plan = kc._plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l1, a, b, coef, None, None, None, None, 2.0,
                                             None, None, 0, 0)
-    assert kc._split_over_centres(plan, a, b, coef, None) is not None
-    assert kc._split_over_centres(plan, a, b, coef, 0.5) is None        # the regularised diagonal needs global indices
+    assert kc._centre_ranges(plan, three_resident=O <= 32) > 1
     got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, bandwidth=2.0)
     assert got.shape == (1, M, O)
     truth = oracle.kernel_times_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", a.cpu(), b.cpu(), coef.cpu(), bandwidth=2.0)
     assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="split over centres")
-    unsplit = kc.run_kernel_coefficients(kermac.kernel_descriptor_laplace_l1, a, b, coef, bandwidth=2.0, _may_split=False)
+    monkeypatch.setattr(kc, "_centre_ranges", lambda plan, three_resident: 1)
+    unsplit = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, bandwidth=2.0)
+    monkeypatch.undo()
     torch.testing.assert_close(got, unsplit, rtol=1e-5, atol=atol_for(truth, 1e-5))
+    # the regularised diagonal is addressed by the global centre index, whatever the range
+    kw = dict(bandwidth=2.0, regularization=0.5, regularization_offset_x=0, regularization_offset_y=N - M)   # n = m + N - M: the last centres
+    got_reg = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, **kw)
+    truth_reg = oracle.run_kernel_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", a.cpu(), b.cpu(), coef.cpu(), **kw)
+    assert (truth_reg - truth).abs().max() > 0, "the diagonal must fall inside the matrix for this check to mean anything"
+    assert_close_to_truth(got_reg, truth_reg, rtol=1e-5, atol=atol_for(truth, 1e-5), what="ranges of centres, regularised diagonal")
     wide = torch.full((M, O + 3), -7.0, device=device)
     out = wide[:, :O]
     assert kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, bandwidth=2.0, out=out) is out
     assert torch.equal(out, got[0]) and torch.all(wide[:, O:] == -7.0)
+
+
+def test_batched_calls_take_the_centres_in_ranges(device, monkeypatch):
+    """A batch with broadcast centres and per-batch bandwidths, cut into ranges of centres with a
+    ragged last range; same values as the uncut launch and as the oracle, and the n_ranges field
+    of the C parameter block on its own with a range count that leaves ranges empty."""
+    from kermac_amd import kernel_coefficients as kc
+    g = torch.Generator().manual_seed(99)
+    L, M, N, K, O = 3, 200, 1100, 20, 12
+    x = make_operand(L, M, K, True, device, g, dist="rand")
+    z = make_operand(1, N, K, True, device, g, batch=False, dist="rand")
+    coef = torch.randn(L, N, O, generator=g).to(device)
+    bw = torch.tensor([1.0, 2.0, 3.0], device=device)
+    truth = oracle.kernel_times_coefficients("DIFF", "ABS", "NOOP", "LAPLACE", x.cpu().contiguous(), z.cpu().contiguous(),
+                                             coef.cpu(), bandwidth=bw.cpu())
+    for ranges in (1, 2, 4, 9, 13):                     # 9 tiles of centres: 13 leaves four ranges empty
+        monkeypatch.setattr(kc, "_centre_ranges", lambda plan, three_resident, r=ranges: r)
+        got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, z, coefficients=coef, bandwidth=bw)
+        assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"{ranges} ranges of centres")

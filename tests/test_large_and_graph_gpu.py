@@ -191,7 +191,7 @@ def test_cut_launches_replay_from_a_hip_graph(device):
     out_fused = torch.empty(1, M, O, device=device)
     plan = coef_module._plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l1, x, z, coef, None, None, None,
                                                      None, 2.0, None, None, 0, 0)
-    assert coef_module._split_over_centres(plan, x, z, coef, None) is not None
+    assert coef_module._centre_ranges(plan, three_resident=True) > 1
     weights = torch.rand(4100, 150, generator=g).to(device)     # cdist_grad's a[K', M']
     centres = torch.randn(30, 4100, generator=g).to(device)     # b[N', K']
     classes = torch.randn(2, 4100, generator=g).to(device)      # c[O', K']
