@@ -139,17 +139,24 @@ def build(force: bool = True, verbose: bool = False, workers: int | None = None,
 
 
 def build_c_example(verbose: bool = False) -> Path:
-    """Link examples/c_abi_cdist.cpp (a HIP host program that uses nothing but the C
-    ABI) against the library, next to it, with an rpath relative to the binary."""
-    source = PACKAGE_DIR.parent / "examples" / "c_abi_cdist.cpp"
+    """Build the two stand-alone HIP programs of examples/ next to the library:
+    c_abi_cdist (uses nothing but the C ABI; linked against the library with an rpath relative
+    to the binary) and valu_issue_rates (the inner-loop instruction mixes of the kernel headers
+    on registers only: the issue ceilings the benchmark reports against)."""
+    examples = PACKAGE_DIR.parent / "examples"
     target = LIB_DIR / "c_abi_cdist"
-    cmd = [_hipcc(), f"--offload-arch={ARCH}", "-O2", "-std=c++17", f"-I{PACKAGE_DIR.parent / 'include'}", str(source),
-           f"-L{LIB_DIR}", "-lkermac_amd", "-Wl,-rpath,$ORIGIN", "-o", str(target)]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"building {source.name} failed:\n{proc.stdout}\n{proc.stderr}")
+    commands = [
+        [_hipcc(), f"--offload-arch={ARCH}", "-O2", "-std=c++17", f"-I{PACKAGE_DIR.parent / 'include'}",
+         str(examples / "c_abi_cdist.cpp"), f"-L{LIB_DIR}", "-lkermac_amd", "-Wl,-rpath,$ORIGIN", "-o", str(target)],
+        [_hipcc(), *[flag for flag in HIPCC_FLAGS if flag != "-fPIC"], str(examples / "valu_issue_rates.hip"),
+         "-o", str(LIB_DIR / "valu_issue_rates")],
+    ]
+    for cmd in commands:
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"building {cmd[-1]} failed:\n{proc.stdout}\n{proc.stderr}")
     return target
 
 
