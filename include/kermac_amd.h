@@ -143,6 +143,16 @@ typedef struct kmc_build_kernel_params {
      * (1 .. k of them; l must be ceil(k_total / k)).  kmc_build_kernel only, not with
      * the matrix-core flags.  No counterpart in the reference. */
     int32_t k_total;
+    /* With the matrix-core flags only (ignored otherwise): a point c[k] that is subtracted from
+     * both operands while they are staged, read at gram_centre[l * gram_centre_bs + k].
+     * Distances do not change; what changes is how much |a|^2 + |b|^2 - 2 a.b cancels, which is
+     * in proportion to the norms: with a centre near the data (its mean: kmc_sample_mean) the
+     * norms are those of the spread of the data, not of its offset from the origin, and tiles of
+     * data with a common offset stay trusted instead of being recomputed.  16-byte aligned, the
+     * stride a multiple of 4, each vector padded with zeros to a multiple of 64 floats
+     * (kmc_sample_mean writes it that way).  NULL: nothing is subtracted. */
+    const float *gram_centre;
+    int64_t gram_centre_bs;
 } kmc_build_kernel_params;
 
 /* Stands in for launch(stream, config, cute_build_kernel<...>, *args)
@@ -166,6 +176,16 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream);
  */
 int kmc_build_kernel_finish(const kmc_build_kernel_params *params, const float *partials, int64_t partial_ld,
                             int64_t partial_bs, int64_t partial_slice, int32_t slices, void *stream);
+
+/*
+ * mean[l*mean_bs + k] = the mean over (a sample of) the rows of the panel x (addressed like the a
+ * operand of kmc_build_kernel: majorness, ld, batch stride bs), for use as gram_centre.  Panels
+ * of up to 4096 rows are averaged whole, longer ones over 16 evenly spaced runs of 256 rows;
+ * the sums run in a fixed order.  Every vector is padded with zeros to a multiple of 64 floats,
+ * so mean needs (l - 1) * mean_bs + roundup(k, 64) floats.  No counterpart in the reference.
+ */
+int kmc_sample_mean(const float *x, int32_t majorness, int32_t rows, int32_t k, int64_t ld, int64_t bs, int32_t l,
+                    float *mean, int64_t mean_bs, void *stream);
 
 /*
  * The cut over k above as one call that allocates nothing.  It has no counterpart in the

@@ -56,6 +56,7 @@ class BuildKernelParams(Structure):
         ("epsilon", c_float),
         ("gram_trust", c_float),
         ("k_total", c_int32),
+        ("gram_centre", _float_p), ("gram_centre_bs", c_int64),
     ]
 
 
@@ -95,6 +96,8 @@ SIGNATURES = {
     "kmc_build_kernel_finish": (ctypes.c_int, [POINTER(BuildKernelParams), c_void_p, c_int64, c_int64, c_int64, c_int32,
                                                c_void_p]),
     "kmc_build_kernel_cut_static": (ctypes.c_int, [POINTER(BuildKernelParams), c_int32, c_void_p]),
+    "kmc_sample_mean": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_int64, c_int32, c_void_p, c_int64,
+                                       c_void_p]),
     "kmc_build_kernel_load_modes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int32), POINTER(c_int32)]),
     "kmc_norm_kernel_gradient": (ctypes.c_int, [POINTER(NormGradientParams), c_void_p]),
     "kmc_kernel_times_coefficients": (ctypes.c_int, [POINTER(KernelCoefficientsParams), c_void_p]),
@@ -182,6 +185,14 @@ STATIC_SCRATCH_BYTES = 64 << 20
 def build_kernel_cut_static(params: BuildKernelParams, ranges: int, stream: int) -> None:
     """The cut over k with the partial sums in the library's static device array: allocates nothing."""
     check(library().kmc_build_kernel_cut_static(byref(params), ranges, c_void_p(stream)))
+
+
+CENTRE_PAD = 64
+
+
+def sample_mean(x: int, majorness: int, rows: int, k: int, ld: int, bs: int, l: int, mean: int, mean_bs: int,
+                stream: int) -> None:
+    check(library().kmc_sample_mean(c_void_p(x), majorness, rows, k, ld, bs, l, c_void_p(mean), mean_bs, c_void_p(stream)))
 
 
 def build_kernel_jit(function: int, params: BuildKernelParams, stream: int) -> None:

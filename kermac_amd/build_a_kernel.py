@@ -198,16 +198,19 @@ def _hyper_parameter(name, value, L, device, require_device):
 #   launches are bound by the result stores, and the direct kernel has the cheaper
 #   epilogue and no repair launch (M = N = 30000, K = 16: 1.2 ms against 2.4 .. 2.6 ms).
 _L2_DEFAULT_MIN_K = 64
-_L2_MODES = ("direct", "gram", "gram_bf16")
+_L2_AUTO_MIN_TERMS = 1e9          # "auto": below L * M * N * K terms the direct kernel is launched
+_L2_MODES = ("direct", "gram", "gram_bf16", "auto")
 # The process-wide setting, and per host thread what `l2_mode(...)` blocks have put on top
 # of it: two threads can evaluate squared differences in different modes at the same time.
 _l2_process = {"mode": os.environ.get("KERMAC_AMD_L2_MODE", "direct"), "trust": None, "min_k": _L2_DEFAULT_MIN_K}
+if _l2_process["mode"] not in _L2_MODES:
+    raise ValueError(f"KERMAC_AMD_L2_MODE must be one of {_L2_MODES}, got {_l2_process['mode']!r}")
 _l2_thread = threading.local()
 
 
 def _l2_setting(mode, trust, min_k):
     if mode not in _L2_MODES:
-        raise ValueError(f"l2 mode must be 'direct', 'gram' or 'gram_bf16', got {mode!r}")
+        raise ValueError(f"l2 mode must be 'direct', 'gram', 'gram_bf16' or 'auto', got {mode!r}")
     if trust is not None and not trust > 0.0:
         raise ValueError("trust must be positive")
     if min_k is not None and min_k < 0:
@@ -267,7 +270,7 @@ class _LaunchPlan:
     """Everything needed to launch: the C parameter block, the tensor that will
     be returned, and references that keep device memory alive until launch."""
 
-    __slots__ = ("params", "out", "keepalive", "swapped", "L", "M", "N", "K")
+    __slots__ = ("params", "out", "keepalive", "swapped", "L", "M", "N", "K", "l2_auto")
 
 
 def _plan_run_kernel(
@@ -410,13 +413,19 @@ def _plan_run_kernel(
         # (bit-identical result, about half the time); this keeps it to the full computation
         params.flags |= _backend.FLAG_NO_SYMMETRY
     l2 = _l2_current()
-    if (l2["mode"] in ("gram", "gram_bf16") and d._inner_operator is InnerOperator.DIFF
+    l2_auto = False
+    if (l2["mode"] != "direct" and d._inner_operator is InnerOperator.DIFF
             and d._inner_power is PowerType.SQUARE and K >= l2["min_k"]):
-        # also for the fused coefficient product (no out matrix here): it has a matrix-core variant too
-        params.flags |= _backend.FLAG_L2_GRAM
-        if l2["mode"] == "gram_bf16":
-            params.flags |= _backend.FLAG_L2_GRAM_BF16
-        params.gram_trust = _gram_trust(K, l2)
+        # "auto" leaves small problems (launches that take a few tens of microseconds: the two extra
+        # launches of the matrix-core path would show) to the direct kernel, and run_kernel gives it
+        # the calls whose grid it would rather cut over k
+        l2_auto = l2["mode"] == "auto"
+        if not l2_auto or float(L) * M * N * K >= _L2_AUTO_MIN_TERMS:
+            # also for the fused coefficient product (no out matrix here): it has a matrix-core variant too
+            params.flags |= _backend.FLAG_L2_GRAM
+            if l2["mode"] == "gram_bf16" or (l2_auto and stats_c is not None):
+                params.flags |= _backend.FLAG_L2_GRAM_BF16
+            params.gram_trust = _gram_trust(K, l2)
     params.m, params.n, params.k, params.l = M, N, K, L
     params.a, params.a_ld, params.a_bs = a.data_ptr(), stats_a.leading_dimension_stride, stats_a.batch_stride
     params.b, params.b_ld, params.b_bs = b.data_ptr(), stats_b.leading_dimension_stride, stats_b.batch_stride
@@ -432,6 +441,7 @@ def _plan_run_kernel(
     plan = _LaunchPlan()
     plan.params, plan.out, plan.keepalive, plan.swapped = params, out, keepalive, swapped
     plan.L, plan.M, plan.N, plan.K = L, M, N, K
+    plan.l2_auto = l2_auto
     return plan
 
 
@@ -519,12 +529,37 @@ def run_kernel(
                 print(f"(Kermac Debug) Launching kernel: {function_name}")
             _backend.build_kernel_jit(function, block, stream)
 
+    matrix_core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16
+    if plan.l2_auto and params.flags & matrix_core:
+        # a grid that the direct kernel would cut over k (a small result over a long contraction)
+        # stays with it: the matrix-core kernels are launched uncut
+        params.flags &= ~matrix_core
+        if _cut_over_contraction(params) is None:
+            params.flags |= matrix_core
     cut = _cut_over_contraction(params)
+    if params.flags & matrix_core:
+        plan.keepalive.append(_attach_gram_centre(params, stream, a.device))
     if cut is None:
         launch(params)
     else:
         _run_cut_over_contraction(cut, params, launch, stream, a.device)
     return plan.out
+
+
+def _attach_gram_centre(params, stream, device):
+    """Matrix-core launches subtract a point near the data from both operands while staging them
+    (include/kermac_amd.h, gram_centre): the mean of a sample of the rows of the first operand,
+    computed by the library into a small buffer allocated here.  KERMAC_AMD_L2_CENTRE=0 keeps the
+    operands as they are."""
+    if os.environ.get("KERMAC_AMD_L2_CENTRE", "1") in ("", "0") or params.m == 0 or params.k == 0 or params.l == 0:
+        return None
+    padded = -(-params.k // _backend.CENTRE_PAD) * _backend.CENTRE_PAD
+    batches = params.l if params.a_bs != 0 else 1
+    centre = torch.empty((batches, padded), dtype=torch.float32, device=device)
+    _backend.sample_mean(params.a, params.a_majorness, params.m, params.k, params.a_ld, params.a_bs, batches,
+                         centre.data_ptr(), padded, stream)
+    params.gram_centre, params.gram_centre_bs = centre.data_ptr(), (padded if batches > 1 else 0)
+    return centre
 
 
 # A workgroup owns one 128 x 128 tile of the result and walks the whole contraction index, so

@@ -107,6 +107,14 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
             return fail(KMC_ERR_INVALID_ARGUMENT, "k_total cannot be combined with the matrix-core flags");
     }
     args->k_total = p->k_total;
+    args->centre = nullptr;
+    args->centre_bs = 0;
+    if ((p->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16)) && p->gram_centre) {
+        if (!aligned16(p->gram_centre) || p->gram_centre_bs % 4 != 0 || p->gram_centre_bs < 0)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "gram_centre must be 16-byte aligned with a batch stride that is a multiple of 4");
+        args->centre = p->gram_centre;
+        args->centre_bs = p->gram_centre_bs;
+    }
     args->outer_power = p->outer_power;
     args->kernel_type = p->kernel_type;
     args->c_vec = need_c && !(p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) && aligned16(p->c) && p->c_ld % 4 == 0 &&

@@ -51,7 +51,13 @@ struct BuildKernelArgs {
     int k_total;         // 0, or: the batch entries are consecutive ranges of k terms of one contraction of
                          // k_total terms, and the last entry walks only what is left
     int grid_width;      // gridDim.x: tiles_m * tiles_n_padded, or (symmetric) the tiles of one triangle
+    // Matrix-core kernels only: a point c[k] (per batch entry, padded with zeros to a multiple of
+    // GRAM_CENTRE_PAD floats, 16-byte aligned) that is subtracted from both operands while they are
+    // staged; null: nothing is subtracted.
+    const float *centre; i64 centre_bs;
 };
+
+constexpr int GRAM_CENTRE_PAD = 64;
 
 constexpr int BK_TILE_M = 128;
 constexpr int BK_TILE_N = 128;
@@ -178,6 +184,27 @@ struct TileLoader {
     }
 
     __device__ __forceinline__ void advance() { ptr += step; }
+
+    // c[i] = centre[k of register i] for the current slice; `slice_centre` points at the slice's
+    // first k.  No predicates: the vector is padded with zeros past K.
+    __device__ __forceinline__ void load_centre(float (&c)[8], const float *slice_centre) const
+    {
+        if (MODE == LOAD_COL_VEC) {
+            const float lo = slice_centre[lane_k], hi = slice_centre[lane_k + 8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) c[i] = i < 4 ? lo : hi;
+        } else if (MODE == LOAD_COL_SCALAR) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) c[i] = slice_centre[lane_k + 2 * i];
+        } else if (MODE == LOAD_ROW_VEC) {
+            const float4 v = *reinterpret_cast<const float4 *>(slice_centre + lane_k);
+            c[0] = c[4] = v.x; c[1] = c[5] = v.y; c[2] = c[6] = v.z; c[3] = c[7] = v.w;
+        } else {
+            const float v = slice_centre[lane_k];
+#pragma unroll
+            for (int i = 0; i < 8; i++) c[i] = v;
+        }
+    }
 
     // Write the 8 registers into one LDS slice laid out [k][row] with pitch BK_LDS_PITCH.
     __device__ __forceinline__ void store(float *slice, const float (&r)[8]) const

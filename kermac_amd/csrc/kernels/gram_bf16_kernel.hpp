@@ -140,17 +140,25 @@ struct GramStep {
     static constexpr int value = N;
 };
 
-template <int LOAD_A, int LOAD_B, bool FULL, bool QUADS = false>
+template <int LOAD_A, int LOAD_B, bool FULL, bool CENTRED, bool QUADS = false>
 __device__ __forceinline__ void gram_bf16_walk(
     gram_float16 (&acc)[2][2], float &square_a, float &square_b, RowOwnerLoader<LOAD_A> &load_a,
     RowOwnerLoader<LOAD_B> &load_b, gram_chunk *lds_a, gram_chunk *lds_b, int k_total, int m_valid, int n_valid,
-    int wave_m, int wave_n, int h, int i)
+    int wave_m, int wave_n, int h, int i, const float *centre)
 {
+    typedef const float __attribute__((address_space(4))) *uniform_pointer;
+    constexpr bool COL_A = RowOwnerLoader<LOAD_A>::COL, COL_B = RowOwnerLoader<LOAD_B>::COL;
     const int k_slices = (k_total + BK_TILE_K - 1) / BK_TILE_K;
     const int k_tail = k_total - (k_slices - 1) * BK_TILE_K;
     // Raw values of two slices in flight: [set][operand][element].  A set that has no
     // slice to take holds zeros, which split into zeros and add nothing to the norms.
     float stage[2][2][8];
+    // The k of the centre (see gram_walk) that match a lane's 8 values, through scalar loads so
+    // that they cost no vector registers: the K half of a K-major loader is uniform over the wave
+    // (8 values: cen[set][half 0]); the lanes of a row-major loader alternate between the two
+    // halves, so both are fetched (16 values) and every lane picks its own when it subtracts.
+    // Loaders of one kind share them.
+    float cen[2][2][8];
 
     auto fetch = [&](auto set, int slice) {
         constexpr int S = decltype(set)::value;
@@ -164,9 +172,19 @@ __device__ __forceinline__ void gram_bf16_walk(
                 load_b.template load_part<!FULL, QUADS>(stage[S][1], which, n_valid, kv);
             load_a.advance();
             load_b.advance();
+            if (CENTRED) {
+                const uniform_pointer of_slice = (uniform_pointer)(centre + slice * BK_TILE_K);
+                // the half of a K-major loader, or both halves for a row-major one
+                const int first = COL_A ? 8 * load_a.half : (COL_B ? 8 * load_b.half : 0);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    cen[S][0][e] = of_slice[first + e];
+                    if (!COL_A || !COL_B) cen[S][1][e] = of_slice[(COL_A || COL_B ? 0 : 8) + e + (COL_A != COL_B ? 8 * (1 - (COL_A ? load_a.half : load_b.half)) : 0)];
+                }
+            }
         } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) stage[S][0][e] = stage[S][1][e] = 0.0f;
+            for (int e = 0; e < 8; e++) stage[S][0][e] = stage[S][1][e] = cen[S][0][e] = cen[S][1][e] = 0.0f;
         }
     };
     const int write_a = load_a.half * BK_TILE_M + load_a.row;
@@ -184,6 +202,15 @@ __device__ __forceinline__ void gram_bf16_walk(
         constexpr int PART = decltype(part)::value;
         constexpr int pair = PART / 3, phase = PART % 3;
         constexpr int operand = pair / 4, q = pair % 4;
+        if (phase == 0 && CENTRED) {
+            constexpr bool col = operand == 0 ? COL_A : COL_B;
+            // cen[S][0] is the half of the K-major loader if there is one, else half 0; cen[S][1] the other half
+            const int uniform_half = COL_A ? load_a.half : load_b.half;     // meaningful when one loader is K-major
+            const int lane_half = operand == 0 ? load_a.half : load_b.half;
+            const bool other = col ? false : ((COL_A || COL_B) ? lane_half != uniform_half : lane_half != 0);
+            stage[S][operand][2 * q] -= other ? cen[S][1][2 * q] : cen[S][0][2 * q];
+            stage[S][operand][2 * q + 1] -= other ? cen[S][1][2 * q + 1] : cen[S][0][2 * q + 1];
+        }
         const float x0 = stage[S][operand][2 * q], x1 = stage[S][operand][2 * q + 1];
         if (phase == 0) {
             float &square = operand == 0 ? square_a : square_b;
@@ -263,7 +290,9 @@ __device__ __forceinline__ void gram_bf16_walk(
 // A kernel of its own because the two kinds of predicated loads side by side cost the
 // unpredicated walk of the same kernel 20 % (register allocation), and with a register
 // budget for two waves per SIMD: within the budget for three the compiler spills 180.
-template <int LOAD_A, int LOAD_B, bool RAGGED_K = false>
+// CENTRED: args.centre is subtracted from both operands while they are staged (a kernel of its
+// own: a run-time switch inside the walk breaks the interleaving of matrix instructions and split).
+template <int LOAD_A, int LOAD_B, bool RAGGED_K = false, bool CENTRED = false>
 __global__ __launch_bounds__(BK_THREADS, RAGGED_K ? 2 : GB_WAVES) void gram_bf16_l2_kernel(const BuildKernelArgs args)
 {
     __shared__ gram_chunk lds_a[2 * GB_PANEL_CHUNKS];
@@ -301,15 +330,16 @@ __global__ __launch_bounds__(BK_THREADS, RAGGED_K ? 2 : GB_WAVES) void gram_bf16
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[mt][nt][v] = 0.0f;
 
+    const float *centre = CENTRED ? args.centre + batch * args.centre_bs : nullptr;
     if (RAGGED_K) {
-        gram_bf16_walk<LOAD_A, LOAD_B, false, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k,
-                                                    m_valid, n_valid, wave_m, wave_n, h, i);
+        gram_bf16_walk<LOAD_A, LOAD_B, false, CENTRED, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k,
+                                                    m_valid, n_valid, wave_m, wave_n, h, i, centre);
     } else if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
-        gram_bf16_walk<LOAD_A, LOAD_B, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
-                                             n_valid, wave_m, wave_n, h, i);
+        gram_bf16_walk<LOAD_A, LOAD_B, true, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
+                                             n_valid, wave_m, wave_n, h, i, centre);
     } else {
-        gram_bf16_walk<LOAD_A, LOAD_B, false>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
-                                              n_valid, wave_m, wave_n, h, i);
+        gram_bf16_walk<LOAD_A, LOAD_B, false, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
+                                              n_valid, wave_m, wave_n, h, i, centre);
     }
 
     // Row norms: low K half first, so that the same point gets the same norm in every

@@ -12,10 +12,13 @@ static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStr
 {
     constexpr bool has_ragged_variant = LOAD_A == kmc::LOAD_ROW_VEC || LOAD_B == kmc::LOAD_ROW_VEC;
     hipError_t status;
-    if (has_ragged_variant && args.k % kmc::BK_TILE_K != 0) {
-        status = launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B, has_ragged_variant>, grid, dim3(kmc::BK_THREADS), stream, args);
+    const bool ragged = has_ragged_variant && args.k % kmc::BK_TILE_K != 0;
+    if (args.centre) {
+        status = ragged ? launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B, has_ragged_variant, true>, grid, dim3(kmc::BK_THREADS), stream, args)
+                        : launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B, false, true>, grid, dim3(kmc::BK_THREADS), stream, args);
     } else {
-        status = launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
+        status = ragged ? launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B, has_ragged_variant>, grid, dim3(kmc::BK_THREADS), stream, args)
+                        : launch(kmc::gram_bf16_l2_kernel<LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
     }
     return status;
 }

@@ -21,7 +21,7 @@
 
 namespace kmc {
 
-template <int LOAD_A, int LOAD_B>
+template <int LOAD_A, int LOAD_B, bool CENTRED = false>
 __global__ __launch_bounds__(BK_THREADS, 2) void gram_times_coefficients(const KernelCoefficientsArgs kc)
 {
     static_assert(GRAM_DEPTH == 1, "the staging buffers below hold one slice per stage");
@@ -121,12 +121,13 @@ __global__ __launch_bounds__(BK_THREADS, 2) void gram_times_coefficients(const K
                     for (int v = 0; v < 16; v++) acc[mt][nt][v] = 0.0f;
             const float *frag_a = lds_a + h * BK_LDS_PITCH + wave_m + i;
             const float *frag_b = lds_b + h * BK_LDS_PITCH + wave_n + i;
+            const float *centre = CENTRED ? args.centre + batch * args.centre_bs : nullptr;
             if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % GRAM_STAGE_K == 0) {
-                gram_walk<LOAD_A, LOAD_B, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
-                                                args.k, m_valid, n_valid);
+                gram_walk<LOAD_A, LOAD_B, true, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
+                                                args.k, m_valid, n_valid, centre);
             } else {
-                gram_walk<LOAD_A, LOAD_B, false>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
-                                                 args.k, m_valid, n_valid);
+                gram_walk<LOAD_A, LOAD_B, false, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a,
+                                                          frag_b, args.k, m_valid, n_valid, centre);
             }
             row_norms<LOAD_A>(load_a, square_a, lds_a, lds_norm_a, tid);
             row_norms<LOAD_B>(load_b, square_b, lds_b, lds_norm_b, tid);
@@ -150,7 +151,8 @@ __global__ __launch_bounds__(BK_THREADS, 2) void gram_times_coefficients(const K
                     for (int nt = 0; nt < 2; nt++) {
                         const float norms = norm_a + norm_b[nt];
                         float d2 = norms - 2.0f * acc[mt][nt][v];
-                        if (m_local < m_valid && n_local[nt] < n_valid && d2 < args.gram_trust * norms) distrust = 1;
+                        // a result that is not a number (inf - inf of huge operands) is not trusted either
+                        if (m_local < m_valid && n_local[nt] < n_valid && !(d2 >= args.gram_trust * norms)) distrust = 1;
                         d2 = fmaxf(d2, 0.0f);
                         float value = epilogue_value(d2, outer_power, kernel_type, p_outer, neg_gamma, args.epsilon);
                         if (regularize && args.reg_off_x + m0 + m_local == args.reg_off_y + n0 + n_local[nt])

@@ -81,16 +81,22 @@ constexpr int GRAM_STAGE_FLOATS = GRAM_DEPTH * BK_LDS_SLICE;   // per operand an
 // stage t+1 in flight while stage t is consumed), feed the matrix cores, and keep
 // per-register sums of squares of everything staged.  FULL = no load needs a
 // predicate.  Ends with a barrier.
-template <int LOAD_A, int LOAD_B, bool FULL>
+template <int LOAD_A, int LOAD_B, bool FULL, bool CENTRED>
 __device__ __forceinline__ void gram_walk(
     gram_float16 (&acc)[2][2], float (&square_a)[8], float (&square_b)[8],
     TileLoader<LOAD_A> &load_a, TileLoader<LOAD_B> &load_b, float *lds_a, float *lds_b,
-    const float *frag_a, const float *frag_b, int k_total, int m_valid, int n_valid)
+    const float *frag_a, const float *frag_b, int k_total, int m_valid, int n_valid, const float *centre)
 {
     const int k_slices = (k_total + BK_TILE_K - 1) / BK_TILE_K;
     const int k_tail = k_total - (k_slices - 1) * BK_TILE_K;
     const int stages = (k_slices + GRAM_DEPTH - 1) / GRAM_DEPTH;
     float stage_a[GRAM_DEPTH][8], stage_b[GRAM_DEPTH][8];
+    // CENTRED: `centre` is subtracted from everything that is staged: distances do not
+    // change, but norms and dot products shrink to the spread of the data around that point, and
+    // with them the error of |a|^2 + |b|^2 - 2 a.b.  Rows past M / N become -centre; they are
+    // never stored.  Both loaders of one mode hold the same k per register.
+    float centre_a[GRAM_DEPTH][8], centre_b[GRAM_DEPTH][8];
+    const float *next_centre = centre;
 
     // The loaders point at the next slice to fetch and move on after every fetch.
     auto fetch = [&](int stage) {
@@ -106,6 +112,11 @@ __device__ __forceinline__ void gram_walk(
                 load_a.load_edge(stage_a[d], m_valid, kv);    // zero fill: adds 0 to norms and dot products
                 load_b.load_edge(stage_b[d], n_valid, kv);
             }
+            if (CENTRED) {
+                load_a.load_centre(centre_a[d], next_centre);
+                if (LOAD_A != LOAD_B) load_b.load_centre(centre_b[d], next_centre);
+                next_centre += BK_TILE_K;
+            }
             load_a.advance();
             load_b.advance();
         }
@@ -115,6 +126,10 @@ __device__ __forceinline__ void gram_walk(
         for (int d = 0; d < GRAM_DEPTH; d++) {
 #pragma unroll
             for (int s = 0; s < 8; s++) {
+                if (CENTRED) {
+                    stage_a[d][s] -= centre_a[d][s];
+                    stage_b[d][s] -= LOAD_A != LOAD_B ? centre_b[d][s] : centre_a[d][s];
+                }
                 square_a[s] += stage_a[d][s] * stage_a[d][s];
                 square_b[s] += stage_b[d][s] * stage_b[d][s];
             }
@@ -167,7 +182,8 @@ __device__ __forceinline__ void gram_walk(
     }
 }
 
-template <int LOAD_A, int LOAD_B>
+// CENTRED: args.centre is subtracted from both operands while they are staged.
+template <int LOAD_A, int LOAD_B, bool CENTRED = false>
 __global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const BuildKernelArgs args)
 {
     __shared__ __attribute__((aligned(16))) float lds_a[2 * GRAM_STAGE_FLOATS];
@@ -209,12 +225,13 @@ __global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const B
 
     const float *frag_a = lds_a + h * BK_LDS_PITCH + wave_m + i;
     const float *frag_b = lds_b + h * BK_LDS_PITCH + wave_n + i;
+    const float *centre = CENTRED ? args.centre + batch * args.centre_bs : nullptr;
     if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % GRAM_STAGE_K == 0) {
-        gram_walk<LOAD_A, LOAD_B, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
-                                        args.k, m_valid, n_valid);
+        gram_walk<LOAD_A, LOAD_B, true, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
+                                        args.k, m_valid, n_valid, centre);
     } else {
-        gram_walk<LOAD_A, LOAD_B, false>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
-                                         args.k, m_valid, n_valid);
+        gram_walk<LOAD_A, LOAD_B, false, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
+                                                  args.k, m_valid, n_valid, centre);
     }
 
     // Row norms, summed in a fixed order so that the same point gets the same norm

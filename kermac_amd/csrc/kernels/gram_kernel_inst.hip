@@ -10,6 +10,7 @@ namespace kmc_host {
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)
 {
+    if (args.centre) return launch(kmc::gram_l2_kernel<LOAD_A, LOAD_B, true>, grid, dim3(kmc::BK_THREADS), stream, args);
     return launch(kmc::gram_l2_kernel<LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
 }
 

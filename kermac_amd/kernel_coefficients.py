@@ -115,6 +115,9 @@ def run_kernel_coefficients(
     kernel = params.kernel
     aot = _backend.kernel_times_coefficients_has_variant(kernel.inner_operator, kernel.inner_power)
     matrix_core = bool(kernel.flags & _backend.FLAG_L2_GRAM)
+    if matrix_core:
+        from .build_a_kernel import _attach_gram_centre
+        plan.keepalive.append(_attach_gram_centre(kernel, stream, a.device))
     ranges = _centre_ranges(plan, three_resident=aot and not matrix_core and plan.O <= 32)
     partial = None
     if ranges > 1:

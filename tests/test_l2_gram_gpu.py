@@ -115,7 +115,7 @@ def test_empty_contraction_gives_zeros(device, gram_mode):
     assert torch.count_nonzero(out) == 0
 
 
-def test_bf16_flag_alone_through_the_c_abi(device):
+def test_bf16_flag_alone_through_the_c_abi(device, monkeypatch):
     """KMC_FLAG_L2_GRAM_BF16 implies the matrix-core path; a caller of the C ABI need not set both flags."""
     from kermac_amd import _backend
     from kermac_amd.build_a_kernel import _plan_run_kernel
@@ -129,11 +129,9 @@ def test_bf16_flag_alone_through_the_c_abi(device):
     plan.params.gram_trust = 0.25
     _backend.build_kernel(plan.params, torch.cuda.current_stream(device).cuda_stream)
     assert_close_to_truth(out, oracle.cdist(a.cpu(), b.cpu(), p=2.0), rtol=1e-5, what="bf16 flag alone")
-    kermac.set_l2_mode("gram_bf16", min_k=0)
-    try:
+    monkeypatch.setenv("KERMAC_AMD_L2_CENTRE", "0")          # the call above gave no gram_centre either
+    with kermac.l2_mode("gram_bf16", min_k=0):
         assert torch.equal(out, kermac.cdist(a, b, p=2.0))
-    finally:
-        kermac.set_l2_mode("direct")
 
 
 def test_full_size(device, gram_mode):
@@ -152,3 +150,58 @@ def test_full_size(device, gram_mode):
     self_out = kermac.cdist(a_store.t()[:5000], a_store.t()[:5000], p=2.0)[0]
     assert torch.all(torch.diagonal(self_out) == 0)
     assert torch.equal(self_out, self_out.t())
+
+
+@pytest.mark.parametrize("layout", ["cc", "rr", "cr", "rc"])
+def test_data_with_a_common_offset_stays_on_the_matrix_cores(device, gram_mode, monkeypatch, layout):
+    """Points in [100, 101]^K: around the origin the expansion |a|^2 + |b|^2 - 2 a.b cancels four
+    digits and every tile is recomputed by the direct kernel; around the centre that the Python
+    layer hands to the library (the mean of a sample of the rows of the first operand) the norms
+    are those of the spread, the tiles stay trusted, and the result keeps the stated tolerance.
+    That the matrix-core values were kept shows in the bits: a repaired tile equals the direct
+    kernel's result exactly."""
+    g = torch.Generator().manual_seed(17)
+    M, N, K = 300, 260, 96
+    a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False, dist="rand") + 100.0
+    b = make_operand(1, N, K, layout[1] == "c", device, g, batch=False, dist="rand") + 100.0
+    truth = oracle.cdist(a.cpu(), b.cpu(), p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        direct = kermac.cdist(a, b, p=2.0)[0]
+    centred = kermac.cdist(a, b, p=2.0)[0]
+    assert_close_to_truth(centred, truth, rtol=1e-5, what=f"offset data, centred, {layout}")
+    assert not torch.equal(centred, direct), "every tile was repaired: the centre did not take effect"
+    monkeypatch.setenv("KERMAC_AMD_L2_CENTRE", "0")
+    uncentred = kermac.cdist(a, b, p=2.0)[0]
+    assert torch.equal(uncentred, direct), "without a centre every tile of this data must be distrusted and repaired"
+    # batched, the centre per batch entry; a broadcast first operand has one
+    monkeypatch.setenv("KERMAC_AMD_L2_CENTRE", "1")
+    shifts = torch.tensor([0.0, 50.0, -30.0], device=device)[:, None, None]
+    ab = (a - 100.0)[None] + shifts
+    bb = (b - 100.0)[None] + shifts
+    got = kermac.cdist(ab, bb, p=2.0)
+    for l in range(3):
+        assert_close_to_truth(got[l], oracle.cdist(ab[l].cpu(), bb[l].cpu(), p=2.0)[0], rtol=1e-5, what=f"batch {l}")
+    got = kermac.cdist(a, bb + 100.0 - shifts, p=2.0)
+    assert_close_to_truth(got[2], truth, rtol=1e-5, what="broadcast first operand")
+
+
+def test_sample_mean_through_the_c_abi(device):
+    """kmc_sample_mean: whole panels up to 4096 rows, 16 runs of 256 rows beyond; zero padding to 64."""
+    from kermac_amd import _backend
+    g = torch.Generator().manual_seed(23)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    for rows, K, col_major, L in ((1, 1, False, 1), (300, 70, False, 2), (300, 70, True, 2), (5000, 33, True, 1), (9000, 130, False, 3)):
+        x = make_operand(L, rows, K, col_major, device, g, dist="rand") + 3.0
+        padded = -(-K // 64) * 64
+        mean = torch.full((L, padded + 5), -1.0, device=device)
+        ld = x.stride(2) if col_major else x.stride(1)
+        _backend.sample_mean(x.data_ptr(), _backend.COL_MAJOR if col_major else _backend.ROW_MAJOR, rows, K, ld, x.stride(0), L,
+                             mean.data_ptr(), padded + 5, stream)
+        torch.cuda.synchronize()
+        if rows <= 4096:
+            sample = x
+        else:
+            starts = [(j * (rows - 256)) // 15 for j in range(16)]
+            sample = torch.cat([x[:, s:s + 256] for s in starts], dim=1)
+        assert_close_to_truth(mean[:, :K], sample.double().mean(dim=1), rtol=1e-5, what=f"sample mean rows={rows} K={K}")
+        assert torch.all(mean[:, K:padded] == 0.0) and torch.all(mean[:, padded:] == -1.0)
