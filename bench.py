@@ -7,10 +7,12 @@ One "step" is one ``kermac_amd.cdist`` call on the headline configuration:
 a_store[K=1024, M=30000], b_store[K=1024, N=30000] ~ N(0,1) (seed 1), passed as
 K-major panels, out_store[N, M] fp32 (3.6 GB), p = 1.0.  Inputs and the output
 buffer are resident in HBM before the timed region.  The same data is then timed
-for p = 2.0 and p = 1.3 (with and without the 1/p epilogue) and reported in
-``per_p``.  Work is counted as 3 fp32 operations per (m, n, k) -- subtract,
+for p = 2.0 (the default mode, which puts this problem on the matrix cores, and the
+vector-ALU kernel by name) and p = 1.3 (with and without the 1/p epilogue) and reported in
+``per_p``; ``other_configs`` holds the gradient and the fused kernel-matrix x coefficients
+configurations.  Work is counted as 3 fp32 operations per (m, n, k) -- subtract,
 power, accumulate -- i.e. 3*M*N*K = 2.7648e12 per call, against the published
-fp32 vector peak of 157.3 TFLOP/s.
+fp32 vector peak of 157.3 TFLOP/s.  The last leg times torch.cdist on the host cores.
 
 Prints ONE JSON line on stdout; progress goes to stderr.
 """
@@ -265,7 +267,8 @@ def bench_kernel_coef(kermac, device, args, steps=None, warmup=None, with_gaussi
         gaussian = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP,
                                            kermac.KernelType.GAUSSIAN)
         call = lambda: kermac.run_kernel(gaussian, x.transpose(1, 2), z.t(), out=out, bandwidth=9.0, coefficients=coef)
-        _, gaussian_ms = time_call(call, side_steps, 1)
+        with kermac.l2_mode("direct"):
+            _, gaussian_ms = time_call(call, side_steps, 1)
         with kermac.l2_mode("gram"):
             _, gaussian_mfma_ms = time_call(call, side_steps, 1)
         d2 = torch.cdist(x[0, :, rows].t().double(), z.t().double(), p=2.0) ** 2
@@ -276,7 +279,7 @@ def bench_kernel_coef(kermac, device, args, steps=None, warmup=None, with_gaussi
         check_parity("gaussian x coefficients (matrix cores) slab, max abs err / mean |truth|", gaussian_err, 1e-4)
         extra["gaussian_same_shape"] = {"vector_ms": round(gaussian_ms, 3), "matrix_core_ms": round(gaussian_mfma_ms, 3),
                                         "matrix_core_parity_max_err_over_mean": gaussian_err,
-                                        "opt_in": "kermac_amd.l2_mode('gram')"}
+                                        "note": "matrix cores are what the default l2 mode 'auto' picks here"}
     ops = float(L) * nx * mz * (3 * k + 2 * o)
     nbytes = 4.0 * (L * k * nx + k * mz + 2 * L * nx * o)
     return side_line("fused Laplace kernel matrix x coefficients ms, L=4 N=M=16384 K=256 O=32",
@@ -309,6 +312,9 @@ def main():
     parser.add_argument("--only-p1", action="store_true", help="time only the headline p = 1.0 configuration")
     parser.add_argument("--only-p", type=float, default=None,
                         help="time only cdist with this p as the step (for profiling one kernel: 2.0, 1.3, ...)")
+    parser.add_argument("--l2-mode", choices=["auto", "direct", "gram", "gram_bf16"], default=None,
+                        help="how squared differences (p = 2) are evaluated in the timed step; default: the library's "
+                             "default, 'auto' (matrix cores with repair of ill-conditioned tiles for large problems)")
     parser.add_argument("--workload", choices=["cdist", "cdist_grad", "kernel_coef"], default="cdist",
                         help="cdist (default, the headline metric, with the other two configurations as extra keys); "
                              "cdist_grad = only the Laplace-kernel RFM gradient configuration; kernel_coef = only the "
@@ -325,6 +331,8 @@ def main():
 
     import kermac_amd as kermac
 
+    if args.l2_mode is not None:
+        kermac.set_l2_mode(args.l2_mode)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     if args.workload != "cdist":
@@ -352,24 +360,35 @@ def main():
 
     if not args.only_p1 and args.only_p is None:
         side_steps = max(2, min(args.steps, 5))
-        for p, skip, rtol in ((2.0, False, 1e-5), (1.3, False, 1e-4), (1.3, True, 1e-4)):
-            label = f"{p}" + ("_skip_epilogue" if skip else "")
+        for p, skip, rtol, mode in ((2.0, False, 1e-5, None), (2.0, False, 1e-5, "direct"), (1.3, False, 1e-4, None),
+                                    (1.3, True, 1e-4, None)):
+            label = f"{p}" + ("_skip_epilogue" if skip else "") + (f"_{mode}" if mode else "")
             log(f"timing p = {label}")
-            _, k_ms = time_cdist(kermac, a, b, out, p, skip, side_steps, 1)
+            with kermac.l2_mode(mode or kermac.get_l2_mode()):
+                _, k_ms = time_cdist(kermac, a, b, out, p, skip, side_steps, 1)
             e = parity_slab(out, a, b, p, skip)
             log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
             check_parity(f"cdist p={label} slab max rel err", e, rtol)
             per_p[label] = p_entry(k_ms, e, rtol)
+        per_p["2.0"]["l2_mode"] = kermac.get_l2_mode()
+        per_p["2.0"]["note"] = ("default mode 'auto': |a-c|^2 + |b-c|^2 - 2 (a-c).(b-c) with the cross term on the bf16 matrix "
+                                "instruction (three exact bf16 pieces per operand), c = sample mean, ill-conditioned tiles "
+                                "recomputed by the direct kernel; the vector-ALU kernel is per_p['2.0_direct']")
         # Fractional p costs five instructions per (m, n, k), two of them transcendentals that issue at a
-        # quarter of the rate (measured 19.3e12 lane-operations/s for v_exp_f32 / v_log_f32 against 66e12 for
-        # v_add_f32): 2 / 19.3e12 + 3 / 66e12 seconds per term is the issue floor of this instruction mix.
-        floor_ms = M * N * K * (2 / 19.3e12 + 3 / 66e12) * 1e3
+        # quarter of the rate.  Rates measured with kermac_amd/_lib/valu_issue_rates (examples/valu_issue_rates.hip):
+        # v_exp_f32 / v_log_f32 19.0e12 lane-operations/s, v_add_f32 65.4e12 -> 2 / 19.0e12 + 3 / 65.4e12 s per term
+        # is the sum of the parts; the kernel's own chain (sub, log2, mul, exp2, add) on registers alone runs at
+        # 27.86e12 lane-operations/s, i.e. 5 / 27.86e12 s per term: mixing the two kinds costs a fifth on top.
+        floor_ms = M * N * K * (2 / 19.0e12 + 3 / 65.4e12) * 1e3
+        chain_ms = M * N * K * 5 / 27.86e12 * 1e3
         for label in ("1.3", "1.3_skip_epilogue"):
             per_p[label]["issue_floor_ms"] = round(floor_ms, 1)
             per_p[label]["frac_of_issue_ceiling"] = round(floor_ms / per_p[label]["ms"], 4)
+            per_p[label]["isolated_chain_ms"] = round(chain_ms, 1)
+            per_p[label]["frac_of_isolated_chain"] = round(chain_ms / per_p[label]["ms"], 4)
 
-        # Opt-in matrix-core path for p = 2 (|a|^2 + |b|^2 - 2 a.b on fp32 MFMA, ill-conditioned tiles
-        # recomputed directly); same 1e-5 tolerance.  Reported beside the default direct path.
+        # The two matrix-core paths for p = 2 by name (|a|^2 + |b|^2 - 2 a.b on fp32 MFMA, ill-conditioned tiles
+        # recomputed directly); same 1e-5 tolerance.  The default 'auto' picks the second for this problem.
         # "gram_bf16": the cross term on the bf16 matrix instruction from three exact bf16 pieces per operand.
         for mode, label in (("gram", "2.0_gram_mfma"), ("gram_bf16", "2.0_gram_bf16_mfma")):
             log(f"timing p = 2.0, l2 mode '{mode}'")
@@ -379,7 +398,7 @@ def main():
             log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
             check_parity(f"cdist p=2.0 ({mode}) slab max rel err", e, 1e-5)
             per_p[label] = p_entry(k_ms, e, 1e-5, mfma_tflops=round((1 if mode == "gram" else 6) * 2.0 * M * N * K / k_ms / 1e9, 2),
-                                   opt_in=f"kermac_amd.l2_mode('{mode}')")
+                                   l2_mode=mode)
 
         # x against x (the kernel matrix of a training set): the library computes the tiles on and
         # below the diagonal only and stores each twice; bit-identical to the full computation.
@@ -406,6 +425,9 @@ def main():
     achieved = OPS_PER_CALL / kernel_ms / 1e9
     traffic, traffic_source = measured_traffic() if headline_p == 1.0 else (None, None)
     inner = {1.0: "POW_ABS", 2.0: "POW_SQUARE"}.get(headline_p, "POW_POW")
+    headline_kernel = f"kmc::build_kernel<OP_DIFF,{inner},LOAD_COL_VEC,LOAD_COL_VEC>"
+    if headline_p == 2.0 and kermac.get_l2_mode() != "direct":
+        headline_kernel = "kmc::gram_bf16_l2_kernel / kmc::gram_l2_kernel (l2 mode %s)" % kermac.get_l2_mode()
     line = {
         "metric": "cdist ms and % fp32-VALU peak at M=N=30000,K=1024 for p=1/1.3/2",
         "value": round(wall_ms, 3),
@@ -425,7 +447,7 @@ def main():
         "per_p": per_p,
         "roofline": {
             "bound": "valu_fp32",
-            "kernel": f"kmc::build_kernel<OP_DIFF,{inner},LOAD_COL_VEC,LOAD_COL_VEC>",
+            "kernel": headline_kernel,
             "achieved": round(achieved, 2),
             "peak": PEAK_FP32_VALU_TFLOPS,
             "unit": "TFLOP/s",

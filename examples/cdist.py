@@ -30,7 +30,7 @@ def parse_args():
     ap.add_argument("-a", "--try_align", action="store_true", help="accepted for compatibility (alignment is automatic)")
     ap.add_argument("-d", "--debug", action="store_true", help="print what is launched")
     ap.add_argument("-t", "--transposes", type=str, default=None, help="three of 'n'/'t' for a, b, out")
-    ap.add_argument("--l2_mode", choices=["direct", "gram", "gram_bf16"], default="direct", help="evaluation of p = 2 (see set_l2_mode)")
+    ap.add_argument("--l2_mode", choices=["auto", "direct", "gram", "gram_bf16"], default="auto", help="evaluation of p = 2 (see set_l2_mode)")
     ap.add_argument("--skip_numeric_compare", action="store_true", help="do not compare with torch.cdist")
     ap.add_argument("--skip_torch", action="store_true", help="do not run torch.cdist at all")
     ap.add_argument("--warmup", type=int, default=2)

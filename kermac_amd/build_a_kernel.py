@@ -202,7 +202,8 @@ _L2_AUTO_MIN_TERMS = 1e9          # "auto": below L * M * N * K terms the direct
 _L2_MODES = ("direct", "gram", "gram_bf16", "auto")
 # The process-wide setting, and per host thread what `l2_mode(...)` blocks have put on top
 # of it: two threads can evaluate squared differences in different modes at the same time.
-_l2_process = {"mode": os.environ.get("KERMAC_AMD_L2_MODE", "direct"), "trust": None, "min_k": _L2_DEFAULT_MIN_K}
+DEFAULT_L2_MODE = os.environ.get("KERMAC_AMD_L2_MODE", "auto")      # what the process starts with
+_l2_process = {"mode": DEFAULT_L2_MODE, "trust": None, "min_k": _L2_DEFAULT_MIN_K}
 if _l2_process["mode"] not in _L2_MODES:
     raise ValueError(f"KERMAC_AMD_L2_MODE must be one of {_L2_MODES}, got {_l2_process['mode']!r}")
 _l2_thread = threading.local()

@@ -30,7 +30,7 @@ CASES = (
 def gram_mode():
     kermac.set_l2_mode("gram", min_k=0)
     yield
-    kermac.set_l2_mode("direct")
+    kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
 
 
 def atol_for(truth, rtol):
@@ -86,7 +86,7 @@ def test_distrusted_tiles_take_the_direct_arithmetic(device):
     try:
         gram = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, z, bandwidth=3.0, coefficients=coef)
     finally:
-        kermac.set_l2_mode("direct")
+        kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
     assert torch.equal(gram, direct)
     truth = oracle.kernel_times_coefficients("DIFF", "SQUARE", "SQRT", "LAPLACE", x.cpu(), z.cpu(), coef.cpu(),
                                              bandwidth=3.0)
@@ -98,7 +98,7 @@ def test_distrusted_tiles_take_the_direct_arithmetic(device):
     try:
         mixed = kermac.run_kernel(GAUSSIAN, x, z2, bandwidth=4.0, coefficients=coef)
     finally:
-        kermac.set_l2_mode("direct")
+        kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
     truth = oracle.kernel_times_coefficients("DIFF", "SQUARE", "NOOP", "GAUSSIAN", x.cpu(), z2.cpu(), coef.cpu(),
                                              bandwidth=4.0)
     assert_close_to_truth(mixed, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="some tiles distrusted")

@@ -304,7 +304,7 @@ def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
         assert f & _backend.FLAG_L2_GRAM and f & _backend.FLAG_L2_GRAM_BF16 and trust == pytest.approx(0.25)
         assert flags(kermac.kernel_descriptor_l1_norm)[0] & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16) == 0
     finally:
-        kermac.set_l2_mode("direct")
+        kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
     # the default trust grows with K so that very long sums fall back to the direct kernel
     from kermac_amd.build_a_kernel import _gram_trust
     default = {"trust": None}
@@ -519,7 +519,7 @@ def test_l2_mode_blocks_are_per_thread():
     thread = threading.Thread(target=worker)
     thread.start()
     assert ready.wait(10)
-    assert kermac.get_l2_mode() == "direct"             # the other thread's block does not leak
+    assert kermac.get_l2_mode() == kermac.DEFAULT_L2_MODE             # the other thread's block does not leak
     with kermac.l2_mode("gram", trust=0.5):
         assert kermac.get_l2_mode() == "gram"
         plan = _plan_run_kernel(kermac.kernel_descriptor_l2_norm, torch.zeros(4, 64), torch.zeros(4, 64), None, None,
@@ -531,8 +531,8 @@ def test_l2_mode_blocks_are_per_thread():
         assert kermac.get_l2_mode() == "gram"
     release.set()
     thread.join()
-    assert seen == {"worker_inside": "gram_bf16", "worker_after": "direct"}
-    assert kermac.get_l2_mode() == "direct"
+    assert seen == {"worker_inside": "gram_bf16", "worker_after": kermac.DEFAULT_L2_MODE}
+    assert kermac.get_l2_mode() == kermac.DEFAULT_L2_MODE
     with pytest.raises(ValueError):
         with kermac.l2_mode("fast"):
             pass

@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 def gram_mode(request):
     kermac.set_l2_mode(request.param, min_k=0)      # also the short contractions, which would stay direct
     yield
-    kermac.set_l2_mode("direct")
+    kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
 
 
 def test_mode_switch_validation():
@@ -31,7 +31,7 @@ def test_mode_switch_validation():
         kermac.set_l2_mode("gram", trust=0.0)
     with pytest.raises(ValueError):
         kermac.set_l2_mode("gram", min_k=-1)
-    assert kermac.get_l2_mode() == "direct"
+    assert kermac.get_l2_mode() == kermac.DEFAULT_L2_MODE
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (128, 128, 16), (129, 127, 17), (300, 515, 70), (1000, 1000, 64),
@@ -205,3 +205,49 @@ def test_sample_mean_through_the_c_abi(device):
             sample = torch.cat([x[:, s:s + 256] for s in starts], dim=1)
         assert_close_to_truth(mean[:, :K], sample.double().mean(dim=1), rtol=1e-5, what=f"sample mean rows={rows} K={K}")
         assert torch.all(mean[:, K:padded] == 0.0) and torch.all(mean[:, padded:] == -1.0)
+
+
+def test_auto_mode_picks_the_kernel_by_shape(device):
+    """The default mode: squared differences go to the matrix cores (split-bf16 for a stored
+    matrix, fp32 for the fused coefficient product) when the problem is large enough to pay for
+    the two extra launches, to the direct kernel when it is small or when its grid is one that
+    the direct path would cut over k; everything else is untouched."""
+    from kermac_amd import _backend, build_a_kernel as module
+    from kermac_amd.kernel_coefficients import _plan_run_kernel_coefficients
+    assert kermac.get_l2_mode() == kermac.DEFAULT_L2_MODE == "auto"
+    core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16
+
+    def planned(M, N, K, descriptor=kermac.kernel_descriptor_l2_norm, **kw):
+        a = torch.empty(M, K, device=device)
+        b = torch.empty(N, K, device=device)
+        return module._plan_run_kernel(descriptor, a, b, None, kw.get("p"), None, None, kw.get("bandwidth"), None, None, 0, 0, False)
+
+    big = planned(4000, 4000, 128)
+    assert big.l2_auto and big.params.flags & core == core and big.params.gram_trust > 0
+    assert planned(500, 500, 128).params.flags & core == 0                       # 3.2e7 terms: direct
+    assert planned(4000, 4000, 32).params.flags & core == 0                      # K below min_k: direct
+    assert planned(4000, 4000, 128, kermac.kernel_descriptor_l1_norm).params.flags & core == 0
+    assert planned(4000, 4000, 128, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0).params.flags & core == core
+    a = torch.empty(4000, 128, device=device)
+    fused = _plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l2, a, a, torch.empty(4000, 8, device=device), None,
+                                          None, None, None, 2.0, None, None, 0, 0)
+    assert fused.params.kernel.flags & core == _backend.FLAG_L2_GRAM            # fp32 matrix instruction there
+    # a small result over a long contraction: marked, then handed back to the direct kernel and cut over k
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(300, 40000, generator=g).to(device)
+    y = torch.randn(280, 40000, generator=g).to(device)
+    assert planned(300, 280, 40000).params.flags & core == core
+    got = kermac.cdist(x, y, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0])
+    assert_close_to_truth(got, oracle.cdist(x.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, what="auto, long contraction")
+    # a large problem in auto mode equals the explicit split-bf16 mode, near-duplicate tiles included
+    g = torch.Generator().manual_seed(6)
+    points = torch.randn(2000, 256, generator=g)
+    points[1000:] = points[:1000] + 1e-4 * torch.randn(1000, 256, generator=g)       # every point has a near twin
+    points = points.to(device)
+    got = kermac.cdist(points, points.clone(), p=2.0)[0]
+    with kermac.l2_mode("gram_bf16"):
+        assert torch.equal(got, kermac.cdist(points, points.clone(), p=2.0)[0])
+    assert_close_to_truth(got, oracle.cdist(points.cpu(), points.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30,
+                          what="auto, near-duplicate points")

@@ -31,7 +31,7 @@ DESCRIPTORS = {
 def l2_mode(request):
     kermac.set_l2_mode(request.param, min_k=0)
     yield request.param
-    kermac.set_l2_mode("direct")
+    kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
 
 
 @pytest.mark.parametrize("name", list(DESCRIPTORS))
