@@ -149,8 +149,9 @@ typedef struct kmc_build_kernel_params {
      * in proportion to the norms: with a centre near the data (its mean: kmc_sample_mean) the
      * norms are those of the spread of the data, not of its offset from the origin, and tiles of
      * data with a common offset stay trusted instead of being recomputed.  16-byte aligned, the
-     * stride a multiple of 4, each vector padded with zeros to a multiple of 64 floats
-     * (kmc_sample_mean writes it that way).  NULL: nothing is subtracted. */
+     * stride a multiple of 4; each vector is padded with zeros to a multiple of 64 floats and
+     * followed by one float that says whether to subtract at all (0: this batch entry is taken
+     * as it is; kmc_sample_mean writes all of this).  NULL: nothing is subtracted. */
     const float *gram_centre;
     int64_t gram_centre_bs;
 } kmc_build_kernel_params;
@@ -181,8 +182,12 @@ int kmc_build_kernel_finish(const kmc_build_kernel_params *params, const float *
  * mean[l*mean_bs + k] = the mean over (a sample of) the rows of the panel x (addressed like the a
  * operand of kmc_build_kernel: majorness, ld, batch stride bs), for use as gram_centre.  Panels
  * of up to 4096 rows are averaged whole, longer ones over 16 evenly spaced runs of 256 rows;
- * the sums run in a fixed order.  Every vector is padded with zeros to a multiple of 64 floats,
- * so mean needs (l - 1) * mean_bs + roundup(k, 64) floats.  No counterpart in the reference.
+ * the sums run in a fixed order.  Per batch entry the call writes 2 * roundup(k, 64) + 64 floats
+ * (mean_bs must be at least that for l > 1): the mean padded with zeros to a multiple of 64, a
+ * flag in the next float -- 1, or 0 when the mean is so close to the origin against the spread of
+ * the rows around it (|mean|^2 <= variance / 64) that subtracting it would change nothing worth
+ * its cost; the matrix-core kernels read it -- then 63 unused floats and the variance per k.
+ * Two small launches on the stream.  No counterpart in the reference.
  */
 int kmc_sample_mean(const float *x, int32_t majorness, int32_t rows, int32_t k, int64_t ld, int64_t bs, int32_t l,
                     float *mean, int64_t mean_bs, void *stream);

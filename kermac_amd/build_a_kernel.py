@@ -198,7 +198,7 @@ def _hyper_parameter(name, value, L, device, require_device):
 #   launches are bound by the result stores, and the direct kernel has the cheaper
 #   epilogue and no repair launch (M = N = 30000, K = 16: 1.2 ms against 2.4 .. 2.6 ms).
 _L2_DEFAULT_MIN_K = 64
-_L2_AUTO_MIN_TERMS = 1e9          # "auto": below L * M * N * K terms the direct kernel is launched
+_L2_AUTO_MIN_TERMS = 5e8          # "auto": below L * M * N * K terms the direct kernel is launched
 _L2_MODES = ("direct", "gram", "gram_bf16", "auto")
 # The process-wide setting, and per host thread what `l2_mode(...)` blocks have put on top
 # of it: two threads can evaluate squared differences in different modes at the same time.
@@ -554,12 +554,14 @@ def _attach_gram_centre(params, stream, device):
     operands as they are."""
     if os.environ.get("KERMAC_AMD_L2_CENTRE", "1") in ("", "0") or params.m == 0 or params.k == 0 or params.l == 0:
         return None
-    padded = -(-params.k // _backend.CENTRE_PAD) * _backend.CENTRE_PAD
+    # per batch entry: the centre padded to a multiple of 64 floats, a flag (subtract or not: the
+    # library leaves it out when the centre is negligible against the spread) and the variances
+    width = 2 * (-(-params.k // _backend.CENTRE_PAD) * _backend.CENTRE_PAD) + _backend.CENTRE_PAD
     batches = params.l if params.a_bs != 0 else 1
-    centre = torch.empty((batches, padded), dtype=torch.float32, device=device)
+    centre = torch.empty((batches, width), dtype=torch.float32, device=device)
     _backend.sample_mean(params.a, params.a_majorness, params.m, params.k, params.a_ld, params.a_bs, batches,
-                         centre.data_ptr(), padded, stream)
-    params.gram_centre, params.gram_centre_bs = centre.data_ptr(), (padded if batches > 1 else 0)
+                         centre.data_ptr(), width, stream)
+    params.gram_centre, params.gram_centre_bs = centre.data_ptr(), (width if batches > 1 else 0)
     return centre
 
 

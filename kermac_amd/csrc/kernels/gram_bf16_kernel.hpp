@@ -330,17 +330,22 @@ __global__ __launch_bounds__(BK_THREADS, RAGGED_K ? 2 : GB_WAVES) void gram_bf16
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[mt][nt][v] = 0.0f;
 
-    const float *centre = CENTRED ? args.centre + batch * args.centre_bs : nullptr;
-    if (RAGGED_K) {
-        gram_bf16_walk<LOAD_A, LOAD_B, false, CENTRED, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k,
-                                                    m_valid, n_valid, wave_m, wave_n, h, i, centre);
-    } else if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
-        gram_bf16_walk<LOAD_A, LOAD_B, true, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
-                                             n_valid, wave_m, wave_n, h, i, centre);
-    } else {
-        gram_bf16_walk<LOAD_A, LOAD_B, false, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
-                                              n_valid, wave_m, wave_n, h, i, centre);
-    }
+    const float *centre = CENTRED ? centre_to_subtract(args, batch) : nullptr;
+    auto walk = [&](auto centred) {
+        constexpr bool C = decltype(centred)::value;
+        if (RAGGED_K) {
+            gram_bf16_walk<LOAD_A, LOAD_B, false, C, true>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
+                                                           n_valid, wave_m, wave_n, h, i, centre);
+        } else if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % BK_TILE_K == 0) {
+            gram_bf16_walk<LOAD_A, LOAD_B, true, C>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
+                                                    n_valid, wave_m, wave_n, h, i, centre);
+        } else {
+            gram_bf16_walk<LOAD_A, LOAD_B, false, C>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, args.k, m_valid,
+                                                     n_valid, wave_m, wave_n, h, i, centre);
+        }
+    };
+    if (CENTRED && centre) walk(GramSwitch<CENTRED>{});
+    else walk(GramSwitch<false>{});
 
     // Row norms: low K half first, so that the same point gets the same norm in every
     // workgroup and on either side.  The buffers of the walk are free by now.

@@ -121,14 +121,19 @@ __global__ __launch_bounds__(BK_THREADS, 2) void gram_times_coefficients(const K
                     for (int v = 0; v < 16; v++) acc[mt][nt][v] = 0.0f;
             const float *frag_a = lds_a + h * BK_LDS_PITCH + wave_m + i;
             const float *frag_b = lds_b + h * BK_LDS_PITCH + wave_n + i;
-            const float *centre = CENTRED ? args.centre + batch * args.centre_bs : nullptr;
-            if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % GRAM_STAGE_K == 0) {
-                gram_walk<LOAD_A, LOAD_B, true, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
-                                                args.k, m_valid, n_valid, centre);
-            } else {
-                gram_walk<LOAD_A, LOAD_B, false, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a,
-                                                          frag_b, args.k, m_valid, n_valid, centre);
-            }
+            const float *centre = CENTRED ? centre_to_subtract(args, batch) : nullptr;
+            auto walk = [&](auto centred) {
+                constexpr bool C = decltype(centred)::value;
+                if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % GRAM_STAGE_K == 0) {
+                    gram_walk<LOAD_A, LOAD_B, true, C>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
+                                                       args.k, m_valid, n_valid, centre);
+                } else {
+                    gram_walk<LOAD_A, LOAD_B, false, C>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
+                                                        args.k, m_valid, n_valid, centre);
+                }
+            };
+            if (CENTRED && centre) walk(GramSwitch<CENTRED>{});
+            else walk(GramSwitch<false>{});
             row_norms<LOAD_A>(load_a, square_a, lds_a, lds_norm_a, tid);
             row_norms<LOAD_B>(load_b, square_b, lds_b, lds_norm_b, tid);
             __syncthreads();

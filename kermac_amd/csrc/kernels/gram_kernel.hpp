@@ -33,6 +33,23 @@ namespace kmc {
 
 typedef float gram_float16 __attribute__((ext_vector_type(16)));
 
+template <bool B>
+struct GramSwitch {
+    static constexpr bool value = B;
+};
+
+// The centre of batch entry `batch` if it is to be subtracted, else null.  The vector (k floats,
+// padded with zeros to a multiple of GRAM_CENTRE_PAD) is followed by a flag: 0 says that the
+// centre is too close to the origin to matter (kmc_sample_mean decides), and the walk then leaves
+// the subtraction out.  Uniform over the workgroup.
+__device__ __forceinline__ const float *centre_to_subtract(const BuildKernelArgs &args, int batch)
+{
+    if (!args.centre) return nullptr;
+    const float *centre = args.centre + batch * args.centre_bs;
+    const int padded = (args.k + GRAM_CENTRE_PAD - 1) / GRAM_CENTRE_PAD * GRAM_CENTRE_PAD;
+    return centre[padded] != 0.0f ? centre : nullptr;
+}
+
 // norm[row] = sum over everything the workgroup staged for that row of `square`.
 // `partial` is scratch for lanes_per_row() x 128 floats.  Contains one barrier;
 // the caller adds another before reading `norm`.
@@ -225,14 +242,19 @@ __global__ __launch_bounds__(BK_THREADS, GRAM_WAVES) void gram_l2_kernel(const B
 
     const float *frag_a = lds_a + h * BK_LDS_PITCH + wave_m + i;
     const float *frag_b = lds_b + h * BK_LDS_PITCH + wave_n + i;
-    const float *centre = CENTRED ? args.centre + batch * args.centre_bs : nullptr;
-    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % GRAM_STAGE_K == 0) {
-        gram_walk<LOAD_A, LOAD_B, true, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
-                                        args.k, m_valid, n_valid, centre);
-    } else {
-        gram_walk<LOAD_A, LOAD_B, false, CENTRED>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b,
-                                                  args.k, m_valid, n_valid, centre);
-    }
+    const float *centre = CENTRED ? centre_to_subtract(args, batch) : nullptr;
+    auto walk = [&](auto centred) {
+        constexpr bool C = decltype(centred)::value;
+        if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && args.k % GRAM_STAGE_K == 0) {
+            gram_walk<LOAD_A, LOAD_B, true, C>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b, args.k,
+                                               m_valid, n_valid, centre);
+        } else {
+            gram_walk<LOAD_A, LOAD_B, false, C>(acc, square_a, square_b, load_a, load_b, lds_a, lds_b, frag_a, frag_b, args.k,
+                                                m_valid, n_valid, centre);
+        }
+    };
+    if (CENTRED && centre) walk(GramSwitch<CENTRED>{});
+    else walk(GramSwitch<false>{});
 
     // Row norms, summed in a fixed order so that the same point gets the same norm
     // in every workgroup (results are reproducible and x-vs-x matrices symmetric):

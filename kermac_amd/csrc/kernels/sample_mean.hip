@@ -4,7 +4,12 @@
 // those around the centre).  Up to 4096 rows are averaged exactly as given; of a longer panel
 // 16 runs of 256 consecutive rows, evenly spaced from the first row to the last.  The sums run
 // in a fixed order, so the same panel always gives the same centre.  The result is padded with
-// zeros to a multiple of GRAM_CENTRE_PAD floats, as the kernels expect it.
+// zeros to a multiple of GRAM_CENTRE_PAD floats, as the kernels expect it, and followed by a
+// flag: 1 when subtracting the centre is worth its cost, 0 when the centre is so close to the
+// origin, measured against the spread of the sampled rows around it (|c|^2 <= spread^2 / 64), that
+// the norms -- and with them the cancellation -- would change by less than 2 %.  The matrix-core
+// kernels then skip the subtraction for that batch entry.  Layout per batch entry:
+// [centre, padded][flag, 63 unused floats][variance per k, padded] = 2 * padded + 64 floats.
 #include <hip/hip_runtime.h>
 
 #include "../host/host_common.hpp"
@@ -19,6 +24,12 @@ struct SampleMeanArgs {
     float *mean; i64 mean_bs;
     int samples;         // rows that are averaged
 };
+
+// mean of squares minus square of mean, per k, goes behind the centre and its flag
+__device__ __forceinline__ float *variance_of(const SampleMeanArgs &args, int batch)
+{
+    return args.mean + batch * args.mean_bs + args.k_padded + GRAM_CENTRE_PAD;
+}
 
 constexpr int SM_MAX_SAMPLES = 4096;
 constexpr int SM_RUN = 256;
@@ -38,14 +49,24 @@ __global__ __launch_bounds__(256) void sample_mean_rows(const SampleMeanArgs arg
     const int kk = threadIdx.x & 63, group = threadIdx.x >> 6;
     const int k = blockIdx.x * 64 + kk;
     const float *x = args.x + blockIdx.y * args.bs;
-    float sum = 0.0f;
+    __shared__ float partial_squares[4][64];
+    float sum = 0.0f, squares = 0.0f;
     if (k < args.k)
-        for (int s = group; s < args.samples; s += 4) sum += x[sampled_row(args, s) * args.ld + k];
+        for (int s = group; s < args.samples; s += 4) {
+            const float v = x[sampled_row(args, s) * args.ld + k];
+            sum += v;
+            squares += v * v;
+        }
     partial[group][kk] = sum;
+    partial_squares[group][kk] = squares;
     __syncthreads();
     if (group == 0 && k < args.k_padded) {
         const float total = ((partial[0][kk] + partial[1][kk]) + partial[2][kk]) + partial[3][kk];
-        args.mean[blockIdx.y * args.mean_bs + k] = (k < args.k && args.samples > 0) ? total / (float)args.samples : 0.0f;
+        const float total_squares = ((partial_squares[0][kk] + partial_squares[1][kk]) + partial_squares[2][kk]) + partial_squares[3][kk];
+        const bool live = k < args.k && args.samples > 0;
+        const float mean = live ? total / (float)args.samples : 0.0f;
+        args.mean[blockIdx.y * args.mean_bs + k] = mean;
+        variance_of(args, blockIdx.y)[k] = live ? fmaxf(total_squares / (float)args.samples - mean * mean, 0.0f) : 0.0f;
     }
 }
 
@@ -56,15 +77,55 @@ __global__ __launch_bounds__(256) void sample_mean_columns(const SampleMeanArgs 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int k = blockIdx.x * 4 + wave;
     const float *x = args.x + blockIdx.y * args.bs;
-    float sum = 0.0f;
+    __shared__ float partial_squares[4][64];
+    float sum = 0.0f, squares = 0.0f;
     if (k < args.k)
-        for (int s = lane; s < args.samples; s += 64) sum += x[(i64)k * args.ld + sampled_row(args, s)];
+        for (int s = lane; s < args.samples; s += 64) {
+            const float v = x[(i64)k * args.ld + sampled_row(args, s)];
+            sum += v;
+            squares += v * v;
+        }
     partial[wave][lane] = sum;
+    partial_squares[wave][lane] = squares;
     __syncthreads();
     if (lane == 0 && k < args.k_padded) {
-        float total = 0.0f;
-        for (int j = 0; j < 64; j++) total += partial[wave][j];
-        args.mean[blockIdx.y * args.mean_bs + k] = (k < args.k && args.samples > 0) ? total / (float)args.samples : 0.0f;
+        float total = 0.0f, total_squares = 0.0f;
+        for (int j = 0; j < 64; j++) {
+            total += partial[wave][j];
+            total_squares += partial_squares[wave][j];
+        }
+        const bool live = k < args.k && args.samples > 0;
+        const float mean = live ? total / (float)args.samples : 0.0f;
+        args.mean[blockIdx.y * args.mean_bs + k] = mean;
+        variance_of(args, blockIdx.y)[k] = live ? fmaxf(total_squares / (float)args.samples - mean * mean, 0.0f) : 0.0f;
+    }
+}
+
+// One workgroup per batch entry: |c|^2 against the summed variance, both added in a fixed order.
+__global__ __launch_bounds__(256) void centre_flag(const SampleMeanArgs args)
+{
+    __shared__ float norms[256], spreads[256];
+    const float *centre = args.mean + blockIdx.x * args.mean_bs;
+    const float *variance = variance_of(args, blockIdx.x);
+    float norm = 0.0f, spread = 0.0f;
+    for (int k = threadIdx.x; k < args.k; k += 256) {
+        norm += centre[k] * centre[k];
+        spread += variance[k];
+    }
+    norms[threadIdx.x] = norm;
+    spreads[threadIdx.x] = spread;
+    __syncthreads();
+    for (int width = 128; width > 0; width >>= 1) {
+        if ((int)threadIdx.x < width) {
+            norms[threadIdx.x] += norms[threadIdx.x + width];
+            spreads[threadIdx.x] += spreads[threadIdx.x + width];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x < GRAM_CENTRE_PAD) {
+        // not-a-number data: keep the subtraction (the comparison is false), the repair decides
+        const bool needless = norms[0] <= spreads[0] * (1.0f / 64.0f);
+        args.mean[blockIdx.x * args.mean_bs + args.k_padded + threadIdx.x] = (threadIdx.x == 0 && !needless) ? 1.0f : 0.0f;
     }
 }
 
@@ -82,8 +143,9 @@ extern "C" int kmc_sample_mean(const float *x, int32_t majorness, int32_t rows, 
     const int k_padded = (k + kmc::GRAM_CENTRE_PAD - 1) / kmc::GRAM_CENTRE_PAD * kmc::GRAM_CENTRE_PAD;
     if (k == 0 || l == 0) return KMC_OK;
     if (!mean || (rows > 0 && !x)) return fail(KMC_ERR_INVALID_ARGUMENT, "null pointer");
-    if (l > 1 && mean_bs < k_padded)
-        return fail(KMC_ERR_INVALID_ARGUMENT, "mean_bs = %lld is smaller than k padded to %d", static_cast<long long>(mean_bs), k_padded);
+    if (l > 1 && mean_bs < 2 * k_padded + kmc::GRAM_CENTRE_PAD)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "mean_bs = %lld is smaller than 2 * %d + %d", static_cast<long long>(mean_bs), k_padded,
+                    kmc::GRAM_CENTRE_PAD);
     int status = kmc_host::require_gfx950();
     if (status != KMC_OK) return status;
     kmc::SampleMeanArgs args;
@@ -97,5 +159,7 @@ extern "C" int kmc_sample_mean(const float *x, int32_t majorness, int32_t rows, 
     else
         e = kmc_host::launch(kmc::sample_mean_columns, dim3(k_padded / 4, l), dim3(256), static_cast<hipStream_t>(stream), args);
     if (e != hipSuccess) return kmc_host::fail_hip(e, "sample_mean launch");
+    e = kmc_host::launch(kmc::centre_flag, dim3(l), dim3(256), static_cast<hipStream_t>(stream), args);
+    if (e != hipSuccess) return kmc_host::fail_hip(e, "centre_flag launch");
     return KMC_OK;
 }

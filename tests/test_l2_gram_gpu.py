@@ -186,25 +186,52 @@ def test_data_with_a_common_offset_stays_on_the_matrix_cores(device, gram_mode, 
 
 
 def test_sample_mean_through_the_c_abi(device):
-    """kmc_sample_mean: whole panels up to 4096 rows, 16 runs of 256 rows beyond; zero padding to 64."""
+    """kmc_sample_mean: whole panels up to 4096 rows, 16 runs of 256 rows beyond; zero padding to 64,
+    then the flag (subtract or not) and, 64 floats on, the variance per k of the sampled rows."""
     from kermac_amd import _backend
     g = torch.Generator().manual_seed(23)
     stream = torch.cuda.current_stream(device).cuda_stream
-    for rows, K, col_major, L in ((1, 1, False, 1), (300, 70, False, 2), (300, 70, True, 2), (5000, 33, True, 1), (9000, 130, False, 3)):
-        x = make_operand(L, rows, K, col_major, device, g, dist="rand") + 3.0
+    cases = ((1, 1, False, 1, 3.0), (300, 70, False, 2, 3.0), (300, 70, True, 2, 0.0), (5000, 33, True, 1, 3.0),
+             (9000, 130, False, 3, 0.01), (9000, 130, True, 2, 0.2))
+    for rows, K, col_major, L, shift in cases:
+        x = make_operand(L, rows, K, col_major, device, g, dist="randn") + shift
         padded = -(-K // 64) * 64
-        mean = torch.full((L, padded + 5), -1.0, device=device)
+        width = 2 * padded + 64
+        mean = torch.full((L, width + 5), -1.0, device=device)
         ld = x.stride(2) if col_major else x.stride(1)
         _backend.sample_mean(x.data_ptr(), _backend.COL_MAJOR if col_major else _backend.ROW_MAJOR, rows, K, ld, x.stride(0), L,
-                             mean.data_ptr(), padded + 5, stream)
+                             mean.data_ptr(), width + 5, stream)
         torch.cuda.synchronize()
         if rows <= 4096:
             sample = x
         else:
             starts = [(j * (rows - 256)) // 15 for j in range(16)]
             sample = torch.cat([x[:, s:s + 256] for s in starts], dim=1)
-        assert_close_to_truth(mean[:, :K], sample.double().mean(dim=1), rtol=1e-5, what=f"sample mean rows={rows} K={K}")
-        assert torch.all(mean[:, K:padded] == 0.0) and torch.all(mean[:, padded:] == -1.0)
+        assert_close_to_truth(mean[:, :K], sample.double().mean(dim=1), rtol=1e-5, atol=1e-6,      # sums of values of order 1
+                              what=f"sample mean rows={rows} K={K}")
+        assert torch.all(mean[:, K:padded] == 0.0) and torch.all(mean[:, width:] == -1.0)
+        variance = mean[:, padded + 64:padded + 64 + K]
+        assert_close_to_truth(variance, sample.double().var(dim=1, unbiased=False), rtol=1e-3, atol=1e-6,
+                              what=f"sample variance rows={rows} K={K}")
+        # shift^2 * K against K / 64: only a centre well inside the cloud of points is left out
+        expect = 0.0 if shift * shift <= 1.0 / 256 else 1.0
+        assert torch.all(mean[:, padded] == expect), f"flag rows={rows} K={K} shift={shift}: {mean[:, padded].tolist()}"
+    with pytest.raises(_backend.BackendError, match="mean_bs"):
+        _backend.sample_mean(x.data_ptr(), _backend.ROW_MAJOR, rows, K, ld, x.stride(0), 2, mean.data_ptr(), padded, stream)
+
+
+def test_a_negligible_centre_is_left_out(device, gram_mode, monkeypatch):
+    """Points spread around the origin: the library sees that the sample mean is negligible against
+    the spread and runs the walk that subtracts nothing -- the bits equal those of a call without a
+    centre.  A centre that matters changes them."""
+    g = torch.Generator().manual_seed(31)
+    a = torch.randn(700, 256, generator=g).to(device)
+    b = torch.randn(650, 256, generator=g).to(device)
+    with_centre = kermac.cdist(a, b, p=2.0)
+    shifted = kermac.cdist(a + 1.0, b + 1.0, p=2.0)
+    monkeypatch.setenv("KERMAC_AMD_L2_CENTRE", "0")
+    assert torch.equal(with_centre, kermac.cdist(a, b, p=2.0))
+    assert not torch.equal(shifted, kermac.cdist(a + 1.0, b + 1.0, p=2.0))
 
 
 def test_auto_mode_picks_the_kernel_by_shape(device):
@@ -222,29 +249,29 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
         b = torch.empty(N, K, device=device)
         return module._plan_run_kernel(descriptor, a, b, None, kw.get("p"), None, None, kw.get("bandwidth"), None, None, 0, 0, False)
 
-    big = planned(4000, 4000, 128)
+    big = planned(8000, 8000, 128)
     assert big.l2_auto and big.params.flags & core == core and big.params.gram_trust > 0
     assert planned(500, 500, 128).params.flags & core == 0                       # 3.2e7 terms: direct
-    assert planned(4000, 4000, 32).params.flags & core == 0                      # K below min_k: direct
-    assert planned(4000, 4000, 128, kermac.kernel_descriptor_l1_norm).params.flags & core == 0
-    assert planned(4000, 4000, 128, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0).params.flags & core == core
-    a = torch.empty(4000, 128, device=device)
-    fused = _plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l2, a, a, torch.empty(4000, 8, device=device), None,
+    assert planned(16000, 16000, 32).params.flags & core == 0                    # K below min_k: direct
+    assert planned(8000, 8000, 128, kermac.kernel_descriptor_l1_norm).params.flags & core == 0
+    assert planned(8000, 8000, 128, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0).params.flags & core == core
+    a = torch.empty(8000, 128, device=device)
+    fused = _plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l2, a, a, torch.empty(8000, 8, device=device), None,
                                           None, None, None, 2.0, None, None, 0, 0)
     assert fused.params.kernel.flags & core == _backend.FLAG_L2_GRAM            # fp32 matrix instruction there
     # a small result over a long contraction: marked, then handed back to the direct kernel and cut over k
     g = torch.Generator().manual_seed(5)
-    x = torch.randn(300, 40000, generator=g).to(device)
-    y = torch.randn(280, 40000, generator=g).to(device)
-    assert planned(300, 280, 40000).params.flags & core == core
+    x = torch.randn(400, 40000, generator=g).to(device)
+    y = torch.randn(380, 40000, generator=g).to(device)
+    assert planned(400, 380, 40000).params.flags & core == core
     got = kermac.cdist(x, y, p=2.0)[0]
     with kermac.l2_mode("direct"):
         assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0])
     assert_close_to_truth(got, oracle.cdist(x.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, what="auto, long contraction")
     # a large problem in auto mode equals the explicit split-bf16 mode, near-duplicate tiles included
     g = torch.Generator().manual_seed(6)
-    points = torch.randn(2000, 256, generator=g)
-    points[1000:] = points[:1000] + 1e-4 * torch.randn(1000, 256, generator=g)       # every point has a near twin
+    points = torch.randn(4400, 256, generator=g)
+    points[2200:] = points[:2200] + 1e-4 * torch.randn(2200, 256, generator=g)       # every point has a near twin
     points = points.to(device)
     got = kermac.cdist(points, points.clone(), p=2.0)[0]
     with kermac.l2_mode("gram_bf16"):
