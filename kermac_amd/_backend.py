@@ -57,6 +57,7 @@ class BuildKernelParams(Structure):
         ("gram_trust", c_float),
         ("k_total", c_int32),
         ("gram_centre", _float_p), ("gram_centre_bs", c_int64),
+        ("gram_workspace", c_void_p), ("gram_workspace_bytes", c_int64),
     ]
 
 
@@ -98,6 +99,7 @@ SIGNATURES = {
     "kmc_build_kernel_cut_static": (ctypes.c_int, [POINTER(BuildKernelParams), c_int32, c_void_p]),
     "kmc_sample_mean": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_int64, c_int32, c_void_p, c_int64,
                                        c_void_p]),
+    "kmc_gram_workspace_bytes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int64)]),
     "kmc_build_kernel_load_modes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int32), POINTER(c_int32)]),
     "kmc_norm_kernel_gradient": (ctypes.c_int, [POINTER(NormGradientParams), c_void_p]),
     "kmc_kernel_times_coefficients": (ctypes.c_int, [POINTER(KernelCoefficientsParams), c_void_p]),
@@ -193,6 +195,13 @@ CENTRE_PAD = 64
 def sample_mean(x: int, majorness: int, rows: int, k: int, ld: int, bs: int, l: int, mean: int, mean_bs: int,
                 stream: int) -> None:
     check(library().kmc_sample_mean(c_void_p(x), majorness, rows, k, ld, bs, l, c_void_p(mean), mean_bs, c_void_p(stream)))
+
+
+def gram_workspace_bytes(params: BuildKernelParams) -> int:
+    """Bytes of gram_workspace that kmc_build_kernel would use for these parameters (0: none)."""
+    needed = c_int64(0)
+    check(library().kmc_gram_workspace_bytes(byref(params), byref(needed)))
+    return needed.value
 
 
 def build_kernel_jit(function: int, params: BuildKernelParams, stream: int) -> None:

@@ -53,7 +53,8 @@ HOST_SOURCES = [
 # Device translation units without per-variant defines.
 EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_inst.hip",
                         "kernels/gram_coefficients_inst.hip", "kernels/gram_bf16_kernel_inst.hip",
-                        "kernels/finish_partials.hip", "kernels/cut_static_scratch.hip", "kernels/sample_mean.hip"]
+                        "kernels/finish_partials.hip", "kernels/cut_static_scratch.hip", "kernels/sample_mean.hip",
+                        "kernels/gram_f16_wide_inst.hip"]
 
 
 def _hipcc() -> str:

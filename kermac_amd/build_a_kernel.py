@@ -540,6 +540,7 @@ def run_kernel(
     cut = _cut_over_contraction(params)
     if params.flags & matrix_core:
         plan.keepalive.append(_attach_gram_centre(params, stream, a.device))
+        plan.keepalive.append(_attach_gram_workspace(params, a.device))
     if cut is None:
         launch(params)
     else:
@@ -563,6 +564,21 @@ def _attach_gram_centre(params, stream, device):
                          centre.data_ptr(), width, stream)
     params.gram_centre, params.gram_centre_bs = centre.data_ptr(), (width if batches > 1 else 0)
     return centre
+
+
+def _attach_gram_workspace(params, device):
+    """Large squared-difference problems in the split-bf16 mode go through a workspace (include/
+    kermac_amd.h, gram_workspace: both operands split once into fp16 pieces, then 256 x 256 tiles);
+    the library says how much it wants for this call, 0 when it would not use one.
+    KERMAC_AMD_L2_WORKSPACE=0 keeps every call on the one-step kernel."""
+    if os.environ.get("KERMAC_AMD_L2_WORKSPACE", "1") in ("", "0"):
+        return None
+    needed = _backend.gram_workspace_bytes(params)
+    if needed == 0:
+        return None
+    workspace = torch.empty(needed, dtype=torch.uint8, device=device)
+    params.gram_workspace, params.gram_workspace_bytes = workspace.data_ptr(), needed
+    return workspace
 
 
 # A workgroup owns one 128 x 128 tile of the result and walks the whole contraction index, so

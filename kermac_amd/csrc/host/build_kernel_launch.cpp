@@ -142,6 +142,8 @@ kmc_host::build_launcher_fn find_launcher(int inner_operator, int inner_power)
 namespace kmc_host {
 hipError_t launch_gram_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
 hipError_t launch_gram_bf16_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
+int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
+hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
 hipError_t launch_finish_partials(const kmc::BuildKernelArgs &kernel, const float *partials, int64_t partial_ld,
                                   int64_t partial_bs, int64_t partial_slice, int slices, int vec, hipStream_t stream);
 }
@@ -169,6 +171,17 @@ int kmc_build_kernel_load_modes(const kmc_build_kernel_params *params, int32_t *
     if (status != KMC_OK) return status;
     if (load_a) *load_a = la;
     if (load_b) *load_b = lb;
+    return KMC_OK;
+}
+
+int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes)
+{
+    if (!bytes) return fail(KMC_ERR_INVALID_ARGUMENT, "bytes: null pointer");
+    kmc::BuildKernelArgs args;
+    int load_a = 0, load_b = 0;
+    int status = prepare(params, true, &args, &load_a, &load_b);
+    if (status != KMC_OK) return status;
+    *bytes = gram_f16_wide_bytes(params, args);
     return KMC_OK;
 }
 
@@ -201,10 +214,15 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
         if (params->inner_operator != KMC_OP_DIFF || params->inner_power != KMC_POW_SQUARE)
             return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L2_GRAM needs inner_operator DIFF and inner_power SQUARE");
         // Matrix-core pass over every tile, then the direct kernel over the tiles it marked.
-        hipError_t g = (params->flags & KMC_FLAG_L2_GRAM_BF16)
-                           ? launch_gram_bf16_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream))
-                           : launch_gram_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
-        if (g != hipSuccess) return fail_hip(g, "gram_l2_kernel launch");
+        bool wide = false;
+        hipError_t g = launch_gram_f16_wide(params, args, static_cast<hipStream_t>(stream), &wide);
+        if (g != hipSuccess) return fail_hip(g, "gram_f16_wide launches");
+        if (!wide) {
+            g = (params->flags & KMC_FLAG_L2_GRAM_BF16)
+                    ? launch_gram_bf16_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream))
+                    : launch_gram_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
+            if (g != hipSuccess) return fail_hip(g, "gram_l2_kernel launch");
+        }
         args.repair_only = 1;
     }
     hipError_t e = launch(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));

@@ -1,0 +1,161 @@
+// Host side of the two-piece fp16 matrix-core path for large squared-difference problems
+// (gram_f16_wide.hpp): when it applies, how the caller's workspace is divided, and the launches.
+// One instantiation per kernel: the layout of an operand in memory is a run-time property of the
+// two row kernels and does not reach the product kernel at all.
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+
+#include "../host/host_common.hpp"
+#include "launch.hpp"
+#include "gram_f16_wide.hpp"
+
+namespace kmc_host {
+
+namespace {
+
+constexpr int64_t REGION_ALIGN = 256;
+
+struct OperandRegions {
+    int rows_pad, batches;
+    int64_t pieces_bs;       // chunks per batch entry
+    int64_t stats_bs;        // floats per batch entry, for the squares and for the magnitudes
+    int64_t pieces, squares, magnitudes, unscale;   // byte offsets into the workspace
+};
+
+struct WideLayout {
+    int slices, slices_per_range, ranges;
+    int tiles_m, tiles_n, tiles_n_padded;
+    OperandRegions a, b;
+    int64_t bytes;
+};
+
+int min_wide_tiles()
+{
+    // Below this many 256 x 256 tiles over the batch the chip is not filled (a CU holds one
+    // workgroup) and the one-step kernel with its 128 x 128 tiles is the faster one.  Read on
+    // every call, so that a test can lower it for small shapes.
+    const char *text = std::getenv("KERMAC_AMD_WIDE_MIN_TILES");
+    const int parsed = text ? std::atoi(text) : 0;
+    return parsed > 0 ? parsed : 192;
+}
+
+int64_t place(int64_t &cursor, int64_t bytes)
+{
+    const int64_t at = cursor;
+    cursor = (cursor + bytes + REGION_ALIGN - 1) / REGION_ALIGN * REGION_ALIGN;
+    return at;
+}
+
+void place_operand(OperandRegions &r, int rows, bool broadcast, int l, const WideLayout &layout, int64_t &cursor)
+{
+    r.rows_pad = (rows + kmc::GW_TILE - 1) / kmc::GW_TILE * kmc::GW_TILE;
+    r.batches = broadcast ? 1 : l;
+    r.pieces_bs = static_cast<int64_t>(layout.slices + kmc::GW_EXTRA_SLICES) * kmc::GW_SEGMENTS * r.rows_pad;
+    r.stats_bs = static_cast<int64_t>(layout.ranges) * r.rows_pad;
+    r.pieces = place(cursor, r.batches * r.pieces_bs * 16);
+    r.squares = place(cursor, r.batches * r.stats_bs * 4);
+    r.magnitudes = place(cursor, r.batches * r.stats_bs * 4);
+    r.unscale = place(cursor, static_cast<int64_t>(r.batches) * r.rows_pad * 4);
+}
+
+bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, WideLayout *layout)
+{
+    if (!(p->flags & KMC_FLAG_L2_GRAM_BF16) || args.symmetric) return false;
+    if (p->inner_operator != KMC_OP_DIFF || p->inner_power != KMC_POW_SQUARE) return false;
+    if (args.m < 1 || args.n < 1 || args.l < 1 || args.k < 32) return false;
+    layout->tiles_m = (args.m + kmc::GW_TILE - 1) / kmc::GW_TILE;
+    layout->tiles_n = (args.n + kmc::GW_TILE - 1) / kmc::GW_TILE;
+    if (static_cast<int64_t>(layout->tiles_m) * layout->tiles_n * args.l < min_wide_tiles()) return false;
+    int padded = (layout->tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
+    if ((padded - layout->tiles_n) * 8 > layout->tiles_n) padded = layout->tiles_n;
+    if (static_cast<int64_t>(layout->tiles_m) * padded > 0x7fffffff) return false;
+    layout->tiles_n_padded = padded;
+    layout->slices = (args.k + kmc::BK_TILE_K - 1) / kmc::BK_TILE_K;
+    // at most 8 ranges of K per row: enough workgroups for the row kernels, few partial sums
+    layout->slices_per_range = layout->slices / 8 > 8 ? (layout->slices + 7) / 8 : 8;
+    layout->ranges = (layout->slices + layout->slices_per_range - 1) / layout->slices_per_range;
+    int64_t cursor = 0;
+    // an operand that is the same for every batch entry is split once, unless the centre differs
+    const bool one_centre = !args.centre || args.centre_bs == 0;
+    place_operand(layout->a, args.m, args.a_bs == 0 && one_centre, args.l, *layout, cursor);
+    place_operand(layout->b, args.n, args.b_bs == 0 && one_centre, args.l, *layout, cursor);
+    layout->bytes = cursor;
+    return true;
+}
+
+kmc::GramRowsArgs rows_args(const float *x, int64_t ld, int64_t bs, int rows, int majorness, bool scalar_only,
+                            const kmc::BuildKernelArgs &args, const WideLayout &layout, const OperandRegions &r, char *workspace)
+{
+    kmc::GramRowsArgs rows_of = {};
+    rows_of.x = x; rows_of.ld = ld; rows_of.bs = bs;
+    rows_of.rows = rows; rows_of.k = args.k;
+    rows_of.row_major = majorness == KMC_ROW_MAJOR;
+    rows_of.vec = rows_of.row_major && !scalar_only && aligned16(x) && ld % 4 == 0 && bs % 4 == 0;
+    rows_of.centre = args.centre; rows_of.centre_bs = args.centre_bs;
+    rows_of.pieces = reinterpret_cast<kmc::gram_chunk *>(workspace + r.pieces); rows_of.pieces_bs = r.pieces_bs;
+    rows_of.squares = reinterpret_cast<float *>(workspace + r.squares);
+    rows_of.magnitudes = reinterpret_cast<float *>(workspace + r.magnitudes);
+    rows_of.unscale = reinterpret_cast<float *>(workspace + r.unscale);
+    rows_of.stats_bs = r.stats_bs; rows_of.unscale_bs = r.rows_pad;
+    rows_of.rows_pad = r.rows_pad; rows_of.slices = layout.slices;
+    rows_of.slices_per_range = layout.slices_per_range; rows_of.ranges = layout.ranges;
+    return rows_of;
+}
+
+hipError_t launch_rows(const kmc::GramRowsArgs &rows_of, int batches, hipStream_t stream)
+{
+    const dim3 grid(rows_of.rows_pad / kmc::GW_ROW_THREADS, rows_of.ranges, batches);
+    hipError_t status = launch(kmc::gram_row_stats, grid, dim3(kmc::GW_ROW_THREADS), stream, rows_of);
+    if (status != hipSuccess) return status;
+    return launch(kmc::gram_f16_split, grid, dim3(kmc::GW_ROW_THREADS), stream, rows_of);
+}
+
+}  // namespace
+
+// Bytes of workspace the path needs for this problem; 0 when it does not apply.
+int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args)
+{
+    WideLayout layout;
+    return wide_layout(p, args, &layout) ? layout.bytes : 0;
+}
+
+// Row statistics and split of both operands, then the product kernel.  `*taken` says whether the
+// path applied (and the launches were made); if not, nothing was launched.
+hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken)
+{
+    *taken = false;
+    WideLayout layout;
+    if (!p->gram_workspace || !wide_layout(p, args, &layout) || p->gram_workspace_bytes < layout.bytes ||
+        (reinterpret_cast<uintptr_t>(p->gram_workspace) & (REGION_ALIGN - 1)) != 0)
+        return hipSuccess;
+    char *workspace = static_cast<char *>(p->gram_workspace);
+    const bool scalar_only = (p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) != 0;
+    const kmc::GramRowsArgs rows_a = rows_args(args.a, args.a_ld, args.a_bs, args.m, p->a_majorness, scalar_only, args, layout, layout.a, workspace);
+    const kmc::GramRowsArgs rows_b = rows_args(args.b, args.b_ld, args.b_bs, args.n, p->b_majorness, scalar_only, args, layout, layout.b, workspace);
+    hipError_t status = launch_rows(rows_a, layout.a.batches, stream);
+    if (status != hipSuccess) return status;
+    status = launch_rows(rows_b, layout.b.batches, stream);
+    if (status != hipSuccess) return status;
+
+    kmc::GramWideArgs wide = {};
+    wide.kernel = args;
+    wide.pieces_a = rows_a.pieces; wide.pieces_b = rows_b.pieces;
+    wide.pieces_a_bs = layout.a.batches > 1 ? layout.a.pieces_bs : 0;
+    wide.pieces_b_bs = layout.b.batches > 1 ? layout.b.pieces_bs : 0;
+    wide.squares_a = rows_a.squares; wide.squares_b = rows_b.squares;
+    wide.stats_a_bs = layout.a.batches > 1 ? layout.a.stats_bs : 0;
+    wide.stats_b_bs = layout.b.batches > 1 ? layout.b.stats_bs : 0;
+    wide.unscale_a = rows_a.unscale; wide.unscale_b = rows_b.unscale;
+    wide.unscale_a_bs = layout.a.batches > 1 ? layout.a.rows_pad : 0;
+    wide.unscale_b_bs = layout.b.batches > 1 ? layout.b.rows_pad : 0;
+    wide.rows_pad_a = layout.a.rows_pad; wide.rows_pad_b = layout.b.rows_pad;
+    wide.slices = layout.slices; wide.ranges = layout.ranges;
+    wide.wide_tiles_m = layout.tiles_m; wide.wide_tiles_n = layout.tiles_n; wide.wide_tiles_n_padded = layout.tiles_n_padded;
+    const dim3 grid(static_cast<unsigned>(layout.tiles_m) * layout.tiles_n_padded, args.l, 1);
+    status = launch(kmc::gram_f16_wide, grid, dim3(kmc::GW_THREADS), stream, wide);
+    if (status == hipSuccess) *taken = true;
+    return status;
+}
+
+}  // namespace kmc_host

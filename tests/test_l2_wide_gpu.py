@@ -1,0 +1,226 @@
+"""GPU tests of the route that large squared-difference problems take in the split-bf16 mode when
+the caller brings a workspace (include/kermac_amd.h, gram_workspace): row statistics, both
+operands split once into two fp16 pieces per value with a power-of-two scale per row, then
+256 x 256 tiles on the fp16 matrix instruction.  Same stated tolerance as every p = 2 path: 1e-5
+relative to the float64 truth -- trusted 128 x 128 parts by the error bound of the expansion,
+distrusted parts because the direct kernel recomputes them.
+
+KERMAC_AMD_WIDE_MIN_TILES=1 sends the small shapes of these tests down the route, which by itself
+only takes problems of at least 192 tiles.
+"""
+import pytest
+import torch
+
+import kermac_amd as kermac
+from kermac_amd import _backend, build_a_kernel as module
+from oracle import oracle
+from tests.helpers import assert_close_to_truth, make_operand
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def wide(monkeypatch):
+    monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
+    kermac.set_l2_mode("gram_bf16", min_k=0)
+    yield
+    kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
+
+
+def one_step(fn, monkeypatch):
+    """The same call on the one-step kernel."""
+    monkeypatch.setenv("KERMAC_AMD_L2_WORKSPACE", "0")
+    try:
+        return fn()
+    finally:
+        monkeypatch.setenv("KERMAC_AMD_L2_WORKSPACE", "1")
+
+
+def workspace_bytes(a, b, descriptor=kermac.kernel_descriptor_l2_norm, **kw):
+    plan = module._plan_run_kernel(descriptor, a, b, None, None, None, None, kw.get("bandwidth"), None, None, 0, 0, False)
+    return _backend.gram_workspace_bytes(plan.params)
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 260, 96), (515, 770, 70), (1000, 900, 200), (257, 255, 33), (256, 512, 1024),
+                                   (1, 700, 64), (640, 3, 48)])
+@pytest.mark.parametrize("layout", ["cc", "rr", "cr", "rc"])
+def test_random_data_matches_truth(device, wide, M, N, K, layout):
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
+    a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False)
+    b = make_operand(1, N, K, layout[1] == "c", device, g, batch=False)
+    assert workspace_bytes(a, b) > 0
+    for c_col in (False, True):
+        out = torch.empty(N, M, device=device).t() if c_col else torch.empty(M, N, device=device)
+        got = kermac.cdist(a, b, out=out, p=2.0)
+        assert_close_to_truth(got, oracle.cdist(a.cpu(), b.cpu(), p=2.0)[0], rtol=1e-5,
+                              what=f"wide {M}x{N}x{K} {layout} out col-major={c_col}")
+
+
+def test_when_the_route_applies(device, monkeypatch):
+    """kmc_gram_workspace_bytes: 0 without the split-bf16 flag, for a panel against itself, for
+    short contractions and for problems of fewer than 192 tiles of 256 x 256 over the batch."""
+    a = torch.empty(5000, 128, device=device)
+    b = torch.empty(4000, 128, device=device)
+    with kermac.l2_mode("gram_bf16"):
+        assert workspace_bytes(a, b) > 0                                         # 20 x 16 tiles
+        assert workspace_bytes(a, b, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0) > 0
+        assert workspace_bytes(a, b, kermac.kernel_descriptor_l1_norm) == 0
+        assert workspace_bytes(a, a) == 0                                        # symmetric: half the tiles, one-step kernel
+        assert workspace_bytes(a[:3000], b[:3000]) == 0                          # 144 tiles
+        assert workspace_bytes(a[:, :16], b[:, :16]) == 0                        # k < 32
+        assert workspace_bytes(a[:3000].expand(2, 3000, 128), b[:3000].expand(2, 3000, 128)) > 0    # 288 over the batch
+        needed = workspace_bytes(a, b)
+        operands = (5000 + 4000) * 128 * 4
+        assert operands <= needed <= 2 * operands
+    with kermac.l2_mode("gram"):
+        assert workspace_bytes(a, b) == 0
+    with kermac.l2_mode("direct"):
+        assert workspace_bytes(a, b) == 0
+
+
+def test_without_a_workspace_the_one_step_kernel_runs(device, wide, monkeypatch):
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(700, 96, generator=g).to(device)
+    b = torch.randn(600, 96, generator=g).to(device)
+    reference = one_step(lambda: kermac.cdist(a, b, p=2.0), monkeypatch)
+    plan = module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, a, b, None, None, None, None, None, None, None, 0, 0, False)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    keep = module._attach_gram_centre(plan.params, stream, device)
+    needed = _backend.gram_workspace_bytes(plan.params)
+    assert needed > 0
+    workspace = torch.empty(needed, dtype=torch.uint8, device=device)
+    for pointer, size in ((0, 0), (workspace.data_ptr(), needed - 1), (workspace.data_ptr() + 16, needed)):
+        plan.out.fill_(-1.0)
+        plan.params.gram_workspace, plan.params.gram_workspace_bytes = pointer, size
+        _backend.build_kernel(plan.params, stream)
+        assert torch.equal(plan.out, reference), "null, short or misaligned workspace: expected the one-step kernel's bits"
+    plan.params.gram_workspace, plan.params.gram_workspace_bytes = workspace.data_ptr(), needed
+    _backend.build_kernel(plan.params, stream)
+    assert_close_to_truth(plan.out, oracle.cdist(a.cpu(), b.cpu(), p=2.0), rtol=1e-5, what="with the workspace")
+    del keep
+
+
+def test_rows_of_very_different_magnitude(device, wide):
+    """The scale is per row: a row of values around 1e-6 beside rows around 1e+5, and eight orders
+    of magnitude inside every row, keep the tolerance (one scale per operand would put the small
+    rows into fp16's subnormals)."""
+    g = torch.Generator().manual_seed(9)
+    M, N, K = 520, 390, 150
+    within = torch.pow(2.0, -(torch.arange(K) % 27).float())
+    a = torch.randn(M, K, generator=g) * within * torch.pow(2.0, (torch.arange(M) % 37 - 18).float())[:, None]
+    b = torch.randn(N, K, generator=g) * within * torch.pow(2.0, (torch.arange(N) % 37 - 18).float())[:, None]
+    a, b = a.to(device), b.to(device)
+    got = kermac.cdist(a, b, p=2.0)
+    assert_close_to_truth(got, oracle.cdist(a.cpu(), b.cpu(), p=2.0), rtol=1e-5, what="rows of different magnitude")
+
+
+def test_near_duplicates_are_repaired_part_by_part(device, wide, monkeypatch):
+    """Every point of b has a twin in a: the parts of 128 x 128 that hold a twin pair are distrusted
+    and come from the direct kernel bit for bit; no marker is left behind."""
+    g = torch.Generator().manual_seed(4)
+    a = torch.randn(600, 128, generator=g)
+    b = a[:500] + 1e-5 * torch.randn(500, 128, generator=g)
+    a, b = a.to(device), b.to(device)
+    got = kermac.cdist(a, b, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        direct = kermac.cdist(a, b, p=2.0)[0]
+    assert not torch.isnan(got).any()
+    assert_close_to_truth(got, oracle.cdist(a.cpu(), b.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30, what="near duplicates")
+    for part in range(0, 500, 128):                      # the parts on the diagonal hold the twins
+        stop = min(part + 128, 500)
+        assert torch.equal(got[part:stop, part:stop], direct[part:stop, part:stop])
+    assert not torch.equal(got, direct), "every part was repaired: the matrix-core values were not kept"
+
+
+def test_data_that_is_not_a_number(device, wide):
+    """A NaN and an infinity in a: their rows come out as the direct kernel gives them."""
+    g = torch.Generator().manual_seed(6)
+    a = torch.randn(300, 64, generator=g)
+    b = torch.randn(280, 64, generator=g)
+    a[17, 3] = float("nan")
+    a[200, 40] = float("inf")
+    a, b = a.to(device), b.to(device)
+    got = kermac.cdist(a, b, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        direct = kermac.cdist(a, b, p=2.0)[0]
+    assert torch.equal(torch.isnan(got), torch.isnan(direct)) and torch.equal(torch.isinf(got), torch.isinf(direct))
+    finite = torch.isfinite(direct)
+    rows = torch.ones(300, dtype=torch.bool)
+    rows[17] = rows[200] = False
+    assert torch.equal(finite.cpu(), rows[:, None].expand(300, 280))
+    truth = oracle.cdist(a.cpu(), b.cpu(), p=2.0)[0]
+    assert_close_to_truth(got[rows.to(device)], truth[rows], rtol=1e-5, what="rows without NaN or infinity")
+
+
+@pytest.mark.parametrize("layout", ["cc", "rr"])
+def test_offset_data_and_batches(device, wide, monkeypatch, layout):
+    """Points in [100, 101]^K: the centre is subtracted by the split, per batch entry; a first
+    operand that is the same for every batch entry is split once, or once per entry when the
+    centres differ."""
+    g = torch.Generator().manual_seed(17)
+    M, N, K = 300, 260, 96
+    a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False, dist="rand") + 100.0
+    b = make_operand(1, N, K, layout[1] == "c", device, g, batch=False, dist="rand") + 100.0
+    truth = oracle.cdist(a.cpu(), b.cpu(), p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        direct = kermac.cdist(a, b, p=2.0)[0]
+    got = kermac.cdist(a, b, p=2.0)[0]
+    assert_close_to_truth(got, truth, rtol=1e-5, what=f"offset data {layout}")
+    assert not torch.equal(got, direct), "every part was repaired: the centre did not take effect"
+    shifts = torch.tensor([0.0, 50.0, -30.0], device=device)[:, None, None]
+    ab = (a - 100.0)[None] + shifts
+    bb = (b - 100.0)[None] + shifts
+    batched = kermac.cdist(ab, bb, p=2.0)
+    for l in range(3):
+        assert_close_to_truth(batched[l], oracle.cdist(ab[l].cpu(), bb[l].cpu(), p=2.0)[0], rtol=1e-5, what=f"batch {l}")
+    broadcast = kermac.cdist(a, bb + 100.0 - shifts, p=2.0)                  # a for every entry, one centre
+    assert_close_to_truth(broadcast[2], truth, rtol=1e-5, what="first operand for every batch entry")
+    broadcast = kermac.cdist(ab, b - 100.0, p=2.0)                           # b for every entry, a centre per entry
+    for l in range(3):
+        assert_close_to_truth(broadcast[l], oracle.cdist(ab[l].cpu(), (b - 100.0).cpu(), p=2.0)[0], rtol=1e-5,
+                              what=f"second operand for every batch entry, entry {l}")
+
+
+def test_kernel_functions_and_regularisation(device, wide):
+    g = torch.Generator().manual_seed(12)
+    M, N, K = 400, 330, 80
+    a = torch.randn(M, K, generator=g).to(device)
+    b = torch.randn(N, K, generator=g).to(device)
+    gaussian = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP,
+                                       kermac.KernelType.GAUSSIAN)
+    for descriptor, outer, kernel, bandwidth, rtol in ((kermac.kernel_descriptor_laplace_l2, "SQRT", "LAPLACE", float(K), 1e-5),
+                                                       (gaussian, "NOOP", "GAUSSIAN", 10.0, 2e-5)):     # exp(-d^2 / 200) doubles the error of d
+        assert workspace_bytes(a, b, descriptor, bandwidth=bandwidth) > 0
+        got = kermac.run_kernel(descriptor, a, b, bandwidth=bandwidth, regularization=0.25, regularization_offset_x=2,
+                                regularization_offset_y=70)
+        want = oracle.run_kernel("DIFF", "SQUARE", outer, kernel, a.cpu(), b.cpu(), bandwidth=bandwidth, regularization=0.25,
+                                 regularization_offset_x=2, regularization_offset_y=70)
+        assert_close_to_truth(got, want, rtol=rtol, what=kernel)
+        assert (got == 1.25).sum() > 0
+    squares = kermac.cdist(a, b, p=2.0, skip_epilogue=True)
+    assert_close_to_truth(squares, oracle.cdist(a.cpu(), b.cpu(), p=2.0, skip_epilogue=True), rtol=1e-5, what="squared distances")
+
+
+def test_unaligned_result_and_operands(device, wide):
+    g = torch.Generator().manual_seed(3)
+    M, N, K = 310, 270, 37
+    flat = torch.randn(K * (M + 3) + 1, generator=g).to(device)
+    a = flat[1:].view(K, M + 3)[:, :M].t()
+    b = torch.randn(N, K + 5, generator=g).to(device)[:, 2:2 + K]
+    out = torch.empty(N, M + 1, device=device)[:, :M].t()
+    got = kermac.cdist(a, b, out=out, p=2.0)
+    assert_close_to_truth(got, oracle.cdist(a.cpu(), b.cpu(), p=2.0)[0], rtol=1e-5, what="unaligned")
+
+
+def test_large_problem_takes_the_route_by_itself(device):
+    """The default mode at a size above the threshold: the result equals the explicit mode with the
+    workspace and differs from the one-step kernel's, and keeps the tolerance on slabs."""
+    assert kermac.get_l2_mode() == "auto"
+    g = torch.Generator().manual_seed(8)
+    a = torch.randn(128, 4200, generator=g).to(device).t()
+    b = torch.randn(128, 3900, generator=g).to(device).t()
+    assert workspace_bytes(a, b) > 0
+    got = kermac.cdist(a, b, p=2.0)[0]
+    truth = torch.cdist(a[:300].double(), b.double(), p=2.0)
+    assert_close_to_truth(got[:300], truth, rtol=1e-5, what="auto, wide")
+    assert not torch.isnan(got[::128, ::128]).any()
