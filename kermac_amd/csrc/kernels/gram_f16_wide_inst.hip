@@ -30,14 +30,18 @@ struct WideLayout {
     int64_t bytes;
 };
 
-int min_wide_tiles()
+// Whether the route pays for its extra launches and its coarser tiles (a CU holds one workgroup of
+// 256 x 256, so a few hundred tiles do not fill the chip as evenly as four times as many of
+// 128 x 128).  From a sweep against the one-step kernel, wide / one-step time: K = 1024 0.92 at 144
+// tiles, 0.76 at 256, 0.63 from 1024 on; K = 256 1.01 at 576, 0.87 at 1024, 0.80 at 4096; K = 64 1.0
+// at 1024, 0.9 from 2304 on; K = 32 never below 1.  KERMAC_AMD_WIDE_MIN_TILES = t replaces the rule
+// by "at least t tiles" (read on every call, so that a test can send small shapes down the route).
+bool wide_pays(int64_t tiles, int k)
 {
-    // Below this many 256 x 256 tiles over the batch the chip is not filled (a CU holds one
-    // workgroup) and the one-step kernel with its 128 x 128 tiles is the faster one.  Read on
-    // every call, so that a test can lower it for small shapes.
     const char *text = std::getenv("KERMAC_AMD_WIDE_MIN_TILES");
-    const int parsed = text ? std::atoi(text) : 0;
-    return parsed > 0 ? parsed : 192;
+    const int forced = text ? std::atoi(text) : 0;
+    if (forced > 0) return tiles >= forced && k >= 1;
+    return k >= 64 && tiles >= 128 && tiles * k >= 147456;
 }
 
 int64_t place(int64_t &cursor, int64_t bytes)
@@ -63,10 +67,10 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
 {
     if (!(p->flags & KMC_FLAG_L2_GRAM_BF16) || args.symmetric) return false;
     if (p->inner_operator != KMC_OP_DIFF || p->inner_power != KMC_POW_SQUARE) return false;
-    if (args.m < 1 || args.n < 1 || args.l < 1 || args.k < 32) return false;
+    if (args.m < 1 || args.n < 1 || args.l < 1) return false;
     layout->tiles_m = (args.m + kmc::GW_TILE - 1) / kmc::GW_TILE;
     layout->tiles_n = (args.n + kmc::GW_TILE - 1) / kmc::GW_TILE;
-    if (static_cast<int64_t>(layout->tiles_m) * layout->tiles_n * args.l < min_wide_tiles()) return false;
+    if (!wide_pays(static_cast<int64_t>(layout->tiles_m) * layout->tiles_n * args.l, args.k)) return false;
     int padded = (layout->tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
     if ((padded - layout->tiles_n) * 8 > layout->tiles_n) padded = layout->tiles_n;
     if (static_cast<int64_t>(layout->tiles_m) * padded > 0x7fffffff) return false;

@@ -42,7 +42,7 @@ def workspace_bytes(a, b, descriptor=kermac.kernel_descriptor_l2_norm, **kw):
 
 
 @pytest.mark.parametrize("M,N,K", [(300, 260, 96), (515, 770, 70), (1000, 900, 200), (257, 255, 33), (256, 512, 1024),
-                                   (1, 700, 64), (640, 3, 48)])
+                                   (1, 700, 64), (640, 3, 48), (300, 200, 5), (128, 128, 16), (513, 257, 1)])
 @pytest.mark.parametrize("layout", ["cc", "rr", "cr", "rc"])
 def test_random_data_matches_truth(device, wide, M, N, K, layout):
     g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
@@ -58,19 +58,20 @@ def test_random_data_matches_truth(device, wide, M, N, K, layout):
 
 def test_when_the_route_applies(device, monkeypatch):
     """kmc_gram_workspace_bytes: 0 without the split-bf16 flag, for a panel against itself, for
-    short contractions and for problems of fewer than 192 tiles of 256 x 256 over the batch."""
-    a = torch.empty(5000, 128, device=device)
-    b = torch.empty(4000, 128, device=device)
+    short contractions and for problems of too few tiles of 256 x 256 over the batch for their k."""
+    a = torch.empty(5000, 512, device=device)
+    b = torch.empty(4000, 512, device=device)
     with kermac.l2_mode("gram_bf16"):
         assert workspace_bytes(a, b) > 0                                         # 20 x 16 tiles
         assert workspace_bytes(a, b, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0) > 0
         assert workspace_bytes(a, b, kermac.kernel_descriptor_l1_norm) == 0
         assert workspace_bytes(a, a) == 0                                        # symmetric: half the tiles, one-step kernel
-        assert workspace_bytes(a[:3000], b[:3000]) == 0                          # 144 tiles
-        assert workspace_bytes(a[:, :16], b[:, :16]) == 0                        # k < 32
-        assert workspace_bytes(a[:3000].expand(2, 3000, 128), b[:3000].expand(2, 3000, 128)) > 0    # 288 over the batch
+        assert workspace_bytes(a[:2500], b[:2500]) == 0                          # 100 tiles
+        assert workspace_bytes(a[:, :32], b[:, :32]) == 0                        # k < 64
+        assert workspace_bytes(a[:, :128], b[:, :128]) == 0                      # 320 tiles at k = 128
+        assert workspace_bytes(a[:2500].expand(3, 2500, 512), b[:2500].expand(3, 2500, 512)) > 0    # 300 over the batch
         needed = workspace_bytes(a, b)
-        operands = (5000 + 4000) * 128 * 4
+        operands = (5000 + 4000) * 512 * 4
         assert operands <= needed <= 2 * operands
     with kermac.l2_mode("gram"):
         assert workspace_bytes(a, b) == 0
@@ -217,8 +218,8 @@ def test_large_problem_takes_the_route_by_itself(device):
     workspace and differs from the one-step kernel's, and keeps the tolerance on slabs."""
     assert kermac.get_l2_mode() == "auto"
     g = torch.Generator().manual_seed(8)
-    a = torch.randn(128, 4200, generator=g).to(device).t()
-    b = torch.randn(128, 3900, generator=g).to(device).t()
+    a = torch.randn(512, 4700, generator=g).to(device).t()
+    b = torch.randn(512, 4200, generator=g).to(device).t()
     assert workspace_bytes(a, b) > 0
     got = kermac.cdist(a, b, p=2.0)[0]
     truth = torch.cdist(a[:300].double(), b.double(), p=2.0)
