@@ -200,10 +200,21 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsA
 
 // Workgroup -> tile, as tile_of_workgroup of build_kernel.hpp with bands of GW_BAND_N tiles: a
 // CU holds one workgroup, so the 32 of an XCD cover 4 n tiles x 8 m tiles of a band at a time.
+// SYMMETRIC (a panel against itself): the ids count through the tiles on and below the diagonal,
+// row r of the triangle starting at id r (r + 1) / 2.
+template <bool SYMMETRIC>
 __device__ __forceinline__ bool wide_tile_of_workgroup(const GramWideArgs &args, int &tile_m, int &tile_n)
 {
     const int rotated = blockIdx.x + blockIdx.y % gridDim.x;
     const int linear = rotated >= (int)gridDim.x ? rotated - (int)gridDim.x : rotated;
+    if (SYMMETRIC) {
+        int row = (int)((sqrtf(8.0f * (float)linear + 1.0f) - 1.0f) * 0.5f);
+        while (row * (row + 1) / 2 > linear) row--;
+        while ((row + 1) * (row + 2) / 2 <= linear) row++;
+        tile_m = row;
+        tile_n = linear - row * (row + 1) / 2;
+        return true;
+    }
     const int band_tiles = GW_BAND_N * args.wide_tiles_m;
     const int band = linear / band_tiles;
     const int band_height = min(GW_BAND_N, args.wide_tiles_n_padded - band * GW_BAND_N);
@@ -227,6 +238,14 @@ __device__ __forceinline__ bool wide_tile_of_workgroup(const GramWideArgs &args,
 // leaves nothing in flight.  The compiler therefore does not count these copies either; the walk
 // waits for them itself, and no other vector load is issued between the first copy and the wait
 // for all of them behind the walk.
+//
+// SYMMETRIC: b is a, the result is symmetric, and it is made so bit for bit: one workgroup per
+// tile on or below the diagonal; what lies below the diagonal is stored a second time, mirrored;
+// of a 128 x 128 part on the diagonal the lower triangle is stored and mirrored (the two halves of
+// such a part are computed with the pieces in exchanged roles and differ in the last bit); the
+// part above the diagonal inside a diagonal tile is not stored from its own values at all.  A
+// distrusted part is left to the repair launch, which mirrors what it recomputes.
+template <bool SYMMETRIC>
 __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs args)
 {
     __shared__ gram_chunk lds0[GW_BUFFER_CHUNKS];
@@ -240,7 +259,7 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
     const int tid = threadIdx.x;
     const int batch = blockIdx.y;
     int tile_m, tile_n;
-    if (!wide_tile_of_workgroup(args, tile_m, tile_n)) return;
+    if (!wide_tile_of_workgroup<SYMMETRIC>(args, tile_m, tile_n)) return;
     const int m0 = tile_m * GW_TILE;
     const int n0 = tile_n * GW_TILE;
     const int m_valid = args.kernel.m - m0;
@@ -485,9 +504,15 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
                     if (kernel.reg_off_x + m0 + m_local == kernel.reg_off_y + n0 + n_local[nt]) acc[mt][nt][v] = diagonal_value;
             }
     }
-    const int part = (wave & 1) + 2 * (wave >> 2);
-    if (distrusted != 0 && lane == 0) lds_distrust[part] = 1;
+    const int part_m = wave & 1, part_n = wave >> 2;
+    const int part = part_m + 2 * part_n;
+    // where this wave's part lies: below the diagonal of the result (stored and mirrored), on it
+    // (lower triangle stored and mirrored), above it inside a diagonal tile (not stored)
+    const bool on_diagonal = SYMMETRIC && tile_m == tile_n && part_m == part_n;
+    const bool above = SYMMETRIC && tile_m == tile_n && part_m < part_n;
+    if (distrusted != 0 && lane == 0 && !above) lds_distrust[part] = 1;
     __syncthreads();
+    if (above) return;
     const bool repair = lds_distrust[part] != 0;
     // the first element of a part is held by lane 0 of the wave that starts the part
     if (repair && lane == 0 && (wave_n & 127) == 0) acc[0][0][0] = __uint_as_float(BK_REPAIR_MARKER);
@@ -503,14 +528,32 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
             for (int g = 0; g < 4; g++) {
                 const int m_local = wave_m + mt * 32 + 8 * g + 4 * h;
                 const float v4[4] = {acc[mt][nt][4 * g], acc[mt][nt][4 * g + 1], acc[mt][nt][4 * g + 2], acc[mt][nt][4 * g + 3]};
-                if (kernel.c_vec && (full || m_local + 3 < m_valid)) {
+                const bool whole = !on_diagonal || m_local >= n_local[nt];
+                if (kernel.c_vec && whole && (full || m_local + 3 < m_valid)) {
                     *reinterpret_cast<float4 *>(row + m_local) = make_float4(v4[0], v4[1], v4[2], v4[3]);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        if (m_local + e < m_valid) row[m_local + e] = v4[e];
+                        if (m_local + e < m_valid && (!on_diagonal || m_local + e >= n_local[nt])) row[m_local + e] = v4[e];
                 }
             }
+    }
+
+    // The same values at C(n, m), where the 32 consecutive n of a half wave are the contiguous ones.
+    if (SYMMETRIC && !repair) {
+        float *mirror = kernel.c + batch * kernel.c_bs + (i64)m0 * kernel.c_ld + n0;
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+            if (!full && n_local[nt] >= n_valid) continue;
+#pragma unroll
+            for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int m_local = wave_m + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+                    if ((full || m_local < m_valid) && (!on_diagonal || m_local > n_local[nt]))
+                        mirror[(i64)m_local * kernel.c_ld + n_local[nt]] = acc[mt][nt][v];
+                }
+        }
     }
 }
 

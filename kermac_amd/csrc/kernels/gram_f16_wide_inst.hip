@@ -65,12 +65,15 @@ void place_operand(OperandRegions &r, int rows, bool broadcast, int l, const Wid
 
 bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, WideLayout *layout)
 {
-    if (!(p->flags & KMC_FLAG_L2_GRAM_BF16) || args.symmetric) return false;
+    if (!(p->flags & KMC_FLAG_L2_GRAM_BF16)) return false;
     if (p->inner_operator != KMC_OP_DIFF || p->inner_power != KMC_POW_SQUARE) return false;
     if (args.m < 1 || args.n < 1 || args.l < 1) return false;
     layout->tiles_m = (args.m + kmc::GW_TILE - 1) / kmc::GW_TILE;
     layout->tiles_n = (args.n + kmc::GW_TILE - 1) / kmc::GW_TILE;
-    if (!wide_pays(static_cast<int64_t>(layout->tiles_m) * layout->tiles_n * args.l, args.k)) return false;
+    // a panel against itself: the tiles on and below the diagonal
+    const int64_t tiles = args.symmetric ? static_cast<int64_t>(layout->tiles_m) * (layout->tiles_m + 1) / 2
+                                         : static_cast<int64_t>(layout->tiles_m) * layout->tiles_n;
+    if (!wide_pays(tiles * args.l, args.k)) return false;
     int padded = (layout->tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
     if ((padded - layout->tiles_n) * 8 > layout->tiles_n) padded = layout->tiles_n;
     if (static_cast<int64_t>(layout->tiles_m) * padded > 0x7fffffff) return false;
@@ -83,7 +86,8 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
     // an operand that is the same for every batch entry is split once, unless the centre differs
     const bool one_centre = !args.centre || args.centre_bs == 0;
     place_operand(layout->a, args.m, args.a_bs == 0 && one_centre, args.l, *layout, cursor);
-    place_operand(layout->b, args.n, args.b_bs == 0 && one_centre, args.l, *layout, cursor);
+    if (args.symmetric) layout->b = layout->a;      // one panel, split once
+    else place_operand(layout->b, args.n, args.b_bs == 0 && one_centre, args.l, *layout, cursor);
     layout->bytes = cursor;
     return true;
 }
@@ -139,8 +143,10 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     const kmc::GramRowsArgs rows_b = rows_args(args.b, args.b_ld, args.b_bs, args.n, p->b_majorness, scalar_only, args, layout, layout.b, workspace);
     hipError_t status = launch_rows(rows_a, layout.a.batches, stream);
     if (status != hipSuccess) return status;
-    status = launch_rows(rows_b, layout.b.batches, stream);
-    if (status != hipSuccess) return status;
+    if (!args.symmetric) {
+        status = launch_rows(rows_b, layout.b.batches, stream);
+        if (status != hipSuccess) return status;
+    }
 
     kmc::GramWideArgs wide = {};
     wide.kernel = args;
@@ -156,8 +162,13 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     wide.rows_pad_a = layout.a.rows_pad; wide.rows_pad_b = layout.b.rows_pad;
     wide.slices = layout.slices; wide.ranges = layout.ranges;
     wide.wide_tiles_m = layout.tiles_m; wide.wide_tiles_n = layout.tiles_n; wide.wide_tiles_n_padded = layout.tiles_n_padded;
-    const dim3 grid(static_cast<unsigned>(layout.tiles_m) * layout.tiles_n_padded, args.l, 1);
-    status = launch(kmc::gram_f16_wide, grid, dim3(kmc::GW_THREADS), stream, wide);
+    if (args.symmetric) {
+        const dim3 grid(static_cast<unsigned>(layout.tiles_m) * (layout.tiles_m + 1) / 2, args.l, 1);
+        status = launch(kmc::gram_f16_wide<true>, grid, dim3(kmc::GW_THREADS), stream, wide);
+    } else {
+        const dim3 grid(static_cast<unsigned>(layout.tiles_m) * layout.tiles_n_padded, args.l, 1);
+        status = launch(kmc::gram_f16_wide<false>, grid, dim3(kmc::GW_THREADS), stream, wide);
+    }
     if (status == hipSuccess) *taken = true;
     return status;
 }

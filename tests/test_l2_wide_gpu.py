@@ -57,21 +57,22 @@ def test_random_data_matches_truth(device, wide, M, N, K, layout):
 
 
 def test_when_the_route_applies(device, monkeypatch):
-    """kmc_gram_workspace_bytes: 0 without the split-bf16 flag, for a panel against itself, for
+    """kmc_gram_workspace_bytes: 0 without the split-bf16 flag, for
     short contractions and for problems of too few tiles of 256 x 256 over the batch for their k."""
-    a = torch.empty(5000, 512, device=device)
+    a = torch.empty(7000, 512, device=device)
     b = torch.empty(4000, 512, device=device)
     with kermac.l2_mode("gram_bf16"):
-        assert workspace_bytes(a, b) > 0                                         # 20 x 16 tiles
+        assert workspace_bytes(a, b) > 0                                         # 28 x 16 tiles
         assert workspace_bytes(a, b, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0) > 0
         assert workspace_bytes(a, b, kermac.kernel_descriptor_l1_norm) == 0
-        assert workspace_bytes(a, a) == 0                                        # symmetric: half the tiles, one-step kernel
+        assert 0 < workspace_bytes(a, a) < 0.6 * workspace_bytes(a, a.clone())   # 406 tiles of the triangle; one panel, split once
+        assert workspace_bytes(a[:3500], a[:3500]) == 0                          # 14 * 15 / 2 = 105 tiles of the triangle
         assert workspace_bytes(a[:2500], b[:2500]) == 0                          # 100 tiles
         assert workspace_bytes(a[:, :32], b[:, :32]) == 0                        # k < 64
         assert workspace_bytes(a[:, :128], b[:, :128]) == 0                      # 320 tiles at k = 128
         assert workspace_bytes(a[:2500].expand(3, 2500, 512), b[:2500].expand(3, 2500, 512)) > 0    # 300 over the batch
         needed = workspace_bytes(a, b)
-        operands = (5000 + 4000) * 512 * 4
+        operands = (7000 + 4000) * 512 * 4
         assert operands <= needed <= 2 * operands
     with kermac.l2_mode("gram"):
         assert workspace_bytes(a, b) == 0
@@ -225,3 +226,42 @@ def test_large_problem_takes_the_route_by_itself(device):
     truth = torch.cdist(a[:300].double(), b.double(), p=2.0)
     assert_close_to_truth(got[:300], truth, rtol=1e-5, what="auto, wide")
     assert not torch.isnan(got[::128, ::128]).any()
+
+
+@pytest.mark.parametrize("rows,K,col_major", [(129, 20, True), (700, 48, True), (515, 33, False), (1024, 64, False), (300, 200, True)])
+def test_a_panel_against_itself(device, wide, monkeypatch, rows, K, col_major):
+    """One workgroup per 256 x 256 tile on or below the diagonal; the result is symmetric bit for bit,
+    equals the full computation to rounding and the truth to the stated tolerance."""
+    g = torch.Generator().manual_seed(rows + K)
+    x = torch.randn(K, rows, generator=g).to(device).t() if col_major else torch.randn(rows, K, generator=g).to(device)
+    assert workspace_bytes(x, x) > 0
+    for out_col_major in (True, False):
+        store = torch.full((rows, rows + 4), float("nan"), device=device)
+        out = store[:, :rows].t() if out_col_major else store[:, :rows]
+        got = kermac.cdist(x, x, out=out, p=2.0)
+        assert got.shape == (rows, rows)
+        assert torch.equal(got, got.t()), "not symmetric"
+        assert torch.all(torch.diagonal(got) == 0)
+        assert torch.isnan(store[:, rows:]).all(), "wrote outside the out view"
+        full = kermac.cdist(x, x.clone(memory_format=torch.preserve_format), p=2.0)[0]
+        torch.testing.assert_close(got, full, rtol=2e-6, atol=1e-6)
+        assert_close_to_truth(got, oracle.cdist(x.cpu(), x.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30, what=f"self {rows}x{K}")
+
+
+def test_a_batch_of_panels_against_themselves_with_near_twins(device, wide):
+    g = torch.Generator().manual_seed(11)
+    L, rows, K = 3, 400, 40
+    x = torch.randn(L, K, rows, generator=g).to(device).transpose(1, 2)
+    bw = torch.tensor([5.0, 9.0, 14.0], device=device)
+    got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, x, bandwidth=bw, regularization=1e-3)
+    assert torch.equal(got, got.transpose(1, 2))
+    truth = oracle.build_kernel("DIFF", "SQUARE", "SQRT", "LAPLACE", x.cpu().contiguous(), x.cpu().contiguous(),
+                                bandwidth=bw.cpu(), regularization=1e-3)
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-7, what="batched self matrix")
+    # near-duplicate rows: those parts are recomputed, and mirrored, by the repair launch
+    y = torch.randn(600, 24, generator=g).to(device)
+    y[300:] = y[:300] + 1e-4 * torch.randn(300, 24, generator=g).to(device)
+    d_self = kermac.cdist(y, y, p=2.0)[0]
+    assert torch.equal(d_self, d_self.t())
+    assert not torch.isnan(d_self).any()
+    assert_close_to_truth(d_self, oracle.cdist(y.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30, what="near duplicates")
