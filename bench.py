@@ -371,8 +371,9 @@ def main():
             check_parity(f"cdist p={label} slab max rel err", e, rtol)
             per_p[label] = p_entry(k_ms, e, rtol)
         per_p["2.0"]["l2_mode"] = kermac.get_l2_mode()
-        per_p["2.0"]["note"] = ("default mode 'auto': |a-c|^2 + |b-c|^2 - 2 (a-c).(b-c) with the cross term on the bf16 matrix "
-                                "instruction (three exact bf16 pieces per operand), c = sample mean, ill-conditioned tiles "
+        per_p["2.0"]["note"] = ("default mode 'auto': |a-c|^2 + |b-c|^2 - 2 (a-c).(b-c), c = sample mean, with the cross term on "
+                                "the fp16 matrix instruction (both operands split once into two fp16 pieces per value, scaled per "
+                                "row, in a workspace; 256 x 256 tiles; three piece products), ill-conditioned 128 x 128 parts "
                                 "recomputed by the direct kernel; the vector-ALU kernel is per_p['2.0_direct']")
         # Fractional p costs five instructions per (m, n, k), two of them transcendentals that issue at a
         # quarter of the rate.  Rates measured with kermac_amd/_lib/valu_issue_rates (examples/valu_issue_rates.hip):
@@ -390,15 +391,25 @@ def main():
         # The two matrix-core paths for p = 2 by name (|a|^2 + |b|^2 - 2 a.b on fp32 MFMA, ill-conditioned tiles
         # recomputed directly); same 1e-5 tolerance.  The default 'auto' picks the second for this problem.
         # "gram_bf16": the cross term on the bf16 matrix instruction from three exact bf16 pieces per operand.
-        for mode, label in (("gram", "2.0_gram_mfma"), ("gram_bf16", "2.0_gram_bf16_mfma")):
-            log(f"timing p = 2.0, l2 mode '{mode}'")
-            with kermac.l2_mode(mode):
-                _, k_ms = time_cdist(kermac, a, b, out, 2.0, False, side_steps, 1)
-                e = parity_slab(out, a, b, 2.0, False)
+        # "gram_bf16" takes the workspace route for a problem of this size (two fp16 pieces, three products); with
+        # KERMAC_AMD_L2_WORKSPACE=0 it is the one-step kernel (three bf16 pieces split inside every workgroup, six products).
+        for mode, label, products, workspace in (("gram", "2.0_gram_mfma", 1, "1"), ("gram_bf16", "2.0_gram_bf16_mfma", 3, "1"),
+                                                 ("gram_bf16", "2.0_gram_bf16_one_step", 6, "0")):
+            log(f"timing p = 2.0, l2 mode '{mode}'" + ("" if workspace == "1" else " without a workspace"))
+            saved = os.environ.get("KERMAC_AMD_L2_WORKSPACE")
+            os.environ["KERMAC_AMD_L2_WORKSPACE"] = workspace
+            try:
+                with kermac.l2_mode(mode):
+                    _, k_ms = time_cdist(kermac, a, b, out, 2.0, False, side_steps, 1)
+                    e = parity_slab(out, a, b, 2.0, False)
+            finally:
+                if saved is None:
+                    del os.environ["KERMAC_AMD_L2_WORKSPACE"]
+                else:
+                    os.environ["KERMAC_AMD_L2_WORKSPACE"] = saved
             log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
-            check_parity(f"cdist p=2.0 ({mode}) slab max rel err", e, 1e-5)
-            per_p[label] = p_entry(k_ms, e, 1e-5, mfma_tflops=round((1 if mode == "gram" else 6) * 2.0 * M * N * K / k_ms / 1e9, 2),
-                                   l2_mode=mode)
+            check_parity(f"cdist p=2.0 ({label}) slab max rel err", e, 1e-5)
+            per_p[label] = p_entry(k_ms, e, 1e-5, mfma_tflops=round(products * 2.0 * M * N * K / k_ms / 1e9, 2), l2_mode=mode)
 
         # x against x (the kernel matrix of a training set): the library computes the tiles on and
         # below the diagonal only and stores each twice; bit-identical to the full computation.
@@ -409,6 +420,13 @@ def main():
         check_parity("cdist p=1.0 (a against itself) slab max rel err", e, 1e-5)
         per_p["1.0_a_against_itself"] = {"ms": round(k_ms, 3), "parity_max_rel_err": e, "rtol": 1e-5,
                                          "note": "symmetric result: half the tiles computed, each stored twice"}
+        log("timing p = 2.0, a against itself")
+        _, k_ms = time_cdist(kermac, a, a, out, 2.0, False, side_steps, 1)
+        e = parity_slab(out, a, a, 2.0, False, slabs=OFF_DIAGONAL_SLABS)
+        log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
+        check_parity("cdist p=2.0 (a against itself) slab max rel err", e, 1e-5)
+        per_p["2.0_a_against_itself"] = {"ms": round(k_ms, 3), "parity_max_rel_err": e, "rtol": 1e-5, "l2_mode": kermac.get_l2_mode(),
+                                         "note": "symmetric result on the workspace route: the 256 x 256 tiles on and below the diagonal"}
 
         # The two other configurations of the path, timed in this same run so that the default invocation
         # covers them: each entry is the line `--workload <name>` prints on its own.
@@ -427,7 +445,7 @@ def main():
     inner = {1.0: "POW_ABS", 2.0: "POW_SQUARE"}.get(headline_p, "POW_POW")
     headline_kernel = f"kmc::build_kernel<OP_DIFF,{inner},LOAD_COL_VEC,LOAD_COL_VEC>"
     if headline_p == 2.0 and kermac.get_l2_mode() != "direct":
-        headline_kernel = "kmc::gram_bf16_l2_kernel / kmc::gram_l2_kernel (l2 mode %s)" % kermac.get_l2_mode()
+        headline_kernel = "kmc::gram_f16_wide / kmc::gram_bf16_l2_kernel / kmc::gram_l2_kernel (l2 mode %s)" % kermac.get_l2_mode()
     line = {
         "metric": "cdist ms and % fp32-VALU peak at M=N=30000,K=1024 for p=1/1.3/2",
         "value": round(wall_ms, 3),
