@@ -167,9 +167,10 @@ typedef struct kmc_build_kernel_params {
 } kmc_build_kernel_params;
 
 /* Bytes of gram_workspace that kmc_build_kernel would use for these parameters, 0 when it would
- * not use one (no KMC_FLAG_L2_GRAM_BF16, a panel against itself, a problem too small to gain:
- * fewer than 128 tiles of 256 x 256 over the batch, k < 64, or tiles * k below 147456).  About 1.1 times the bytes of
- * both operands.  No counterpart in the reference. */
+ * not use one (no KMC_FLAG_L2_GRAM_BF16, or a problem too small to gain: fewer than 128 tiles of
+ * 256 x 256 over the batch, k < 64, or tiles * k below 147456; of a panel against itself the tiles
+ * on and below the diagonal count, and the panel is split once).  About 1.1 times the bytes of the
+ * operands.  No counterpart in the reference. */
 int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes);
 
 /* Stands in for launch(stream, config, cute_build_kernel<...>, *args)
