@@ -250,7 +250,22 @@ typedef struct kmc_norm_gradient_params {
     const float *d; int64_t d_ld; int64_t d_bs;   /* [n, m], m contiguous */
     float *e; int64_t e_ld_n; int64_t e_ld_o; int64_t e_bs; /* [o, n, m], m contiguous */
     const float *p; int64_t p_bs; float p_value;
+    /* KMC_NORM_L1 only (ignored otherwise): device memory the call may use, 256-byte aligned, of at
+     * least the size kmc_norm_gradient_workspace_bytes reports for these parameters.  With it, large
+     * problems run on the fp16 matrix instruction: a and c are split once into two fp16 pieces per
+     * value (a power-of-two scale per row m of a and per row o of c), the sign of d - b is put on
+     * the pieces of a exactly, and the contraction takes 3 matrix instructions per 32 k where the
+     * fp32 kernel issues 8 of twice the duration.  Error of e from the pieces below
+     * 3 * 2^-22 sum_k |c a|, beside the rounding of the fp32 accumulation that both kernels have.
+     * NULL, too small, or a problem for which the query reports 0: the fp32 kernels run. */
+    void *workspace;
+    int64_t workspace_bytes;
 } kmc_norm_gradient_params;
+
+/* Bytes of workspace that kmc_norm_kernel_gradient would use for these parameters, 0 when it would
+ * not use one (another norm than L1, fewer than 2e9 terms m * n * k * l).  About 1.1 times the
+ * bytes of a, b and c.  No counterpart in the reference. */
+int kmc_norm_gradient_workspace_bytes(const kmc_norm_gradient_params *params, int64_t *bytes);
 
 /* Stands in for launch(stream, config, cute_norm_kernel_gradient<NormType>, *args)
  * (src/kermac/cdist_grad.py:192-237). */

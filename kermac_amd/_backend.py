@@ -72,6 +72,7 @@ class NormGradientParams(Structure):
         ("d", _float_p), ("d_ld", c_int64), ("d_bs", c_int64),
         ("e", _float_p), ("e_ld_n", c_int64), ("e_ld_o", c_int64), ("e_bs", c_int64),
         ("p", _float_p), ("p_bs", c_int64), ("p_value", c_float),
+        ("workspace", c_void_p), ("workspace_bytes", c_int64),
     ]
 
 
@@ -102,6 +103,7 @@ SIGNATURES = {
     "kmc_gram_workspace_bytes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int64)]),
     "kmc_build_kernel_load_modes": (ctypes.c_int, [POINTER(BuildKernelParams), POINTER(c_int32), POINTER(c_int32)]),
     "kmc_norm_kernel_gradient": (ctypes.c_int, [POINTER(NormGradientParams), c_void_p]),
+    "kmc_norm_gradient_workspace_bytes": (ctypes.c_int, [POINTER(NormGradientParams), POINTER(c_int64)]),
     "kmc_kernel_times_coefficients": (ctypes.c_int, [POINTER(KernelCoefficientsParams), c_void_p]),
     "kmc_kernel_times_coefficients_has_variant": (ctypes.c_int, [c_int32, c_int32]),
     "kmc_kernel_times_coefficients_jit": (ctypes.c_int, [c_void_p, POINTER(KernelCoefficientsParams), c_void_p]),
@@ -216,6 +218,13 @@ def build_kernel_load_modes(params: BuildKernelParams) -> Tuple[int, int]:
     la, lb = c_int32(0), c_int32(0)
     check(library().kmc_build_kernel_load_modes(byref(params), byref(la), byref(lb)))
     return la.value, lb.value
+
+
+def norm_gradient_workspace_bytes(params: NormGradientParams) -> int:
+    """Bytes of workspace that kmc_norm_kernel_gradient would use for these parameters (0: none)."""
+    needed = c_int64(0)
+    check(library().kmc_norm_gradient_workspace_bytes(byref(params), byref(needed)))
+    return needed.value
 
 
 def norm_kernel_gradient(params: NormGradientParams, stream: int) -> None:

@@ -5,6 +5,7 @@ Same signature as the reference's ``kermac.cdist_grad``
 """
 from __future__ import annotations
 
+import os
 from typing import Union
 
 import numpy as np
@@ -162,8 +163,25 @@ def cdist_grad(
     stream = _current_stream_for(a.device)
     if debug:
         print(f"(Kermac Debug) Launching kernel: norm_kernel_gradient<{('L1', 'L2', 'P')[plan.params.norm_type]}>")
+    workspace = _attach_workspace(plan.params, a.device)
     _backend.norm_kernel_gradient(plan.params, stream)
+    del workspace           # the launches are queued: the allocator hands the memory on in stream order
     return plan.out
+
+
+def _attach_workspace(params, device):
+    """Large L1 gradients run on the fp16 matrix instruction through a workspace (include/
+    kermac_amd.h, kmc_norm_gradient_params::workspace: a and c split once into two fp16 pieces per
+    value, the sign of d - b put on the pieces of a); the library says how much it wants for this
+    call, 0 when it would not use one.  KERMAC_AMD_GRADIENT_WORKSPACE=0 keeps every call on the fp32 kernels."""
+    if os.environ.get("KERMAC_AMD_GRADIENT_WORKSPACE", "1") in ("", "0"):
+        return None
+    needed = _backend.norm_gradient_workspace_bytes(params)
+    if needed == 0:
+        return None
+    workspace = torch.empty(needed, dtype=torch.uint8, device=device)
+    params.workspace, params.workspace_bytes = workspace.data_ptr(), needed
+    return workspace
 
 
 # A workgroup owns 64 (m) x 32 or 16 (n) results and walks the whole contraction index k,

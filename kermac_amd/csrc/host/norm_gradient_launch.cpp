@@ -7,6 +7,9 @@ using namespace kmc_host;
 namespace kmc_host {
 hipError_t launch_norm_gradient(int norm_type, int o_tile, const kmc::NormGradientArgs &args, dim3 grid,
                                 hipStream_t stream);
+int64_t norm_gradient_f16_bytes(const kmc_norm_gradient_params *p);
+hipError_t launch_norm_gradient_f16(const kmc_norm_gradient_params *p, bool a_vec, bool c_vec, bool e_vec, hipStream_t stream,
+                                    bool *taken);
 }
 
 namespace {
@@ -18,7 +21,9 @@ bool vec_ok(const void *ptr, int64_t s0, int64_t s1, int64_t s2, int flags)
 
 }  // namespace
 
-extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void *stream)
+namespace {
+
+int check(const kmc_norm_gradient_params *p)
 {
     if (!p) return fail(KMC_ERR_INVALID_ARGUMENT, "null parameter block");
     if (p->norm_type < KMC_NORM_L1 || p->norm_type > KMC_NORM_P)
@@ -26,6 +31,7 @@ extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void 
     if (p->m < 0 || p->n < 0 || p->o < 0 || p->k < 0 || p->l < 0)
         return fail(KMC_ERR_INVALID_ARGUMENT, "negative extent (m=%d n=%d o=%d k=%d l=%d)", p->m, p->n, p->o, p->k, p->l);
     if (p->m == 0 || p->n == 0 || p->o == 0 || p->l == 0) return KMC_OK;
+    if (p->l > 65535) return fail(KMC_ERR_INVALID_ARGUMENT, "batch count %d exceeds 65535", p->l);
     if (!p->e || !p->d || (p->k > 0 && (!p->a || !p->b || !p->c)))
         return fail(KMC_ERR_INVALID_ARGUMENT, "null tensor pointer");
     if ((p->k > 1 && p->a_ld < p->m) || (p->n > 1 && p->b_ld < p->k) || (p->o > 1 && p->c_ld < p->k) ||
@@ -34,6 +40,35 @@ extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void 
     if (p->a_ld < 0 || p->b_ld < 0 || p->c_ld < 0 || p->d_ld < 0 || p->e_ld_n < 0 || p->e_ld_o < 0 || p->a_bs < 0 ||
         p->b_bs < 0 || p->c_bs < 0 || p->d_bs < 0 || p->e_bs < 0 || p->p_bs < 0)
         return fail(KMC_ERR_INVALID_ARGUMENT, "negative stride");
+    return KMC_OK;
+}
+
+}  // namespace
+
+extern "C" int kmc_norm_gradient_workspace_bytes(const kmc_norm_gradient_params *p, int64_t *bytes)
+{
+    if (!bytes) return fail(KMC_ERR_INVALID_ARGUMENT, "bytes: null pointer");
+    int status = check(p);
+    if (status != KMC_OK) return status;
+    *bytes = (p->m == 0 || p->n == 0 || p->o == 0 || p->l == 0) ? 0 : norm_gradient_f16_bytes(p);
+    return KMC_OK;
+}
+
+extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void *stream)
+{
+    int checked = check(p);
+    if (checked != KMC_OK) return checked;
+    if (p->m == 0 || p->n == 0 || p->o == 0 || p->l == 0) return KMC_OK;
+    if (p->norm_type == KMC_NORM_L1 && p->workspace) {
+        int ready = require_gfx950();
+        if (ready != KMC_OK) return ready;
+        bool taken = false;
+        hipError_t e = launch_norm_gradient_f16(p, vec_ok(p->a, p->a_ld, p->a_bs, 0, p->flags), vec_ok(p->c, p->c_ld, p->c_bs, 0, p->flags),
+                                                vec_ok(p->e, p->e_ld_n, p->e_ld_o, p->e_bs, p->flags), static_cast<hipStream_t>(stream),
+                                                &taken);
+        if (e != hipSuccess) return fail_hip(e, "norm_gradient_l1_f16 launches");
+        if (taken) return KMC_OK;
+    }
 
     // The outputs are cut into at most three runs, each with the kernel that suits its
     // width: whole groups of 32 (and a remainder of 25..31) on the matrix-core kernel with

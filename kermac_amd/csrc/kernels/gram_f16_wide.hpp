@@ -72,6 +72,8 @@ struct GramRowsArgs {
     float *unscale;                       // [batch][rows_pad]: 1 / the row's scale
     i64 stats_bs, unscale_bs;
     int rows_pad, slices, slices_per_range, ranges;
+    int zero_slices;                      // slices behind the last that gram_f16_split fills with zeros (for
+                                          // walks in steps of more than one slice)
 };
 
 struct GramWideArgs {
@@ -123,7 +125,9 @@ __device__ __forceinline__ const float *gram_rows_centre(const GramRowsArgs &arg
     return centre[padded] != 0.0f ? centre : nullptr;      // the flag behind the vector: see centre_to_subtract
 }
 
-// One thread per row, one workgroup per 256 rows and range of slices.
+// One thread per row, one workgroup per 256 rows and range of slices.  (The two row kernels are
+// templates only so that every translation unit that includes this header may hold them.)
+template <int UNUSED = 0>
 __global__ __launch_bounds__(GW_ROW_THREADS) void gram_row_stats(const GramRowsArgs args)
 {
     const int row = blockIdx.x * GW_ROW_THREADS + threadIdx.x;
@@ -149,6 +153,7 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_row_stats(const GramRowsA
     args.magnitudes[at] = not_a_number ? __builtin_nanf("") : magnitude;
 }
 
+template <int UNUSED = 0>
 __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsArgs args)
 {
     const int row = blockIdx.x * GW_ROW_THREADS + threadIdx.x;
@@ -195,6 +200,13 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsA
             for (int half = 0; half < 2; half++)
                 dst[(i64)(2 * p + half) * args.rows_pad] =
                     gram_chunk{piece[p][4 * half], piece[p][4 * half + 1], piece[p][4 * half + 2], piece[p][4 * half + 3]};
+    }
+    if (range == args.ranges - 1) {
+        for (int slice = args.slices; slice < args.slices + args.zero_slices; slice++) {
+            gram_chunk *dst = pieces + (i64)slice * GW_SEGMENTS * args.rows_pad + row;
+#pragma unroll
+            for (int segment = 0; segment < GW_SEGMENTS; segment++) dst[(i64)segment * args.rows_pad] = gram_chunk{0u, 0u, 0u, 0u};
+        }
     }
 }
 

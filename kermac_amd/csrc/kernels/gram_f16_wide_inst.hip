@@ -111,15 +111,16 @@ kmc::GramRowsArgs rows_args(const float *x, int64_t ld, int64_t bs, int rows, in
     return rows_of;
 }
 
-hipError_t launch_rows(const kmc::GramRowsArgs &rows_of, int batches, hipStream_t stream)
+}  // namespace
+
+// Statistics and split of one operand (also used by the gradient's fp16 route).
+hipError_t launch_gram_rows(const kmc::GramRowsArgs &rows_of, int batches, hipStream_t stream)
 {
     const dim3 grid(rows_of.rows_pad / kmc::GW_ROW_THREADS, rows_of.ranges, batches);
-    hipError_t status = launch(kmc::gram_row_stats, grid, dim3(kmc::GW_ROW_THREADS), stream, rows_of);
+    hipError_t status = launch(kmc::gram_row_stats<0>, grid, dim3(kmc::GW_ROW_THREADS), stream, rows_of);
     if (status != hipSuccess) return status;
-    return launch(kmc::gram_f16_split, grid, dim3(kmc::GW_ROW_THREADS), stream, rows_of);
+    return launch(kmc::gram_f16_split<0>, grid, dim3(kmc::GW_ROW_THREADS), stream, rows_of);
 }
-
-}  // namespace
 
 // Bytes of workspace the path needs for this problem; 0 when it does not apply.
 int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args)
@@ -141,10 +142,10 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     const bool scalar_only = (p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) != 0;
     const kmc::GramRowsArgs rows_a = rows_args(args.a, args.a_ld, args.a_bs, args.m, p->a_majorness, scalar_only, args, layout, layout.a, workspace);
     const kmc::GramRowsArgs rows_b = rows_args(args.b, args.b_ld, args.b_bs, args.n, p->b_majorness, scalar_only, args, layout, layout.b, workspace);
-    hipError_t status = launch_rows(rows_a, layout.a.batches, stream);
+    hipError_t status = launch_gram_rows(rows_a, layout.a.batches, stream);
     if (status != hipSuccess) return status;
     if (!args.symmetric) {
-        status = launch_rows(rows_b, layout.b.batches, stream);
+        status = launch_gram_rows(rows_b, layout.b.batches, stream);
         if (status != hipSuccess) return status;
     }
 

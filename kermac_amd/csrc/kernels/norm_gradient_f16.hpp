@@ -1,0 +1,254 @@
+// Kernel-gradient contraction for the L1 norm on the fp16 matrix instruction:
+//
+//   E[m, n, o, l] = sum_k C[o,k,l] * A[m,k,l] * s(m,n,k),     s = copysign(1, D[m,n,l] - B[n,k,l])
+//
+// (reference: include/p_norm_gradient.cuh:407-497 with NormType::L1, whose weight of a term is
+// the sign of d - b, :373-394).  The factor that depends on all of m, n and k is a sign, and a
+// sign can be put on a 16-bit piece exactly.  So A and C are split once, like the operands of
+// gram_f16_wide.hpp and by the same two kernels (a power-of-two scale per row m of A and per row
+// o of C, two fp16 pieces per scaled value, 16-byte chunks of 8 k in the order the matrix
+// instruction reads them), and the contraction over k runs on v_mfma_f32_16x16x32_f16 with
+//
+//   T1 = +-a1, T2 = +-a2 (the sign bit of d - b flipped into both pieces),   T1 c1 + T1 c2 + T2 c1
+//
+// per 32 k: 3 matrix instructions of 16 cycles where the fp32 kernel (norm_gradient_mfma.hpp)
+// issues 8 of 32 cycles.  What a lane computes per (m, n, k) is one subtraction, half a byte
+// permute, half an AND and two halves of an XOR: 3 vector instructions, as many as the fp32
+// kernel spends, which now bound the kernel instead of the matrix pipeline.
+// Accuracy: as in gram_f16_wide.hpp, |x - h1 - h2| <= 2^-22 |x| per value and the dropped product
+// a2 c2 below 2^-22 |a c|: the error of E from the pieces is below 3 * 2^-22 sum_k |c a|, the size
+// of the rounding of an fp32 accumulation over a few terms, beside the fp32 accumulation itself.
+//
+// Workgroup: 4 waves, 64 m x 32 n x 16 o; wave w owns the 8 n  8w .. 8w + 7  and all 64 m as 4 row
+// blocks of 16.  Per 32 k it reads the pieces of C (2 x 16 bytes per lane) and of its A rows
+// (8 x 16 bytes), and per n the 8 values of B that match its 8 k (2 x 16 bytes, the same for the
+// 16 lanes of a row block).  B is copied once into a padded array in the workspace (rows to 32,
+// k to 32 plus what the walk copies ahead), so that everything the walk touches exists and all of
+// it arrives in LDS by global_load_lds_dwordx4, three steps in three buffers, as in
+// gram_f16_wide.hpp (the copies are inline instructions for the reason given there).
+#pragma once
+
+#include "gram_f16_wide.hpp"
+#include "norm_gradient.hpp"
+
+namespace kmc {
+
+typedef float ngf_float4 __attribute__((ext_vector_type(4)));
+
+constexpr int NGF_TILE_M = 64;
+constexpr int NGF_TILE_N = 32;
+constexpr int NGF_TILE_O = 16;
+constexpr int NGF_WAVE_N = 8;
+constexpr int NGF_STEP_K = 32;                 // two slices of the split
+constexpr int NGF_THREADS = 256;
+constexpr int NGF_AHEAD = 3;                   // steps copied ahead of the walk
+constexpr int NGF_A_CHUNKS = 8 * NGF_TILE_M;   // per step: 8 runs (slice, piece, half) of 64 rows
+constexpr int NGF_C_CHUNKS = 8 * NGF_TILE_O;
+constexpr int NGF_B_CHUNKS = NGF_TILE_N * NGF_STEP_K / 4;
+constexpr int NGF_BUFFER_CHUNKS = NGF_A_CHUNKS + NGF_C_CHUNKS + NGF_B_CHUNKS;      // 14 KB
+
+struct NormGradientF16Args {
+    NormGradientArgs g;                        // extents, d, e, strides, o_chunks (of NGF_TILE_O); a, b, c are not read
+    const gram_chunk *pieces_a, *pieces_c;     // gram_f16_split of A (rows m) and of C (rows o)
+    i64 pieces_a_bs, pieces_c_bs;              // per batch entry, in chunks
+    const float *unscale_a, *unscale_c;
+    i64 unscale_a_bs, unscale_c_bs;
+    const float *b_padded;                     // [batch][n_pad][k_pad]
+    i64 b_padded_bs;
+    int rows_pad_a, rows_pad_c, k_pad, steps;
+};
+
+struct GradientPadArgs {
+    const float *b; i64 b_ld, b_bs;
+    float *padded; i64 padded_bs;
+    int n, k, n_pad, k_pad;
+};
+
+// padded[batch][n][k] = b[batch][n][k], zeros beyond n and k.  One thread per 4 k.
+__global__ __launch_bounds__(256) void gradient_pad_b(const GradientPadArgs args)
+{
+    const int quad = blockIdx.x * 256 + threadIdx.x;
+    const int n = blockIdx.y, batch = blockIdx.z;
+    if (quad * 4 >= args.k_pad) return;
+    const float *src = args.b + batch * args.b_bs + (i64)n * args.b_ld;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = (n < args.n && quad * 4 + e < args.k) ? src[quad * 4 + e] : 0.0f;
+    *reinterpret_cast<float4 *>(args.padded + batch * args.padded_bs + (i64)n * args.k_pad + quad * 4) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+__global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const NormGradientF16Args args)
+{
+    __shared__ gram_chunk lds0[NGF_BUFFER_CHUNKS];
+    __shared__ gram_chunk lds1[NGF_BUFFER_CHUNKS];
+    __shared__ gram_chunk lds2[NGF_BUFFER_CHUNKS];
+
+    const NormGradientArgs &g = args.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int q = lane >> 4;     // 8 k of a step (operands), row quad (result)
+    const int r = lane & 15;     // row m (T) / column o (C, result)
+    const int batch = blockIdx.z / g.o_chunks;
+    const int o0 = (blockIdx.z % g.o_chunks) * NGF_TILE_O;
+    const int m0 = blockIdx.x * NGF_TILE_M;
+    const int n0 = blockIdx.y * NGF_TILE_N;
+
+    auto buffer = [&](auto which) -> gram_chunk * {
+        constexpr int B = decltype(which)::value;
+        if constexpr (B == 0) return lds0;
+        else if constexpr (B == 1) return lds1;
+        else return lds2;
+    };
+
+    // Copies per step: A 8 runs of 64 chunks (one per wave and run: 2 per wave), C 8 runs of 16
+    // chunks (2 copies of 4 runs; waves 0 and 2 issue the first, 1 and 3 the second: the same bytes
+    // twice, so that every wave has the same number of copies under way), B 32 rows of 128 bytes
+    // (8 rows per copy, one per wave).  A run (slice, piece, half) of a step starts at chunk
+    // ((2 step + slice) * 4 + 2 piece + half) * rows_pad of an operand's pieces.
+    typedef const __attribute__((address_space(1))) void *global_address;
+    typedef __attribute__((address_space(3))) void *lds_address;
+    const gram_chunk *src[4];
+    i64 advance[4];
+    int dst[4];
+    {
+        const gram_chunk *pieces_a = args.pieces_a + batch * args.pieces_a_bs + m0;
+        const gram_chunk *pieces_c = args.pieces_c + batch * args.pieces_c_bs + o0;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int run = 2 * wave + j;
+            src[j] = pieces_a + (i64)run * args.rows_pad_a + lane;
+            advance[j] = (i64)8 * args.rows_pad_a;
+            dst[j] = run * NGF_TILE_M;
+        }
+        const int c_run = 4 * (wave & 1) + q;
+        src[2] = pieces_c + (i64)c_run * args.rows_pad_c + r;
+        advance[2] = (i64)8 * args.rows_pad_c;
+        dst[2] = NGF_A_CHUNKS + 64 * (wave & 1);
+        // 8 rows of B per wave: lane -> row lane / 8, 16 bytes number lane % 8 of the step's 128
+        const float *b_row = args.b_padded + batch * args.b_padded_bs + (i64)(n0 + 8 * wave + (lane >> 3)) * args.k_pad + 4 * (lane & 7);
+        src[3] = reinterpret_cast<const gram_chunk *>(b_row);
+        advance[3] = NGF_STEP_K / 4;
+        dst[3] = NGF_A_CHUNKS + NGF_C_CHUNKS + 64 * wave;
+    }
+    auto copy_step = [&](auto into) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const unsigned lds_byte = (unsigned)(unsigned long)(lds_address)(buffer(into) + dst[j]);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :
+                         : "v"((global_address)src[j]), "s"(lds_byte)
+                         : "memory", "m0");
+            src[j] += advance[j];
+        }
+    };
+
+    // D[m, n] of this lane's rows, for the 8 n of the wave.
+    float dval[NGF_WAVE_N][4];
+    {
+        const float *d_base = g.d + batch * g.d_bs;
+#pragma unroll
+        for (int nb = 0; nb < NGF_WAVE_N; nb++) {
+            const int n = n0 + NGF_WAVE_N * wave + nb;
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+                const int m = m0 + 16 * mb + r;
+                dval[nb][mb] = (n < g.n && m < g.m) ? d_base[(i64)n * g.d_ld + m] : 0.0f;
+            }
+        }
+    }
+    // the copies are not counted by the compiler: nothing it loads may be under way beside them
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
+    ngf_float4 acc[NGF_WAVE_N][4];
+#pragma unroll
+    for (int nb = 0; nb < NGF_WAVE_N; nb++)
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) acc[nb][mb] = ngf_float4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // lane (q, r): its 8 k are slice q / 2, half q % 2 of the step
+    const int run_of_lane = 4 * (q >> 1) + (q & 1);      // + 2 piece
+    auto step = [&](auto which) {
+        const gram_chunk *lds = buffer(which);
+        gram_half8 fc[GW_PIECES], fa[4][GW_PIECES];
+#pragma unroll
+        for (int p = 0; p < GW_PIECES; p++) fc[p] = __builtin_bit_cast(gram_half8, lds[NGF_A_CHUNKS + (run_of_lane + 2 * p) * NGF_TILE_O + r]);
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int p = 0; p < GW_PIECES; p++)
+                fa[mb][p] = __builtin_bit_cast(gram_half8, lds[(run_of_lane + 2 * p) * NGF_TILE_M + 16 * mb + r]);
+        const float4 *b_rows = reinterpret_cast<const float4 *>(lds + NGF_A_CHUNKS + NGF_C_CHUNKS);
+#pragma unroll
+        for (int nb = 0; nb < NGF_WAVE_N; nb++) {
+            const float4 b_low = b_rows[(NGF_WAVE_N * wave + nb) * (NGF_STEP_K / 4) + 2 * q];
+            const float4 b_high = b_rows[(NGF_WAVE_N * wave + nb) * (NGF_STEP_K / 4) + 2 * q + 1];
+            const float bk[8] = {b_low.x, b_low.y, b_low.z, b_low.w, b_high.x, b_high.y, b_high.z, b_high.w};
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+                gram_chunk t1 = __builtin_bit_cast(gram_chunk, fa[mb][0]);
+                gram_chunk t2 = __builtin_bit_cast(gram_chunk, fa[mb][1]);
+#pragma unroll
+                for (int pair = 0; pair < 4; pair++) {
+                    const unsigned low = __float_as_uint(dval[nb][mb] - bk[2 * pair]);
+                    const unsigned high = __float_as_uint(dval[nb][mb] - bk[2 * pair + 1]);
+                    // the two sign bits, at the sign bits of the two halves of a dword
+                    const unsigned flip = __builtin_amdgcn_perm(high, low, 0x070c030c) & 0x80008000u;
+                    t1[pair] ^= flip;
+                    t2[pair] ^= flip;
+                }
+                const gram_half8 h1 = __builtin_bit_cast(gram_half8, t1), h2 = __builtin_bit_cast(gram_half8, t2);
+                acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h2, fc[0], acc[nb][mb], 0, 0, 0);
+                acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[1], acc[nb][mb], 0, 0, 0);
+                acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[0], acc[nb][mb], 0, 0, 0);
+            }
+        }
+        // the wave's own copies of the next step have arrived (the four of the step after it may
+        // still be under way); behind the barrier everybody's have, and this step's buffer is free
+        __builtin_amdgcn_s_waitcnt(0x0F74);
+        __syncthreads();
+        copy_step(which);
+    };
+
+    copy_step(GramStep<0>{});
+    copy_step(GramStep<1>{});
+    copy_step(GramStep<2>{});
+    __builtin_amdgcn_s_waitcnt(0x0F78);                     // vmcnt(8): step 0 has arrived
+    __syncthreads();
+    for (int done = 0;;) {
+        step(GramStep<0>{});
+        if (++done == args.steps) break;
+        step(GramStep<1>{});
+        if (++done == args.steps) break;
+        step(GramStep<2>{});
+        if (++done == args.steps) break;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
+    // acc[nb][mb][j]: m = m0 + 16 mb + 4 q + j, o = o0 + r, n = n0 + 8 wave + nb
+    const int o = o0 + r;
+    const float unscale_c = args.unscale_c[batch * args.unscale_c_bs + o];
+    float *e_base = g.e + batch * g.e_bs + (i64)o * g.e_ld_o;
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) {
+        const int m = m0 + 16 * mb + 4 * q;
+        const float4 unscale_a = *reinterpret_cast<const float4 *>(args.unscale_a + batch * args.unscale_a_bs + m);
+#pragma unroll
+        for (int nb = 0; nb < NGF_WAVE_N; nb++) {
+            const int n = n0 + NGF_WAVE_N * wave + nb;
+            if (n >= g.n || o >= g.o) continue;
+            const float v[4] = {acc[nb][mb][0] * unscale_a.x * unscale_c, acc[nb][mb][1] * unscale_a.y * unscale_c,
+                                acc[nb][mb][2] * unscale_a.z * unscale_c, acc[nb][mb][3] * unscale_a.w * unscale_c};
+            float *dst = e_base + (i64)n * g.e_ld_n + m;
+            if (g.e_vec && m + 3 < g.m) {
+                *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (m + j < g.m) dst[j] = v[j];
+            }
+        }
+    }
+}
+
+}  // namespace kmc

@@ -1,0 +1,162 @@
+// Host side of the L1 kernel gradient on the fp16 matrix instruction (norm_gradient_f16.hpp): when
+// it applies, how the caller's workspace is divided, and the launches: row statistics and split of
+// A (rows m) and of C (rows o) by the kernels of gram_f16_wide.hpp, a padded copy of B, the
+// contraction.
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+
+#include "../host/host_common.hpp"
+#include "launch.hpp"
+#include "norm_gradient_f16.hpp"
+
+namespace kmc_host {
+
+namespace {
+
+constexpr int64_t REGION_ALIGN = 256;
+
+struct RowsRegions {
+    int rows_pad, batches;
+    int64_t pieces_bs, stats_bs;
+    int64_t pieces, squares, magnitudes, unscale;     // byte offsets into the workspace
+};
+
+struct GradientLayout {
+    int slices, slices_alloc, slices_per_range, ranges, steps;
+    int n_pad, k_pad, b_batches;
+    RowsRegions a, c;
+    int64_t b_padded, b_padded_bs;
+    int64_t bytes;
+};
+
+int64_t place(int64_t &cursor, int64_t bytes)
+{
+    const int64_t at = cursor;
+    cursor = (cursor + bytes + REGION_ALIGN - 1) / REGION_ALIGN * REGION_ALIGN;
+    return at;
+}
+
+void place_rows(RowsRegions &r, int rows, int batches, const GradientLayout &layout, int64_t &cursor)
+{
+    r.rows_pad = (rows + kmc::GW_TILE - 1) / kmc::GW_TILE * kmc::GW_TILE;
+    r.batches = batches;
+    r.pieces_bs = static_cast<int64_t>(layout.slices_alloc) * kmc::GW_SEGMENTS * r.rows_pad;
+    r.stats_bs = static_cast<int64_t>(layout.ranges) * r.rows_pad;
+    r.pieces = place(cursor, r.batches * r.pieces_bs * 16);
+    r.squares = place(cursor, r.batches * r.stats_bs * 4);
+    r.magnitudes = place(cursor, r.batches * r.stats_bs * 4);
+    r.unscale = place(cursor, static_cast<int64_t>(r.batches) * r.rows_pad * 4);
+}
+
+// The route pays where the fp32 kernels are bound by their matrix or vector instructions: enough
+// terms to fill the chip and to carry the five extra launches.  KERMAC_AMD_GRADIENT_F16_MIN_TERMS
+// replaces the threshold (read on every call, so that a test can send small shapes down the route).
+bool f16_pays(const kmc_norm_gradient_params *p)
+{
+    const char *text = std::getenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS");
+    const double forced = text ? std::atof(text) : 0.0;
+    const double terms = static_cast<double>(p->m) * p->n * p->k * p->l;
+    return terms >= (forced > 0.0 ? forced : 2e9);
+}
+
+bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)
+{
+    if (p->norm_type != KMC_NORM_L1 || p->m < 1 || p->n < 1 || p->o < 1 || p->k < 1 || p->l < 1) return false;
+    if (!f16_pays(p)) return false;
+    layout->slices = (p->k + kmc::BK_TILE_K - 1) / kmc::BK_TILE_K;
+    layout->steps = (p->k + kmc::NGF_STEP_K - 1) / kmc::NGF_STEP_K;
+    layout->slices_alloc = 2 * (layout->steps + kmc::NGF_AHEAD);
+    layout->slices_per_range = layout->slices / 8 > 8 ? (layout->slices + 7) / 8 : 8;
+    layout->ranges = (layout->slices + layout->slices_per_range - 1) / layout->slices_per_range;
+    layout->n_pad = (p->n + kmc::NGF_TILE_N - 1) / kmc::NGF_TILE_N * kmc::NGF_TILE_N;
+    layout->k_pad = kmc::NGF_STEP_K * (layout->steps + kmc::NGF_AHEAD);
+    int64_t cursor = 0;
+    place_rows(layout->a, p->m, p->a_bs == 0 ? 1 : p->l, *layout, cursor);
+    place_rows(layout->c, p->o, p->c_bs == 0 ? 1 : p->l, *layout, cursor);
+    layout->b_batches = p->b_bs == 0 ? 1 : p->l;
+    layout->b_padded_bs = static_cast<int64_t>(layout->n_pad) * layout->k_pad;
+    layout->b_padded = place(cursor, layout->b_batches * layout->b_padded_bs * 4);
+    layout->bytes = cursor;
+    const int64_t grid_z = static_cast<int64_t>(p->l) * ((p->o + kmc::NGF_TILE_O - 1) / kmc::NGF_TILE_O);
+    if (grid_z > 65535 || layout->n_pad / kmc::NGF_TILE_N > 65535 || layout->n_pad > 65535) return false;
+    return true;
+}
+
+kmc::GramRowsArgs rows_args(const float *x, int64_t ld, int64_t bs, int rows, bool row_major, bool vec, int k,
+                            const GradientLayout &layout, const RowsRegions &r, char *workspace)
+{
+    kmc::GramRowsArgs rows_of = {};
+    rows_of.x = x; rows_of.ld = ld; rows_of.bs = bs;
+    rows_of.rows = rows; rows_of.k = k;
+    rows_of.row_major = row_major; rows_of.vec = row_major && vec;
+    rows_of.pieces = reinterpret_cast<kmc::gram_chunk *>(workspace + r.pieces); rows_of.pieces_bs = r.pieces_bs;
+    rows_of.squares = reinterpret_cast<float *>(workspace + r.squares);
+    rows_of.magnitudes = reinterpret_cast<float *>(workspace + r.magnitudes);
+    rows_of.unscale = reinterpret_cast<float *>(workspace + r.unscale);
+    rows_of.stats_bs = r.stats_bs; rows_of.unscale_bs = r.rows_pad;
+    rows_of.rows_pad = r.rows_pad; rows_of.slices = layout.slices;
+    rows_of.slices_per_range = layout.slices_per_range; rows_of.ranges = layout.ranges;
+    rows_of.zero_slices = 2 * layout.steps - layout.slices;      // the walk takes two slices per step
+    return rows_of;
+}
+
+}  // namespace
+
+hipError_t launch_gram_rows(const kmc::GramRowsArgs &rows_of, int batches, hipStream_t stream);     // gram_f16_wide_inst.hip
+
+int64_t norm_gradient_f16_bytes(const kmc_norm_gradient_params *p)
+{
+    GradientLayout layout;
+    return gradient_layout(p, &layout) ? layout.bytes : 0;
+}
+
+// `*taken` says whether the route applied (and the launches were made); if not, nothing was launched.
+hipError_t launch_norm_gradient_f16(const kmc_norm_gradient_params *p, bool a_vec, bool c_vec, bool e_vec, hipStream_t stream,
+                                    bool *taken)
+{
+    *taken = false;
+    GradientLayout layout;
+    if (!p->workspace || !gradient_layout(p, &layout) || p->workspace_bytes < layout.bytes ||
+        (reinterpret_cast<uintptr_t>(p->workspace) & (REGION_ALIGN - 1)) != 0)
+        return hipSuccess;
+    char *workspace = static_cast<char *>(p->workspace);
+    (void)a_vec;
+    const kmc::GramRowsArgs rows_a = rows_args(p->a, p->a_ld, p->a_bs, p->m, false, false, p->k, layout, layout.a, workspace);
+    const kmc::GramRowsArgs rows_c = rows_args(p->c, p->c_ld, p->c_bs, p->o, true, c_vec, p->k, layout, layout.c, workspace);
+    hipError_t status = launch_gram_rows(rows_a, layout.a.batches, stream);
+    if (status != hipSuccess) return status;
+    status = launch_gram_rows(rows_c, layout.c.batches, stream);
+    if (status != hipSuccess) return status;
+
+    kmc::GradientPadArgs pad = {};
+    pad.b = p->b; pad.b_ld = p->b_ld; pad.b_bs = p->b_bs;
+    pad.padded = reinterpret_cast<float *>(workspace + layout.b_padded); pad.padded_bs = layout.b_padded_bs;
+    pad.n = p->n; pad.k = p->k; pad.n_pad = layout.n_pad; pad.k_pad = layout.k_pad;
+    status = launch(kmc::gradient_pad_b, dim3((layout.k_pad / 4 + 255) / 256, layout.n_pad, layout.b_batches), dim3(256), stream, pad);
+    if (status != hipSuccess) return status;
+
+    kmc::NormGradientF16Args args = {};
+    args.g.m = p->m; args.g.n = p->n; args.g.o = p->o; args.g.k = p->k; args.g.l = p->l;
+    args.g.d = p->d; args.g.d_ld = p->d_ld; args.g.d_bs = p->d_bs;
+    args.g.e = p->e; args.g.e_ld_n = p->e_ld_n; args.g.e_ld_o = p->e_ld_o; args.g.e_bs = p->e_bs;
+    args.g.o_chunks = (p->o + kmc::NGF_TILE_O - 1) / kmc::NGF_TILE_O;
+    args.g.e_vec = e_vec;
+    args.pieces_a = rows_a.pieces; args.pieces_c = rows_c.pieces;
+    args.pieces_a_bs = layout.a.batches > 1 ? layout.a.pieces_bs : 0;
+    args.pieces_c_bs = layout.c.batches > 1 ? layout.c.pieces_bs : 0;
+    args.unscale_a = rows_a.unscale; args.unscale_c = rows_c.unscale;
+    args.unscale_a_bs = layout.a.batches > 1 ? layout.a.rows_pad : 0;
+    args.unscale_c_bs = layout.c.batches > 1 ? layout.c.rows_pad : 0;
+    args.b_padded = pad.padded;
+    args.b_padded_bs = layout.b_batches > 1 ? layout.b_padded_bs : 0;
+    args.rows_pad_a = layout.a.rows_pad; args.rows_pad_c = layout.c.rows_pad;
+    args.k_pad = layout.k_pad; args.steps = layout.steps;
+    const dim3 grid((p->m + kmc::NGF_TILE_M - 1) / kmc::NGF_TILE_M, layout.n_pad / kmc::NGF_TILE_N,
+                    static_cast<unsigned>(p->l) * args.g.o_chunks);
+    status = launch(kmc::norm_gradient_l1_f16, grid, dim3(kmc::NGF_THREADS), stream, args);
+    if (status == hipSuccess) *taken = true;
+    return status;
+}
+
+}  // namespace kmc_host
