@@ -214,13 +214,33 @@ def bench_cdist_grad(kermac, device, args, steps=None, warmup=None):
     err = ((out[0][:, ns, ms].double() - truth).abs().max() / truth.abs().mean()).item()
     log(f"cdist_grad p=1: {kernel_ms:.2f} ms kernel, slab max abs err / mean |truth| = {err:.2e}")
     check_parity("cdist_grad p=1 (configs[3]) slab, max abs err / mean |truth|", err, 1e-4)
-    ops = (2.0 * o + 3.0) * m_ref * n_ref * k_ref
+    # The same call on the fp32 kernels (no workspace), timed beside it.
+    saved = os.environ.get("KERMAC_AMD_GRADIENT_WORKSPACE")
+    os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"] = "0"
+    try:
+        _, fp32_ms = time_call(lambda: kermac.cdist_grad(a, b, c, d, out=out, p=1.0), max(2, min(steps, 5)), 1)
+        fp32_err = ((out[0][:, ns, ms].double() - truth).abs().max() / truth.abs().mean()).item()
+    finally:
+        if saved is None:
+            del os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"]
+        else:
+            os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"] = saved
+    log(f"  on the fp32 matrix-core kernel: {fp32_ms:.2f} ms, slab max abs err / mean |truth| = {fp32_err:.2e}")
+    check_parity("cdist_grad p=1 (configs[3], fp32 kernels) slab, max abs err / mean |truth|", fp32_err, 1e-4)
+    # Executed matrix work on the default route: three products of fp16 pieces, 2 * O flops each per (m, n, k),
+    # against the dense fp16 peak; the sign work on the vector ALU (2.5 instructions per (m, n, k)) is what bounds it.
+    ops = 3.0 * 2.0 * o * m_ref * n_ref * k_ref
     nbytes = 4.0 * (k_ref * m_ref + n_ref * k_ref + o * k_ref + n_ref * m_ref + o * n_ref * m_ref)
     return side_line("cdist_grad ms, Laplace-kernel RFM gradient M=8192 N=512 O=16 K=8192 p=1",
                      "cdist_grad p=1.0 fp32: a[8192,8192] U(0,1), b[512,8192], d[512,8192] N(0,1)/sqrt(512), "
                      "c[16,8192] N(0,1), out[16,512,8192] (BASELINE configs[3])",
-                     wall_ms, kernel_ms, ops, nbytes, "mfma_fp32", 157.3,
-                     {"parity_max_err_over_mean": err, "tolerance": 1e-4}, args)
+                     wall_ms, kernel_ms, ops, nbytes, "mfma", 2500.0,
+                     {"parity_max_err_over_mean": err, "tolerance": 1e-4,
+                      "route": "a and c split once into two fp16 pieces per value, sign of d - b on the pieces, v_mfma_f32_16x16x32_f16",
+                      "useful_tflops": round((2.0 * o + 3.0) * m_ref * n_ref * k_ref / kernel_ms / 1e9, 2),
+                      "fp32_kernels_same_run": {"ms": round(fp32_ms, 3), "parity_max_err_over_mean": fp32_err,
+                                                "frac_of_fp32_mfma_peak": round((2.0 * o + 3.0) * m_ref * n_ref * k_ref / fp32_ms / 1e9 / 157.3, 4)}},
+                     args)
 
 
 def bench_kernel_coef(kermac, device, args, steps=None, warmup=None, with_gaussian=True):

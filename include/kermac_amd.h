@@ -263,7 +263,7 @@ typedef struct kmc_norm_gradient_params {
 } kmc_norm_gradient_params;
 
 /* Bytes of workspace that kmc_norm_kernel_gradient would use for these parameters, 0 when it would
- * not use one (another norm than L1, fewer than 2e9 terms m * n * k * l).  About 1.1 times the
+ * not use one (another norm than L1, fewer than 3 outputs, fewer than 4e8 terms m * n * k * l).  About 1.1 times the
  * bytes of a, b and c.  No counterpart in the reference. */
 int kmc_norm_gradient_workspace_bytes(const kmc_norm_gradient_params *params, int64_t *bytes);
 

@@ -50,14 +50,19 @@ void place_rows(RowsRegions &r, int rows, int batches, const GradientLayout &lay
 }
 
 // The route pays where the fp32 kernels are bound by their matrix or vector instructions: enough
-// terms to fill the chip and to carry the five extra launches.  KERMAC_AMD_GRADIENT_F16_MIN_TERMS
-// replaces the threshold (read on every call, so that a test can send small shapes down the route).
+// terms to carry the five extra launches, and more than two outputs (its cost does not fall below
+// that of 16 outputs; the vector kernel for one or two is cheaper).  From a sweep, fp32 / fp16 time:
+// O = 16 at 3.4e10 terms 2.5, 1.1e9 1.5, 5.4e8 1.5, 2.7e8 1.1 .. 1.2, 1.3e8 0.86; at 3.4e10 terms
+// O = 1 0.73, O = 2 0.96, O = 4 1.34, O = 17 1.8, O = 64 2.6.  KERMAC_AMD_GRADIENT_F16_MIN_TERMS
+// replaces both conditions by a number of terms (read on every call, so that a test can send small
+// shapes down the route).
 bool f16_pays(const kmc_norm_gradient_params *p)
 {
     const char *text = std::getenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS");
     const double forced = text ? std::atof(text) : 0.0;
     const double terms = static_cast<double>(p->m) * p->n * p->k * p->l;
-    return terms >= (forced > 0.0 ? forced : 2e9);
+    if (forced > 0.0) return terms >= forced;
+    return p->o >= 3 && terms >= 4e8;
 }
 
 bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)

@@ -5,7 +5,7 @@ contraction on the fp16 matrix instruction.  Tolerance as for the other gradient
 result is a signed sum of K products, |got - truth| <= 1e-5 |truth| + 1e-4 mean |truth|.
 
 KERMAC_AMD_GRADIENT_F16_MIN_TERMS=1 sends the small shapes of these tests down the route, which by
-itself only takes problems of at least 2e9 terms.
+itself only takes problems of at least 4e8 terms and 3 outputs.
 """
 import importlib
 
@@ -60,7 +60,8 @@ def test_when_the_route_applies(device, monkeypatch):
     d = torch.empty(512, 4096, device=device)
     assert workspace_bytes(a, b, c, d) > 0                                   # 4.3e9 terms
     assert workspace_bytes(a, b, c, d, p=2.0) == 0 and workspace_bytes(a, b, c, d, p=1.3) == 0
-    assert workspace_bytes(a[:, :1024], b, c, d[:, :1024]) == 0              # 1.1e9 terms
+    assert workspace_bytes(a[:, :256], b[:64], c, d[:64, :256]) == 0         # 3.4e7 terms
+    assert workspace_bytes(a, b, c[:2], d) == 0                              # two outputs: the vector kernel
     needed = workspace_bytes(a, b, c, d)
     operands = 4 * (a.numel() + b.numel() + c.numel())
     assert operands <= needed <= 2 * operands
