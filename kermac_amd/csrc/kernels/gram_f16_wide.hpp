@@ -38,7 +38,10 @@
 // Workspace of one operand and batch entry, in 16-byte chunks of 8 fp16 (one row, one half of a
 // 16-deep K slice, one piece):  chunk[slice][piece][half][row 0 .. rows_pad),  rows_pad a multiple
 // of 256; rows that do not exist and k beyond K hold zeros, so the product kernel has no edge
-// handling in its walk.  Three slices more than K has are allocated and never multiplied.
+// handling in its walk.  Four slices more than K has are allocated and never multiplied.
+// Two compile-time switches leave a part of the product kernel out, for the measurements of what
+// bounds it (the results are then wrong): -DGW_ABLATE_NO_COPY issues no copies from the workspace,
+// -DGW_ABLATE_NO_EPILOGUE returns behind the walk.
 // Statistics: partial[range][row] for the sums of squares and for the magnitudes, one partial per
 // range of K slices that a workgroup walks, combined in the order of the ranges.
 // The reference has no such path (include/build_a_kernel.cuh:339-370 is SIMT only).
@@ -240,10 +243,10 @@ __device__ __forceinline__ bool wide_tile_of_workgroup(const GramWideArgs &args,
 // tiles of 32 x 32, 128 accumulator registers, 24 matrix instructions per slice.
 //
 // The pieces go from the workspace straight into LDS (global_load_lds_dwordx4: a wave copies 64
-// consecutive chunks, no registers involved), three slices in three buffers.  One barrier per
+// consecutive chunks, no registers involved), four slices in four buffers.  One barrier per
 // slice.  The operands of a slice are read into registers during the slice before it, so behind
-// the barrier of slice s the buffer of slice s is free and takes slice s + 3, and slice s + 1,
-// whose copies were issued two slices earlier, is complete and is read.
+// the barrier of slice s the buffer of slice s is free and takes slice s + 4, and slice s + 1,
+// whose copies were issued three slices earlier, is complete and is read.
 //
 // The copies are written as instructions: through the compiler's builtin every later LDS read
 // waits for every copy under way (the copies carry no information on which array they fill), which
@@ -383,7 +386,7 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
         multiply(set, 1, 0);                                // a2 b1
         copy(previous, GramStep<3>{});
         __builtin_amdgcn_sched_barrier(0);
-        // what may still be under way: the four copies issued last, of the slice after the next one
+        // what may still be under way: the eight copies issued last, of the two slices after the next one
         __builtin_amdgcn_s_waitcnt(0x0F78);                 // vmcnt(8), nothing else
         __syncthreads();
         read_operands(GramStep<1 - S>{}, next);
@@ -397,7 +400,7 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    // slices 0 and 1, and three of the four copies of slice 2
+    // slices 0, 1 and 2, and three of the four copies of slice 3
     copy(GramStep<0>{}, GramStep<0>{}); copy(GramStep<0>{}, GramStep<1>{}); copy(GramStep<0>{}, GramStep<2>{}); copy(GramStep<0>{}, GramStep<3>{});
     copy(GramStep<1>{}, GramStep<0>{}); copy(GramStep<1>{}, GramStep<1>{}); copy(GramStep<1>{}, GramStep<2>{}); copy(GramStep<1>{}, GramStep<3>{});
     copy(GramStep<2>{}, GramStep<0>{}); copy(GramStep<2>{}, GramStep<1>{}); copy(GramStep<2>{}, GramStep<2>{}); copy(GramStep<2>{}, GramStep<3>{});
@@ -420,9 +423,11 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
     __syncthreads();
 
 #ifdef GW_ABLATE_NO_EPILOGUE
-    if (args.slices > 0) {
+    if (args.slices > 0) {      // keeps the accumulators alive without storing them
         float sum = 0.0f;
-        for (int mt = 0; mt < 4; mt++) for (int nt = 0; nt < 2; nt++) for (int v = 0; v < 16; v++) sum += acc[mt][nt][v];
+        for (int mt = 0; mt < 4; mt++)
+            for (int nt = 0; nt < 2; nt++)
+                for (int v = 0; v < 16; v++) sum += acc[mt][nt][v];
         if (sum == 123.456f) args.kernel.c[tid] = sum;
         return;
     }
