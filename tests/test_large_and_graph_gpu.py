@@ -176,6 +176,61 @@ def test_operators_replay_from_a_hip_graph(device):
     assert_close_to_truth(out_p1.t(), truth, rtol=1e-5, what="graph replay vs oracle")
 
 
+def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
+    """The routes that go through a workspace allocated by the Python layer (squared differences on
+    the fp16 matrix instruction: centre, row statistics, split, product, repair; the L1 gradient on
+    the fp16 matrix instruction) captured into one graph: the workspace comes from the graph's memory
+    pool, the decision whether to subtract the centre is taken on the device, and every replay on
+    new values equals the eager result bit for bit."""
+    monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
+    monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
+    g = torch.Generator().manual_seed(77)
+    M, N, K, O = 600, 520, 96, 16
+    a_store = torch.randn(K, M, generator=g).to(device)
+    b_store = torch.randn(K, N, generator=g).to(device)
+    b_store[:, :100] = a_store[:, :100] + 1e-5 * torch.randn(K, 100, generator=g).to(device)      # twins: repaired parts
+    weights = torch.rand(N, M, generator=g).to(device)
+    centres = torch.randn(K, N, generator=g).to(device)
+    classes = torch.randn(O, N, generator=g).to(device)
+    samples = torch.randn(K, M, generator=g).to(device)
+    out_p2 = torch.empty(N, M, device=device)
+    out_self = torch.empty(M, M, device=device)
+    out_grad = torch.empty(O, K, M, device=device)
+
+    def run_all():
+        with kermac.l2_mode("gram_bf16", min_k=0):
+            kermac.cdist(a_store.t(), b_store.t(), p=2.0, out=out_p2.t())
+            kermac.cdist(a_store.t(), a_store.t(), p=2.0, out=out_self.t())
+        kermac.cdist_grad(weights, centres, classes, samples, out=out_grad, p=1.0)
+
+    outs = (out_p2, out_self, out_grad)
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run_all()                                               # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run_all()
+    for replay in range(4):
+        a_store.copy_(torch.randn(K, M, generator=g) + (3.0 if replay % 2 else 0.0))     # with and without a centre that matters
+        samples.mul_(1.25)
+        run_all()
+        torch.cuda.synchronize()
+        eager = [o.clone() for o in outs]
+        for o in outs:
+            o.fill_(float("nan"))
+        scratch = torch.randn(256, 256, device=device) @ torch.randn(256, 256, device=device)   # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        del scratch
+        for name, e, o in zip(("p2", "p2 self", "grad"), eager, outs):
+            assert torch.equal(e, o), f"replay {replay}: {name} differs from the eager result"
+    truth = oracle.cdist(a_store.t().cpu(), b_store.t().cpu(), p=2.0)[0]
+    assert_close_to_truth(out_p2.t(), truth, rtol=1e-5, atol=1e-30, what="graph replay vs oracle")
+
+
 def test_cut_launches_replay_from_a_hip_graph(device):
     """The calls that the Python layer cuts into a batched launch plus a sum of partial results
     (few rows against many centres; few results with a deep contraction) allocate a buffer and
