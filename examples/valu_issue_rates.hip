@@ -27,12 +27,13 @@
         } \
     } while (0)
 
-enum Case { P1_ROWS, P2_ROWS, POW_ROWS, PLAIN_ADD, ABS_ADD, EXP2, LOG2, CASES };
+enum Case { P1_ROWS, P2_ROWS, POW_ROWS, PLAIN_ADD, ABS_ADD, EXP2, LOG2, SAD_U32, CASES };
 static const char *case_names[CASES] = {
     "p = 1 rows: 8 v_sub + 8 v_add |x|", "p = 2 rows: 8 v_sub + 8 v_fmac", "p = 1.3 rows: sub, log2, mul, exp2, add",
-    "v_add_f32 (4-byte encoding)",        "v_add_f32 |x| (8-byte encoding)", "v_exp_f32", "v_log_f32"};
+    "v_add_f32 (4-byte encoding)",        "v_add_f32 |x| (8-byte encoding)", "v_exp_f32", "v_log_f32",
+    "v_sad_u32 (|a - b| + c on integers)"};
 // vector instructions per (m, n, k) of the case, and per 8 x 8 rank-1 update
-static const int per_term[CASES] = {2, 2, 5, 1, 1, 1, 1};
+static const int per_term[CASES] = {2, 2, 5, 1, 1, 1, 1, 1};
 
 template <int CASE>
 __global__ __launch_bounds__(1024) void issue(float *out, long long *clocks, int updates, float seed)
@@ -58,6 +59,7 @@ __global__ __launch_bounds__(1024) void issue(float *out, long long *clocks, int
                 if (CASE == ABS_ADD) asm volatile("v_add_f32 %0, |%1|, %0" : "+v"(acc[j][i]) : "v"(fa[i]));
                 if (CASE == EXP2) asm volatile("v_exp_f32 %0, %1" : "=v"(acc[j][i]) : "v"(fa[i]));
                 if (CASE == LOG2) asm volatile("v_log_f32 %0, %1" : "=v"(acc[j][i]) : "v"(fb[i]));
+                if (CASE == SAD_U32) asm volatile("v_sad_u32 %0, %1, %2, %0" : "+v"(acc[j][i]) : "v"(fa[i]), "v"(fb[j]));
             }
     }
     const long long wall1 = wall_clock64(), tick1 = clock64();
@@ -119,7 +121,8 @@ int main()
     for (int waves = 2; waves <= 4; waves++) {
         if (measure<P1_ROWS>(out, clocks, waves) || measure<P2_ROWS>(out, clocks, waves) ||
             measure<POW_ROWS>(out, clocks, waves) || measure<PLAIN_ADD>(out, clocks, waves) ||
-            measure<ABS_ADD>(out, clocks, waves) || measure<EXP2>(out, clocks, waves) || measure<LOG2>(out, clocks, waves))
+            measure<ABS_ADD>(out, clocks, waves) || measure<EXP2>(out, clocks, waves) || measure<LOG2>(out, clocks, waves) ||
+            measure<SAD_U32>(out, clocks, waves))
             return 1;
     }
     CHECK(hipFree(out));
