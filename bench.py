@@ -47,10 +47,11 @@ def measured_traffic():
         with open(TRAFFIC_PROFILE) as handle:
             for text in handle:
                 key, sep, value = text.partition("=")
-                if sep and key.strip() in ("traffic_bytes_per_launch", "measured_at_commit"):
+                if sep and key.strip() in ("traffic_bytes_per_launch", "measured_at_commit", "shader_clock_mhz"):
                     fields[key.strip()] = value.strip()
         return float(fields["traffic_bytes_per_launch"]), {
-            "file": "profiles/" + os.path.basename(TRAFFIC_PROFILE), "commit": fields.get("measured_at_commit")}
+            "file": "profiles/" + os.path.basename(TRAFFIC_PROFILE), "commit": fields.get("measured_at_commit"),
+            "shader_clock_mhz": float(fields["shader_clock_mhz"]) if "shader_clock_mhz" in fields else None}
     except (OSError, KeyError, ValueError):
         return None, None
 
@@ -496,6 +497,10 @@ def main():
             "counting": "3 fp32 ops per (m,n,k); the kernel issues 2 VALU instructions per (m,n,k), so its "
                         "instruction-issue ceiling is 1.5 x 78.6 = 117.9 TFLOP/s in this unit at 2.4 GHz",
             "frac_of_issue_ceiling": round(achieved / 117.9, 4),
+            "clock": {"nominal_mhz_in_peak": 2400,
+                      "shader_mhz_under_this_kernel": (traffic_source or {}).get("shader_clock_mhz"),
+                      "how": "GRBM_GUI_ACTIVE / kernel duration in the profile named by traffic_source; "
+                             "the board sustains less than the nominal clock under this load"},
             "hbm_gbps": round(ALGORITHMIC_BYTES / kernel_ms / 1e6, 1),
             "hbm_frac": round(ALGORITHMIC_BYTES / kernel_ms / 1e6 / PEAK_HBM_GBPS, 4),
         },
