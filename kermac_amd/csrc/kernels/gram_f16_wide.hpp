@@ -165,9 +165,9 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsA
     const float *centre = gram_rows_centre(args, batch);
 
     // scale = 2^(GW_SCALE_EXPONENT - floor(log2 magnitude)), from the exponent field.  Rows of
-    // zeros or of values below 2^-97 take the largest scale used (their squares underflow in
-    // every path); a row with a NaN or an infinity takes the smallest: its products are not
-    // numbers whatever the scale, and the epilogue distrusts them.
+    // zeros or of values below 2^-111 take the largest scale used, 2^125 (the scale and its
+    // inverse must both be normal numbers); a row with a NaN or an infinity takes the smallest:
+    // its products are not numbers whatever the scale.
     float magnitude = 0.0f;
     for (int r = 0; r < args.ranges; r++) {
         const float part = args.magnitudes[batch * args.stats_bs + (i64)r * args.rows_pad + row];
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsA
         if (part != part) break;
     }
     int exponent_field = (__float_as_uint(magnitude) >> 23) & 0xff;
-    exponent_field = max(exponent_field, 30);
+    exponent_field = max(exponent_field, 16);
     const float scale = __uint_as_float((unsigned)(127 + GW_SCALE_EXPONENT + 127 - exponent_field) << 23);
     if (range == 0)
         args.unscale[batch * args.unscale_bs + row] = __uint_as_float((unsigned)(exponent_field - GW_SCALE_EXPONENT) << 23);

@@ -73,6 +73,8 @@ def test_signs_at_zero_and_rows_of_different_magnitude(device, f16_route):
     g = torch.Generator().manual_seed(5)
     M, N, O, K = 150, 40, 16, 96
     a = torch.randn(K, M, generator=g) * torch.pow(2.0, (torch.arange(M) % 31 - 15).float())[None, :]
+    a[:, 0] *= 2.0 ** -100                 # rows far out: the scale is a power of two per row
+    a[:, 1] *= 2.0 ** 100
     c = torch.randn(O, K, generator=g) * torch.pow(2.0, (torch.arange(O) % 9 - 4).float())[:, None]
     b = torch.randn(N, K, generator=g)
     d = torch.randn(N, M, generator=g)
