@@ -18,6 +18,19 @@ from tests.helpers import assert_close_to_truth
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(autouse=True, params=["as launched", "workspace routes"])
+def routes(request, monkeypatch):
+    """Every sweep twice: as the library launches these small shapes by itself, and with the routes
+    that go through a workspace forced onto them (squared differences and the L1 gradient on the
+    fp16 matrix instruction, which by themselves only take large problems)."""
+    if request.param == "workspace routes":
+        monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
+        monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
+        kermac.set_l2_mode("gram_bf16", min_k=0)
+    yield
+    kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
+
 POWERS = {"NOOP": kermac.PowerType.NOOP, "ABS": kermac.PowerType.ABS, "SQUARE": kermac.PowerType.SQUARE,
           "SQRT": kermac.PowerType.SQRT, "POW": kermac.PowerType.POW}
 KERNELS = {"NONE": kermac.KernelType.NONE, "LAPLACE": kermac.KernelType.LAPLACE, "GAUSSIAN": kermac.KernelType.GAUSSIAN}
