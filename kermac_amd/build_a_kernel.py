@@ -576,7 +576,10 @@ def _attach_gram_workspace(params, device):
     needed = _backend.gram_workspace_bytes(params)
     if needed == 0:
         return None
-    workspace = torch.empty(needed, dtype=torch.uint8, device=device)
+    try:
+        workspace = torch.empty(needed, dtype=torch.uint8, device=device)
+    except torch.cuda.OutOfMemoryError:
+        return None             # no room for it: the one-step kernel needs none
     params.gram_workspace, params.gram_workspace_bytes = workspace.data_ptr(), needed
     return workspace
 

@@ -179,7 +179,10 @@ def _attach_workspace(params, device):
     needed = _backend.norm_gradient_workspace_bytes(params)
     if needed == 0:
         return None
-    workspace = torch.empty(needed, dtype=torch.uint8, device=device)
+    try:
+        workspace = torch.empty(needed, dtype=torch.uint8, device=device)
+    except torch.cuda.OutOfMemoryError:
+        return None             # no room for it: the fp32 kernels need none
     params.workspace, params.workspace_bytes = workspace.data_ptr(), needed
     return workspace
 
