@@ -177,11 +177,15 @@ int kmc_build_kernel_load_modes(const kmc_build_kernel_params *params, int32_t *
 int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes)
 {
     if (!bytes) return fail(KMC_ERR_INVALID_ARGUMENT, "bytes: null pointer");
+    if (!params) return fail(KMC_ERR_INVALID_ARGUMENT, "null parameter block");
+    // the result may not be allocated yet when the caller asks: any address stands in for it
+    kmc_build_kernel_params asked = *params;
+    if (!asked.c) asked.c = reinterpret_cast<float *>(static_cast<uintptr_t>(256));
     kmc::BuildKernelArgs args;
     int load_a = 0, load_b = 0;
-    int status = prepare(params, true, &args, &load_a, &load_b);
+    int status = prepare(&asked, true, &args, &load_a, &load_b);
     if (status != KMC_OK) return status;
-    *bytes = gram_f16_wide_bytes(params, args);
+    *bytes = gram_f16_wide_bytes(&asked, args);
     return KMC_OK;
 }
 

@@ -455,6 +455,52 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert isinstance(info.value, _backend.BackendError) and info.value.status == _backend.ERR_WRONG_DEVICE
 
 
+def test_workspace_queries_need_no_gpu(monkeypatch):
+    """kmc_gram_workspace_bytes and kmc_norm_gradient_workspace_bytes decide from the parameter block
+    alone (no device call, no pointer dereferenced, the result need not be allocated yet): which
+    problems take the routes through a workspace, and how much they want."""
+    monkeypatch.delenv("KERMAC_AMD_WIDE_MIN_TILES", raising=False)
+    monkeypatch.delenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", raising=False)
+    fake = 4096
+
+    def squared_differences(m, n, k, l=1, flags=_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16, same=False):
+        params = _backend.BuildKernelParams()
+        params.inner_operator, params.inner_power, params.outer_power = 0, 2, 3      # DIFF, SQUARE, SQRT
+        params.m, params.n, params.k, params.l = m, n, k, l
+        params.a, params.a_ld, params.a_bs = fake, m, m * k
+        params.b, params.b_ld, params.b_bs = (fake if same else fake + 4 * m * k * l), n, n * k
+        params.c_ld, params.c_bs = m, m * n                                          # c stays null: not allocated yet
+        params.flags = flags
+        return _backend.gram_workspace_bytes(params)
+
+    full = squared_differences(8192, 8192, 512)
+    operands = 2 * 8192 * 512 * 4
+    assert operands < full < 1.3 * operands                                          # two fp16 pieces per value, padding, statistics
+    assert squared_differences(8192, 8192, 512, flags=_backend.FLAG_L2_GRAM) == 0    # fp32 matrix instruction: one step
+    assert squared_differences(8192, 8192, 32) == 0                                  # k < 64
+    assert squared_differences(2048, 2048, 512) == 0                                 # 64 tiles
+    assert squared_differences(2048, 2048, 512, l=5) > 0                             # 320 tiles over the batch
+    assert 0 < squared_differences(8192, 8192, 512, same=True) < 0.6 * full          # a panel against itself: split once
+    assert squared_differences(0, 8192, 512) == 0
+    monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
+    assert squared_differences(300, 200, 5) > 0
+
+    def gradient(m, n, o, k, norm_type=0):
+        grad = _backend.NormGradientParams()
+        grad.norm_type = norm_type
+        grad.m, grad.n, grad.o, grad.k, grad.l = m, n, o, k, 1
+        grad.a, grad.b, grad.c, grad.d, grad.e = fake, fake, fake, fake, fake
+        grad.a_ld, grad.b_ld, grad.c_ld, grad.d_ld, grad.e_ld_n, grad.e_ld_o = m, k, k, m, m, m * n
+        return _backend.norm_gradient_workspace_bytes(grad)
+
+    assert gradient(8192, 512, 16, 8192) > 4 * 8192 * 8192                           # the pieces of a alone
+    assert gradient(8192, 512, 16, 8192, norm_type=1) == 0 and gradient(8192, 512, 16, 8192, norm_type=2) == 0
+    assert gradient(8192, 512, 2, 8192) == 0                                         # two outputs: the vector kernel
+    assert gradient(1024, 64, 16, 1024) == 0                                         # 6.7e7 terms
+    monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
+    assert gradient(3, 2, 1, 5) > 0
+
+
 def test_launch_cuts_follow_the_shape_and_the_environment_switch(monkeypatch):
     """The cut over k is decided from the parameter block alone: small and middling results over a
     long contraction are cut, batches, short contractions and large results are not, and
