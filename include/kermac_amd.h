@@ -168,8 +168,9 @@ typedef struct kmc_build_kernel_params {
 
 /* Bytes of gram_workspace that kmc_build_kernel would use for these parameters, 0 when it would
  * not use one (no KMC_FLAG_L2_GRAM_BF16, or a problem too small to gain: fewer than 128 tiles of
- * 256 x 256 over the batch, k < 64, or tiles * k below 147456; of a panel against itself the tiles
- * on and below the diagonal count, and the panel is split once).  About 1.1 times the bytes of the
+ * 256 x 256 over the batch, k < 64, tiles * k below 147456, fewer tiles within a batch entry than
+ * tiles_m * tiles_n >= 2.5 * (tiles_m + tiles_n), or more than 20 % of the tiles' area padding; of
+ * a panel against itself the tiles on and below the diagonal count, and the panel is split once).  About 1.1 times the bytes of the
  * operands.  No counterpart in the reference. */
 int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes);
 
@@ -263,7 +264,8 @@ typedef struct kmc_norm_gradient_params {
 } kmc_norm_gradient_params;
 
 /* Bytes of workspace that kmc_norm_kernel_gradient would use for these parameters, 0 when it would
- * not use one (another norm than L1, fewer than 3 outputs, fewer than 4e8 terms m * n * k * l).  About 1.1 times the
+ * not use one (another norm than L1, fewer than 3 outputs, n < 24, or fewer terms m * n * k * l
+ * than 6.4e9 / min(o, 16): 4e8 at 16 outputs).  About 1.1 times the
  * bytes of a, b and c.  No counterpart in the reference. */
 int kmc_norm_gradient_workspace_bytes(const kmc_norm_gradient_params *params, int64_t *bytes);
 

@@ -32,16 +32,25 @@ struct WideLayout {
 
 // Whether the route pays for its extra launches and its coarser tiles (a CU holds one workgroup of
 // 256 x 256, so a few hundred tiles do not fill the chip as evenly as four times as many of
-// 128 x 128).  From a sweep against the one-step kernel, wide / one-step time: K = 1024 0.92 at 144
-// tiles, 0.76 at 256, 0.63 from 1024 on; K = 256 1.01 at 576, 0.87 at 1024, 0.80 at 4096; K = 64 1.0
-// at 1024, 0.9 from 2304 on; K = 32 never below 1.  KERMAC_AMD_WIDE_MIN_TILES = t replaces the rule
-// by "at least t tiles" (read on every call, so that a test can send small shapes down the route).
-bool wide_pays(int64_t tiles, int k)
+// 128 x 128).  From sweeps against the one-step kernel, one-step / wide time:
+//   * over all tiles of the batch: K = 1024 1.09 at 144 tiles, 1.3 at 256, 1.6 from 1024 on; K = 256 0.99
+//     at 576, 1.15 at 1024, 1.25 at 4096; K = 64 1.0 at 1024, 1.07 from 2304 on; K = 32 never above 1;
+//   * the split of the operands is paid once per row and earned back once per tile the row meets, so
+//     each batch entry needs tiles in both directions: at K = 1024, 64 entries of 2 x 2 tiles 0.74,
+//     of 4 x 4 1.03, of 8 x 8 1.25, of 16 x 16 1.46; 118 x 4 tiles 1.26, 118 x 2 0.83, 391 x 2 0.84.
+//     The rule asks tiles_m * tiles_n / (tiles_m + tiles_n) >= 2.5 (5 x 5, or 4 x 7, or 3 x 15);
+//   * rows that pad the last tile are computed and thrown away: 8 entries of 1280 x 1280 1.24, of
+//     1290 x 1290 (6 x 6 tiles, 30 % padding) 0.86.  The rule asks for at most 20 % padding.
+// KERMAC_AMD_WIDE_MIN_TILES = t replaces the rule by "at least t tiles" (read on every call, so that
+// a test can send small shapes down the route).
+bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t tiles, int k)
 {
     const char *text = std::getenv("KERMAC_AMD_WIDE_MIN_TILES");
     const int forced = text ? std::atoi(text) : 0;
     if (forced > 0) return tiles >= forced && k >= 1;
-    return k >= 64 && tiles >= 128 && tiles * k >= 147456;
+    if (k < 64 || tiles < 128 || tiles * k < 147456) return false;
+    if (2 * tiles_m * tiles_n < 5 * (tiles_m + tiles_n)) return false;
+    return 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
 }
 
 int64_t place(int64_t &cursor, int64_t bytes)
@@ -73,7 +82,7 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
     // a panel against itself: the tiles on and below the diagonal
     const int64_t tiles = args.symmetric ? static_cast<int64_t>(layout->tiles_m) * (layout->tiles_m + 1) / 2
                                          : static_cast<int64_t>(layout->tiles_m) * layout->tiles_n;
-    if (!wide_pays(tiles * args.l, args.k)) return false;
+    if (!wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k)) return false;
     int padded = (layout->tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
     if ((padded - layout->tiles_n) * 8 > layout->tiles_n) padded = layout->tiles_n;
     if (static_cast<int64_t>(layout->tiles_m) * padded > 0x7fffffff) return false;

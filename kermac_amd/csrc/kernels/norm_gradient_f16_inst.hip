@@ -51,18 +51,21 @@ void place_rows(RowsRegions &r, int rows, int batches, const GradientLayout &lay
 
 // The route pays where the fp32 kernels are bound by their matrix or vector instructions: enough
 // terms to carry the five extra launches, and more than two outputs (its cost does not fall below
-// that of 16 outputs; the vector kernel for one or two is cheaper).  From a sweep, fp32 / fp16 time:
-// O = 16 at 3.4e10 terms 2.5, 1.1e9 1.5, 5.4e8 1.5, 2.7e8 1.1 .. 1.2, 1.3e8 0.86; at 3.4e10 terms
-// O = 1 0.73, O = 2 0.96, O = 4 1.34, O = 17 1.8, O = 64 2.6.  KERMAC_AMD_GRADIENT_F16_MIN_TERMS
-// replaces both conditions by a number of terms (read on every call, so that a test can send small
-// shapes down the route).
+// that of 16 outputs; the vector kernel for one or two is cheaper).  From sweeps, fp32 / fp16 time:
+// O = 16 at 3.4e10 terms 2.5, 1.1e9 1.8, 5.4e8 1.1 .. 1.4, 2.7e8 0.8 .. 1.1, 1.3e8 0.66; at 3.4e10
+// terms O = 1 0.73, O = 2 0.93, O = 3 1.21, O = 4 1.31, O = 8 2.1, O = 17 1.7, O = 48 2.6; with few
+// outputs the fp32 kernels are cheaper by nearly that factor and the route is not (16 results per
+// tile whatever O), so the terms are asked for in proportion: 4e8 at 16 outputs, 1.6e9 at 4.  Its
+// tiles hold 32 columns of the result: N = 8 0.90, N = 16 0.86, N = 32 1.37, N = 33 1.49.
+// KERMAC_AMD_GRADIENT_F16_MIN_TERMS replaces the conditions by a number of terms (read on every
+// call, so that a test can send small shapes down the route).
 bool f16_pays(const kmc_norm_gradient_params *p)
 {
     const char *text = std::getenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS");
     const double forced = text ? std::atof(text) : 0.0;
     const double terms = static_cast<double>(p->m) * p->n * p->k * p->l;
     if (forced > 0.0) return terms >= forced;
-    return p->o >= 3 && terms >= 4e8;
+    return p->o >= 3 && p->n >= 24 && terms * (p->o < 16 ? p->o : 16) >= 6.4e9;
 }
 
 bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)

@@ -481,6 +481,10 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert squared_differences(2048, 2048, 512) == 0                                 # 64 tiles
     assert squared_differences(2048, 2048, 512, l=5) > 0                             # 320 tiles over the batch
     assert 0 < squared_differences(8192, 8192, 512, same=True) < 0.6 * full          # a panel against itself: split once
+    assert squared_differences(512, 512, 1024, l=64) == 0                            # 256 tiles, but 2 x 2 per entry: the split is not earned back
+    assert squared_differences(30000, 512, 1024) == 0 and squared_differences(30000, 1024, 1024) > 0
+    assert squared_differences(1290, 1290, 1024, l=8) == 0                           # 6 x 6 tiles, 30 % of them padding
+    assert squared_differences(1280, 1280, 1024, l=8) > 0
     assert squared_differences(0, 8192, 512) == 0
     monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
     assert squared_differences(300, 200, 5) > 0
@@ -497,6 +501,8 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert gradient(8192, 512, 16, 8192, norm_type=1) == 0 and gradient(8192, 512, 16, 8192, norm_type=2) == 0
     assert gradient(8192, 512, 2, 8192) == 0                                         # two outputs: the vector kernel
     assert gradient(1024, 64, 16, 1024) == 0                                         # 6.7e7 terms
+    assert gradient(8192, 16, 16, 8192) == 0                                         # half of every tile of 32 columns unused
+    assert gradient(2048, 128, 4, 2048) == 0 and gradient(2048, 128, 16, 2048) > 0   # 5.4e8 terms: enough for 16 outputs, not for 4
     monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
     assert gradient(3, 2, 1, 5) > 0
 
