@@ -96,7 +96,14 @@ enum kmc_flags {
      * that is symmetric in a and b, so C(m,n) and C(n,m) of an x-against-x matrix agree
      * to rounding only, unless the symmetric shortcut (see KMC_FLAG_NO_SYMMETRY) mirrors
      * them.  kmc_kernel_times_coefficients does not look at this flag. */
-    KMC_FLAG_L2_GRAM_BF16 = 32
+    KMC_FLAG_L2_GRAM_BF16 = 32,
+    /* With gram_workspace only (ignored by every launch that does not go through it): the
+     * workspace still holds the split of `a` that the previous kmc_build_kernel call through this
+     * workspace made, for the same a, a_ld, a_bs, a_majorness, m, k, l and gram_centre and with
+     * `a` unchanged since; it is not made again.  For callers that build the matrix panel by panel
+     * of `b` (the split of `a` is a quarter of the cost of a panel of 2048 rows of b).  Anything
+     * else in those fields of the previous call gives a wrong result, not an error. */
+    KMC_FLAG_GRAM_A_KEPT = 64
 };
 
 /*
@@ -311,6 +318,34 @@ int kmc_kernel_times_coefficients(const kmc_kernel_coefficients_params *params, 
 int kmc_kernel_times_coefficients_has_variant(int32_t inner_operator, int32_t inner_power);
 /* Launch a run-time compiled kmc::kernel_times_coefficients instantiation. */
 int kmc_kernel_times_coefficients_jit(void *function, const kmc_kernel_coefficients_params *params, void *stream);
+
+/*
+ * A stored panel of the kernel matrix times coefficients:
+ *   out[m*out_ld + o + l*out_bs] (+)= sum_n matrix[n*matrix_ld + m + l*matrix_bs] * coef[n*coef_ld + o + l*coef_bs]
+ * The second half of the kernel matrix x coefficients product when the matrix is built in panels
+ * of centres by kmc_build_kernel (c_ld = matrix_ld, m contiguous) instead of inside the fused
+ * kernel: for squared differences the matrix-core routes of kmc_build_kernel build a panel
+ * several times faster than kmc_kernel_times_coefficients walks it.  The sums run in a fixed
+ * order: the same inputs give the same bits.  n = 0 without accumulate stores zeros.  The
+ * reference has no such kernel (its run_kernel stops at the stored matrix out[L,M,N],
+ * src/kermac/build_a_kernel.py:259,378-392); no library routine and no allocation here.
+ */
+typedef struct kmc_matrix_coefficients_params {
+    int32_t m, n, o, l;
+    const float *matrix; int64_t matrix_ld; int64_t matrix_bs;  /* [n, m], m contiguous */
+    const float *coef; int64_t coef_ld; int64_t coef_bs;        /* [n, o], o contiguous */
+    float *out; int64_t out_ld; int64_t out_bs;                 /* [m, o], o contiguous */
+    int32_t accumulate;                                         /* 0: out = product, 1: out += product */
+    /* 0 or 1: one product.  S > 1: the n rows are cut into S consecutive ranges, each walked by
+     * workgroups of its own into a partial product of its own,
+     *   out[m*out_ld + o + l*out_bs + s*out_split_stride],
+     * and the caller adds the S partial products in a fixed order (as with n_ranges of
+     * kmc_kernel_coefficients_params): a workgroup owns 512 rows m, so few rows against a long
+     * panel leave the chip under-used unless the n are cut.  l * S may not exceed 65535. */
+    int32_t n_splits;
+    int64_t out_split_stride;
+} kmc_matrix_coefficients_params;
+int kmc_matrix_times_coefficients(const kmc_matrix_coefficients_params *params, void *stream);
 
 /* ---- run-time compilation (stands in for cuda.core Program / ObjectCode:
  *      src/kermac/module_cache/module_cache.py:13-51, 219-239) ---- */

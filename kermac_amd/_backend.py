@@ -35,6 +35,7 @@ FLAG_L2_GRAM = 4
 FLAG_GENERIC_POWER = 8
 FLAG_NO_SYMMETRY = 16
 FLAG_L2_GRAM_BF16 = 32
+FLAG_GRAM_A_KEPT = 64
 
 _float_p = c_void_p  # device pointers are passed as integers
 
@@ -87,6 +88,18 @@ class KernelCoefficientsParams(Structure):
     ]
 
 
+class MatrixCoefficientsParams(Structure):
+    """struct kmc_matrix_coefficients_params"""
+    _fields_ = [
+        ("m", c_int32), ("n", c_int32), ("o", c_int32), ("l", c_int32),
+        ("matrix", _float_p), ("matrix_ld", c_int64), ("matrix_bs", c_int64),
+        ("coef", _float_p), ("coef_ld", c_int64), ("coef_bs", c_int64),
+        ("out", _float_p), ("out_ld", c_int64), ("out_bs", c_int64),
+        ("accumulate", c_int32),
+        ("n_splits", c_int32), ("out_split_stride", c_int64),
+    ]
+
+
 # Every exported symbol of include/kermac_amd.h: name -> (restype, argtypes).
 SIGNATURES = {
     "kmc_abi_version": (ctypes.c_int, []),
@@ -105,6 +118,7 @@ SIGNATURES = {
     "kmc_norm_kernel_gradient": (ctypes.c_int, [POINTER(NormGradientParams), c_void_p]),
     "kmc_norm_gradient_workspace_bytes": (ctypes.c_int, [POINTER(NormGradientParams), POINTER(c_int64)]),
     "kmc_kernel_times_coefficients": (ctypes.c_int, [POINTER(KernelCoefficientsParams), c_void_p]),
+    "kmc_matrix_times_coefficients": (ctypes.c_int, [POINTER(MatrixCoefficientsParams), c_void_p]),
     "kmc_kernel_times_coefficients_has_variant": (ctypes.c_int, [c_int32, c_int32]),
     "kmc_kernel_times_coefficients_jit": (ctypes.c_int, [c_void_p, POINTER(KernelCoefficientsParams), c_void_p]),
     "kmc_jit_compile": (ctypes.c_int, [
@@ -237,6 +251,10 @@ def kernel_times_coefficients(params: KernelCoefficientsParams, stream: int) -> 
 
 def kernel_times_coefficients_jit(function: int, params: KernelCoefficientsParams, stream: int) -> None:
     check(library().kmc_kernel_times_coefficients_jit(c_void_p(function), byref(params), c_void_p(stream)))
+
+
+def matrix_times_coefficients(params: MatrixCoefficientsParams, stream: int) -> None:
+    check(library().kmc_matrix_times_coefficients(byref(params), c_void_p(stream)))
 
 
 def kernel_times_coefficients_has_variant(inner_operator: int, inner_power: int) -> bool:

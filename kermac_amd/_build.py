@@ -54,7 +54,8 @@ HOST_SOURCES = [
 EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_inst.hip",
                         "kernels/gram_coefficients_inst.hip", "kernels/gram_bf16_kernel_inst.hip",
                         "kernels/finish_partials.hip", "kernels/cut_static_scratch.hip", "kernels/sample_mean.hip",
-                        "kernels/gram_f16_wide_inst.hip", "kernels/norm_gradient_f16_inst.hip"]
+                        "kernels/gram_f16_wide_inst.hip", "kernels/norm_gradient_f16_inst.hip",
+                        "kernels/matrix_times_coefficients.hip"]
 
 
 def _hipcc() -> str:

@@ -151,7 +151,8 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     const bool scalar_only = (p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) != 0;
     const kmc::GramRowsArgs rows_a = rows_args(args.a, args.a_ld, args.a_bs, args.m, p->a_majorness, scalar_only, args, layout, layout.a, workspace);
     const kmc::GramRowsArgs rows_b = rows_args(args.b, args.b_ld, args.b_bs, args.n, p->b_majorness, scalar_only, args, layout, layout.b, workspace);
-    hipError_t status = launch_gram_rows(rows_a, layout.a.batches, stream);
+    // the region of a lies first in the workspace and its size does not depend on b
+    hipError_t status = (p->flags & KMC_FLAG_GRAM_A_KEPT) ? hipSuccess : launch_gram_rows(rows_a, layout.a.batches, stream);
     if (status != hipSuccess) return status;
     if (!args.symmetric) {
         status = launch_gram_rows(rows_b, layout.b.batches, stream);

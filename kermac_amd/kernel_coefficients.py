@@ -118,6 +118,8 @@ def run_kernel_coefficients(
     if matrix_core:
         from .build_a_kernel import _attach_gram_centre
         plan.keepalive.append(_attach_gram_centre(kernel, stream, a.device))
+        if aot and _run_in_panels(plan, stream, a.device, debug):
+            return plan.out
     ranges = _centre_ranges(plan, three_resident=aot and not matrix_core and plan.O <= 32)
     partial = None
     if ranges > 1:
@@ -138,14 +140,108 @@ def run_kernel_coefficients(
             print(f"(Kermac Debug) Launching kernel: {name}")
         _backend.kernel_times_coefficients_jit(function, params, stream)
     if partial is not None:
-        target = plan.out if plan.out.dim() == 3 else plan.out.unsqueeze(0)
-        if target.is_contiguous():
-            torch.sum(partial, dim=0, out=target)
-        else:
-            # the order in which torch adds the ranges depends on the layout of the result: a strided
-            # `out` gets the bits of a contiguous one
-            target.copy_(torch.sum(partial, dim=0))
+        _sum_partials(partial, plan.out)
     return plan.out
+
+
+# Squared differences on the matrix cores: the route of kmc_build_kernel through a workspace
+# (operands split once into fp16 pieces, 256 x 256 tiles) builds the kernel matrix several times
+# faster than the fused kernel walks it, so a large product is taken panel by panel instead: the
+# kernel matrix of all rows against a few thousand centres is written into a buffer that is
+# reused, and kmc_matrix_times_coefficients contracts it with the coefficients of those centres.
+# The full matrix never exists; the panel (1 GiB unless KERMAC_AMD_COEFFICIENT_PANEL_BYTES says
+# otherwise, 0 switches the route off) does.  Measured, fused kernel -> panels: L = 4,
+# M = N = 16384, O = 32 at K = 256 7.5 -> 4.9 ms, at K = 1024 22.4 -> 8.9 ms; M = N = 30000,
+# K = 1024, O = 16 18.5 -> 8.4 ms.  The partial products of the panels (and of the ranges a panel
+# is cut into when the rows alone do not fill the chip) are added in a fixed order.
+_PANEL_BYTES = 1 << 30
+_PANEL_MAX_PARTIAL_BYTES = 512 << 20
+
+
+def _panel_splits(M, O, L, rows):
+    """Ranges of centres per panel for kmc_matrix_times_coefficients: a workgroup per CU, and sums
+    of at most 4096 rows per workgroup."""
+    workgroups = -(-M // 128) * -(-O // 32) * L
+    splits = 1 if workgroups >= 256 else min(-(-256 // workgroups), max(1, rows // 512))
+    return min(max(splits, -(-rows // 4096)), max(1, 65535 // L))
+
+
+def _run_in_panels(plan, stream, device, debug):
+    """The product panel by panel (above); False when this problem stays with the fused kernel."""
+    import os
+
+    from .build_a_kernel import _attach_gram_workspace, _l2_current
+
+    budget = int(os.environ.get("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", _PANEL_BYTES))
+    L, M, N, O = plan.L, plan.M, plan.N, plan.O
+    # l2 mode "gram" asks for the fp32 matrix instruction; the panels are built from fp16 pieces
+    if budget <= 0 or 0 in (L, M, N, O, plan.K) or _l2_current()["mode"] not in ("auto", "gram_bf16"):
+        return False
+    ld = -(-M // 4) * 4                                          # rows of the panel start on 16 bytes
+    rows = min(N, max(256, budget // (4 * L * ld) // 256 * 256))
+    panels = -(-N // rows)
+    rows = min(N, -(-(-(-N // panels)) // 256) * 256)             # panels of equal size, whole tiles
+    panels = -(-N // rows)
+    params = plan.params
+    block = _backend.BuildKernelParams.from_buffer_copy(params.kernel)
+    block.flags |= _backend.FLAG_L2_GRAM_BF16
+    block.n, block.c, block.c_ld, block.c_bs = rows, 256, ld, rows * ld      # c: any address, for the query
+    if _backend.gram_workspace_bytes(block) == 0:
+        return False                                             # panels of this shape would not take the fast route
+    splits = _panel_splits(M, O, L, rows)
+    parts = panels * splits
+    if parts > 1 and 4 * parts * L * M * O > _PANEL_MAX_PARTIAL_BYTES:
+        return False
+    try:
+        panel = torch.empty(L * rows * ld, dtype=torch.float32, device=device)
+        partial = torch.empty((parts, L, M, O), dtype=torch.float32, device=device) if parts > 1 else None
+    except torch.cuda.OutOfMemoryError:
+        return False
+    block.c = panel.data_ptr()
+    workspace = _attach_gram_workspace(block, device)
+    if workspace is None:
+        return False
+    if debug:
+        print(f"(Kermac Debug) Kernel matrix x coefficients in {panels} panels of {rows} centres, "
+              f"{splits} partial products each")
+    row_major_b = block.b_majorness == _backend.ROW_MAJOR
+    contraction = _backend.MatrixCoefficientsParams()
+    contraction.m, contraction.o, contraction.l = M, O, L
+    contraction.matrix, contraction.matrix_ld = panel.data_ptr(), ld
+    contraction.coef_ld, contraction.coef_bs = params.coef_ld, params.coef_bs
+    if partial is None:
+        contraction.out, contraction.out_ld, contraction.out_bs = params.out, params.out_ld, params.out_bs
+    else:
+        contraction.out_ld, contraction.out_bs = O, M * O
+        contraction.n_splits, contraction.out_split_stride = splits, L * M * O
+    first_b, first_offset = params.kernel.b, params.kernel.regularization_offset_y
+    for index in range(panels):
+        n0 = index * rows
+        count = min(rows, N - n0)
+        block.n, block.c_bs = count, count * ld
+        block.b = first_b + 4 * n0 * (block.b_ld if row_major_b else 1)
+        block.regularization_offset_y = first_offset + n0
+        _backend.build_kernel(block, stream)
+        block.flags |= _backend.FLAG_GRAM_A_KEPT                 # the rows are the same for every panel: split once
+        contraction.n, contraction.matrix_bs = count, count * ld
+        contraction.coef = params.coef + 4 * n0 * params.coef_ld
+        if partial is not None:
+            contraction.out = partial.data_ptr() + 4 * index * splits * L * M * O
+        _backend.matrix_times_coefficients(contraction, stream)
+    if partial is not None:
+        _sum_partials(partial, plan.out)
+    plan.keepalive += [panel, partial, workspace]
+    return True
+
+
+def _sum_partials(partial, out):
+    target = out if out.dim() == 3 else out.unsqueeze(0)
+    if target.is_contiguous():
+        torch.sum(partial, dim=0, out=target)
+    else:
+        # the order in which torch adds the ranges depends on the layout of the result: a strided
+        # `out` gets the bits of a contiguous one
+        target.copy_(torch.sum(partial, dim=0))
 
 
 # A workgroup of the fused kernel owns 128 rows of ``a`` (one batch entry, one chunk of up to 64

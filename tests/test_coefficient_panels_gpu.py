@@ -1,0 +1,203 @@
+"""GPU tests of the kernel matrix x coefficients product taken panel by panel: for squared
+differences in the l2 modes "auto" and "gram_bf16", ``run_kernel(..., coefficients=...)`` builds the
+kernel matrix of all rows against a few thousand centres at a time with kmc_build_kernel's
+workspace route and contracts each panel with kmc_matrix_times_coefficients.  Same stated
+tolerance as the fused kernel: rtol 1e-5 against the float64 oracle with an absolute floor
+proportional to the typical magnitude of the signed sum over n.
+
+KERMAC_AMD_WIDE_MIN_TILES=1 and a small KERMAC_AMD_COEFFICIENT_PANEL_BYTES send the small shapes of
+these tests down the route, in several panels.
+"""
+import pytest
+import torch
+
+import kermac_amd as kermac
+from kermac_amd import _backend
+from oracle import oracle
+from tests.helpers import assert_close_to_truth, make_operand
+
+pytestmark = pytest.mark.gpu
+
+GAUSSIAN = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP,
+                                   kermac.KernelType.GAUSSIAN)
+CASES = (
+    (kermac.kernel_descriptor_laplace_l2, ("DIFF", "SQUARE", "SQRT", "LAPLACE"), {"bandwidth": 6.0}),
+    (GAUSSIAN, ("DIFF", "SQUARE", "NOOP", "GAUSSIAN"), {"bandwidth": 5.0}),
+    (kermac.kernel_descriptor_l2_norm, ("DIFF", "SQUARE", "SQRT", "NONE"), {}),
+)
+PANELS = "(Kermac Debug) Kernel matrix x coefficients in"
+
+
+@pytest.fixture
+def panels(monkeypatch):
+    monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "4096")      # the smallest panels: 256 centres
+    kermac.set_l2_mode("gram_bf16", min_k=0)
+    yield
+    kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
+
+
+def atol_for(truth, rtol):
+    return rtol * float(truth.abs().mean()) * 10
+
+
+def contraction(matrix, coef, out, accumulate=0, splits=1):
+    """kmc_matrix_times_coefficients on matrix [L, N, M] (m contiguous), coef [L, N, O], out [S?, L, M, O]."""
+    L, N, M = matrix.shape
+    params = _backend.MatrixCoefficientsParams()
+    params.m, params.n, params.o, params.l = M, N, coef.shape[-1], L
+    params.matrix, params.matrix_ld, params.matrix_bs = matrix.data_ptr(), matrix.stride(1), matrix.stride(0)
+    params.coef, params.coef_ld, params.coef_bs = coef.data_ptr(), coef.stride(1), coef.stride(0)
+    params.out, params.out_ld, params.out_bs = out.data_ptr(), out.stride(-2), out.stride(-3)
+    params.accumulate = accumulate
+    if splits > 1:
+        params.n_splits, params.out_split_stride = splits, out.stride(0)
+    _backend.matrix_times_coefficients(params, torch.cuda.current_stream().cuda_stream)
+
+
+@pytest.mark.parametrize("L,N,M,O", [(1, 1, 1, 1), (2, 77, 130, 5), (3, 1000, 65, 33), (1, 513, 64, 32), (2, 64, 300, 48),
+                                     (1, 9, 7, 17), (1, 4097, 100, 8), (1, 300, 1029, 4), (1, 100, 50, 31), (1, 2100, 600, 12)])
+@pytest.mark.parametrize("padded", [False, True])
+def test_contraction_of_a_stored_panel(device, L, N, M, O, padded):
+    """Both kernels (rows read 4 or 16 bytes per lane), whole and in ranges of n, stored and added,
+    with padded rows of every operand; elements beside the result stay as they were."""
+    g = torch.Generator().manual_seed(L + N + M + O)
+    ld = (M + 3) // 4 * 4 if padded else M
+    matrix = torch.randn(L, N, ld, generator=g).to(device)[:, :, :M]
+    coef = torch.randn(L, N, O + 2, generator=g).to(device)[:, :, :O]
+    truth = torch.bmm(matrix.double().transpose(1, 2), coef.double())
+    scale = torch.bmm(matrix.double().abs().transpose(1, 2), coef.double().abs())
+    store = torch.full((L, M, O + 3), 7.0, device=device)
+    out = store[:, :, :O]
+    contraction(matrix, coef, out)
+    assert float(((out.double() - truth).abs() / scale).max()) < 1e-6
+    again = torch.full_like(store, 7.0)
+    contraction(matrix, coef, again[:, :, :O])
+    assert torch.equal(again, store), "two runs differ"
+    contraction(matrix, coef, out, accumulate=1)
+    assert float(((out.double() - 2 * truth).abs() / scale).max()) < 2e-6
+    assert torch.all(store[:, :, O:] == 7.0), "wrote outside the out view"
+    for splits in (2, 5):
+        partial = torch.full((splits, L, M, O), float("nan"), device=device)
+        contraction(matrix, coef, partial, splits=splits)
+        assert float(((partial.double().sum(0) - truth).abs() / scale).max()) < 1e-6, f"{splits} ranges"
+
+
+def test_contraction_without_rows_stores_zeros(device):
+    matrix = torch.empty(2, 0, 64, device=device)
+    coef = torch.empty(2, 0, 5, device=device)
+    out = torch.full((2, 64, 5), 3.0, device=device)
+    contraction(matrix, coef, out, accumulate=1)
+    assert torch.all(out == 3.0)
+    contraction(matrix, coef, out)
+    assert torch.all(out == 0.0)
+
+
+@pytest.mark.parametrize("M,N,K,O", [(130, 700, 17, 5), (257, 1029, 40, 33), (300, 512, 64, 70), (64, 300, 33, 1), (1000, 260, 24, 16)])
+@pytest.mark.parametrize("layout", ["cc", "rr", "cr"])
+def test_shapes_and_layouts(device, panels, capsys, M, N, K, O, layout):
+    g = torch.Generator().manual_seed(M + N + K + O)
+    a = make_operand(1, M, K, layout[0] == "c", device, g, batch=False)
+    b = make_operand(1, N, K, layout[1] == "c", device, g, batch=False)
+    coef = torch.randn(N, O, generator=g).to(device)
+    for descriptor, names, kw in CASES:
+        got = kermac.run_kernel(descriptor, a, b, coefficients=coef, debug=True, **kw)
+        assert f"{PANELS} {-(-N // 256)} panels of 256 centres" in capsys.readouterr().out
+        assert got.shape == (1, M, O)
+        truth = oracle.kernel_times_coefficients(*names, a.cpu(), b.cpu(), coef.cpu(), **kw)
+        assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"{names} {layout}")
+        assert torch.equal(got, kermac.run_kernel(descriptor, a, b, coefficients=coef, **kw)), "two runs differ"
+
+
+def test_batches_and_a_regularised_diagonal_across_panels(device, panels, capsys):
+    g = torch.Generator().manual_seed(81)
+    L, M, N, K, O = 3, 700, 900, 24, 12
+    x = make_operand(L, M, K, True, device, g)
+    z = make_operand(1, N, K, True, device, g, batch=False)                  # broadcast centres
+    coef = torch.randn(L, N, O + 3, generator=g).to(device)[:, :, :O]         # padded rows
+    bw = torch.tensor([4.0, 6.0, 9.0], device=device)
+    out = torch.full((L, M, O + 1), 5.0, device=device)
+    # the elements with 2 + n == m get 1 + regularization: they lie in each of the four panels
+    kw = dict(bandwidth=bw, regularization=0.5, regularization_offset_x=2, regularization_offset_y=0)
+    got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, z, out=out[..., :O], coefficients=coef, debug=True, **kw)
+    assert f"{PANELS} 4 panels" in capsys.readouterr().out
+    assert torch.all(out[..., O] == 5.0), "wrote outside the out view"
+    truth = oracle.run_kernel_coefficients("DIFF", "SQUARE", "SQRT", "LAPLACE", x.cpu().contiguous(),
+                                           z.cpu().contiguous(), coef.cpu().contiguous(), bandwidth=bw.cpu(),
+                                           regularization=0.5, regularization_offset_x=2, regularization_offset_y=0)
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="panels vs oracle")
+    # without the diagonal the result differs: the test above does see it
+    plain = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, x, z, coefficients=coef, bandwidth=bw)
+    assert not torch.allclose(plain, got, rtol=1e-3, atol=0.0)
+    # rows broadcast over the batch, centres per batch entry, a row-major result view
+    x1 = make_operand(1, M, K, False, device, g, batch=False)
+    zl = make_operand(L, N, K, False, device, g)
+    got = kermac.run_kernel(GAUSSIAN, x1, zl, coefficients=coef, bandwidth=5.0)
+    truth = oracle.run_kernel_coefficients("DIFF", "SQUARE", "NOOP", "GAUSSIAN", x1.cpu().contiguous(),
+                                           zl.cpu().contiguous(), coef.cpu().contiguous(), bandwidth=5.0)
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="broadcast rows")
+
+
+def test_near_duplicates_far_from_the_origin(device, panels):
+    """Parts of the panels whose squared distances cancel are recomputed by the direct kernel
+    before the contraction reads them."""
+    g = torch.Generator().manual_seed(82)
+    base = torch.randn(50, 32, generator=g) + 40.0
+    x = (base.repeat(6, 1) + 1e-3 * torch.randn(300, 32, generator=g)).to(device)
+    z = (base.repeat(12, 1) + 1e-3 * torch.randn(600, 32, generator=g)).to(device)
+    coef = torch.randn(600, 20, generator=g).to(device)
+    for descriptor, names, kw in CASES[:2]:
+        got = kermac.run_kernel(descriptor, x, z, coefficients=coef, **kw)
+        truth = oracle.kernel_times_coefficients(*names, x.cpu(), z.cpu(), coef.cpu(), **kw)
+        assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"{names} near duplicates")
+
+
+def test_which_calls_go_in_panels(device, monkeypatch, capsys):
+    """Squared differences in the modes "auto" and "gram_bf16" only, only when the panels are large
+    enough for the workspace route, and not with KERMAC_AMD_COEFFICIENT_PANEL_BYTES=0."""
+    g = torch.Generator().manual_seed(83)
+    a = torch.randn(2048, 1024, generator=g).to(device)
+    b = torch.randn(8192, 1024, generator=g).to(device)
+    coef = torch.randn(8192, 8, generator=g).to(device)
+
+    def in_panels(descriptor=GAUSSIAN, rows=a, **kw):
+        capsys.readouterr()
+        kw.setdefault("bandwidth", 32.0)
+        kermac.run_kernel(descriptor, rows, b, coefficients=coef, debug=True, **kw)
+        return PANELS in capsys.readouterr().out
+
+    assert kermac.get_l2_mode() == "auto"
+    assert in_panels()                                               # 8 x 32 tiles, 1.7e10 terms
+    assert in_panels(kermac.kernel_descriptor_laplace_l2)
+    assert not in_panels(kermac.kernel_descriptor_laplace_l1)
+    assert not in_panels(rows=a[:512])                               # 2 x 32 tiles: the split is not earned back
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "0")
+    assert not in_panels()
+    monkeypatch.delenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES")
+    monkeypatch.setenv("KERMAC_AMD_L2_WORKSPACE", "0")
+    assert not in_panels()
+    monkeypatch.delenv("KERMAC_AMD_L2_WORKSPACE")
+    for mode, expected in (("gram", False), ("direct", False), ("gram_bf16", True)):
+        with kermac.l2_mode(mode):
+            assert in_panels() == expected, mode
+    with kermac.l2_mode("direct"):
+        direct = kermac.run_kernel(GAUSSIAN, a, b, coefficients=coef, bandwidth=32.0)
+    got = kermac.run_kernel(GAUSSIAN, a, b, coefficients=coef, bandwidth=32.0)
+    assert_close_to_truth(got, direct.double(), rtol=1e-5, atol=atol_for(direct, 1e-5), what="panels vs direct fused kernel")
+
+
+def test_headline_shape_gaussian(device, capsys):
+    """The fused benchmark shape (batch 4, 16384 x 16384, K = 256, O = 32) with a Gaussian kernel in
+    the default mode: four panels of 4096 centres; float64 slabs of the result."""
+    torch.manual_seed(5)
+    L, K, NX, MZ, O = 4, 256, 16384, 16384, 32
+    x = torch.rand(L, K, NX, device=device) * 2 - 1
+    z = torch.rand(K, MZ, device=device) * 2 - 1
+    coef = torch.randn(L, MZ, O, device=device)
+    out = torch.empty(L, NX, O, device=device)
+    kermac.run_kernel(GAUSSIAN, x.transpose(1, 2), z.t(), out=out, bandwidth=9.0, coefficients=coef, debug=True)
+    assert f"{PANELS} 4 panels of 4096 centres" in capsys.readouterr().out
+    for l, rows in ((0, slice(0, 96)), (3, slice(16300, 16384))):
+        d2 = torch.cdist(x[l, :, rows].t().double(), z.t().double(), p=2.0) ** 2
+        truth = torch.exp(-d2 / (2 * 9.0 ** 2)) @ coef[l].double()
+        assert_close_to_truth(out[l, rows], truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"gaussian slab batch {l}")

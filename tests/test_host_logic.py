@@ -507,6 +507,36 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert gradient(3, 2, 1, 5) > 0
 
 
+def test_matrix_times_coefficients_checks_its_arguments_before_any_device_call():
+    """kmc_matrix_times_coefficients: extents, strides and the l * n_splits limit are checked
+    first, and an empty product returns without touching a device."""
+    def params(m=64, n=100, o=8, l=1, **fields):
+        block = _backend.MatrixCoefficientsParams()
+        block.m, block.n, block.o, block.l = m, n, o, l
+        block.matrix, block.matrix_ld, block.matrix_bs = 4096, m, m * n
+        block.coef, block.coef_ld, block.coef_bs = 4096, o, n * o
+        block.out, block.out_ld, block.out_bs = 4096, o, m * o
+        for name, value in fields.items():
+            setattr(block, name, value)
+        return block
+
+    for bad in (params(m=-1), params(matrix_ld=32), params(coef_ld=4), params(out_ld=4), params(out=None),
+                params(matrix=None), params(l=70000), params(l=300, n_splits=300), params(n_splits=-2),
+                params(out_split_stride=-1)):
+        with pytest.raises(_backend.BackendError) as info:
+            _backend.matrix_times_coefficients(bad, 0)
+        assert info.value.status == _backend.ERR_INVALID_ARGUMENT
+    for empty in (params(m=0), params(o=0), params(l=0)):
+        _backend.matrix_times_coefficients(empty, 0)
+    # the Python mirror cuts the n of a panel so that the contraction has a workgroup per CU
+    from kermac_amd.kernel_coefficients import _panel_splits
+    assert _panel_splits(16384, 32, 4, 4096) == 1            # 512 workgroups of 128 rows
+    assert _panel_splits(8192, 8, 1, 4096) == 4              # 64 workgroups
+    assert _panel_splits(8192, 8, 1, 1024) == 2              # at least 512 rows per range
+    assert _panel_splits(30000, 16, 1, 16384) == 4           # sums of at most 4096 rows per workgroup
+    assert _panel_splits(128, 1, 60000, 1 << 20) == 1        # l * n_splits stays below 65536
+
+
 def test_launch_cuts_follow_the_shape_and_the_environment_switch(monkeypatch):
     """The cut over k is decided from the parameter block alone: small and middling results over a
     long contraction are cut, batches, short contractions and large results are not, and
