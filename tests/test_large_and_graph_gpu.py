@@ -184,6 +184,7 @@ def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
     new values equals the eager result bit for bit."""
     monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
     monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "4096")         # panels of 256 centres: three here
     g = torch.Generator().manual_seed(77)
     M, N, K, O = 600, 520, 96, 16
     a_store = torch.randn(K, M, generator=g).to(device)
@@ -196,14 +197,19 @@ def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
     out_p2 = torch.empty(N, M, device=device)
     out_self = torch.empty(M, M, device=device)
     out_grad = torch.empty(O, K, M, device=device)
+    coefficients = torch.randn(N, 5, generator=g).to(device)
+    out_product = torch.empty(1, M, 5, device=device)
 
     def run_all():
         with kermac.l2_mode("gram_bf16", min_k=0):
             kermac.cdist(a_store.t(), b_store.t(), p=2.0, out=out_p2.t())
             kermac.cdist(a_store.t(), a_store.t(), p=2.0, out=out_self.t())
+            # the kernel matrix x coefficients product panel by panel: panel, workspace and partial products
+            kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, a_store.t(), b_store.t(), out=out_product,
+                              bandwidth=10.0, coefficients=coefficients)
         kermac.cdist_grad(weights, centres, classes, samples, out=out_grad, p=1.0)
 
-    outs = (out_p2, out_self, out_grad)
+    outs = (out_p2, out_self, out_grad, out_product)
     side = torch.cuda.Stream(device=device)
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -225,10 +231,13 @@ def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
         graph.replay()
         torch.cuda.synchronize()
         del scratch
-        for name, e, o in zip(("p2", "p2 self", "grad"), eager, outs):
+        for name, e, o in zip(("p2", "p2 self", "grad", "product in panels"), eager, outs):
             assert torch.equal(e, o), f"replay {replay}: {name} differs from the eager result"
     truth = oracle.cdist(a_store.t().cpu(), b_store.t().cpu(), p=2.0)[0]
     assert_close_to_truth(out_p2.t(), truth, rtol=1e-5, atol=1e-30, what="graph replay vs oracle")
+    truth = oracle.kernel_times_coefficients("DIFF", "SQUARE", "SQRT", "LAPLACE", a_store.t().cpu(), b_store.t().cpu(),
+                                             coefficients.cpu(), bandwidth=10.0)
+    assert_close_to_truth(out_product, truth, rtol=1e-5, atol=1e-4 * float(truth.abs().mean()), what="product replay vs oracle")
 
 
 def test_cut_launches_replay_from_a_hip_graph(device):
