@@ -464,8 +464,7 @@ def main():
         torch.cuda.empty_cache()
         for name, fn in (("cdist_grad", bench_cdist_grad), ("kernel_coef", bench_kernel_coef)):
             log(f"other configuration: {name}")
-            side = fn(kermac, device, args, steps=side_steps, warmup=1) if name == "cdist_grad" else \
-                fn(kermac, device, args, steps=side_steps, warmup=1, with_gaussian=False)
+            side = fn(kermac, device, args, steps=side_steps, warmup=1)
             other_configs[name] = {key: side[key] for key in side if key not in ("n_gpus", "higher_is_better", "scaling",
                                                                                   "vs_baseline", "data", "dtype")}
             other_configs[name]["steps"], other_configs[name]["warmup"] = side_steps, 1
