@@ -138,6 +138,23 @@ def test_batches_and_a_regularised_diagonal_across_panels(device, panels, capsys
     assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="broadcast rows")
 
 
+def test_one_panel_goes_straight_into_a_strided_result(device, panels, capsys):
+    """Many rows against one panel of centres: no partial products, the contraction writes the
+    caller's result, here a view with padded rows and shared coefficients."""
+    g = torch.Generator().manual_seed(84)
+    L, M, N, K, O = 8, 4096, 200, 16, 4
+    x = make_operand(L, M, K, True, device, g)
+    z = make_operand(L, N, K, False, device, g)
+    coef = torch.randn(N, O, generator=g).to(device)                          # one set of coefficients for the batch
+    store = torch.full((L, M, O + 2), 5.0, device=device)
+    got = kermac.run_kernel(GAUSSIAN, x, z, out=store[..., :O], coefficients=coef, bandwidth=3.0, debug=True)
+    assert f"{PANELS} 1 panels of 200 centres, 1 partial products each" in capsys.readouterr().out
+    assert torch.all(store[..., O:] == 5.0), "wrote outside the out view"
+    truth = oracle.run_kernel_coefficients("DIFF", "SQUARE", "NOOP", "GAUSSIAN", x.cpu().contiguous(), z.cpu().contiguous(),
+                                           coef.cpu().expand(L, N, O).contiguous(), bandwidth=3.0)
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="one panel")
+
+
 def test_near_duplicates_far_from_the_origin(device, panels):
     """Parts of the panels whose squared distances cancel are recomputed by the direct kernel
     before the contraction reads them."""
