@@ -374,7 +374,8 @@ def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
         pytest.skip("no C compiler")
     structs = {"kmc_build_kernel_params": _backend.BuildKernelParams,
                "kmc_norm_gradient_params": _backend.NormGradientParams,
-               "kmc_kernel_coefficients_params": _backend.KernelCoefficientsParams}
+               "kmc_kernel_coefficients_params": _backend.KernelCoefficientsParams,
+               "kmc_matrix_coefficients_params": _backend.MatrixCoefficientsParams}
     lines = ['#include "kermac_amd.h"', "#include <stddef.h>", "#include <stdio.h>", "int main(void) {"]
     for c_name, binding in structs.items():
         lines.append(f'  printf("{c_name} size %zu\\n", sizeof(struct {c_name}));')
