@@ -22,11 +22,13 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(autouse=True, params=["as launched", "workspace routes"])
 def routes(request, monkeypatch):
     """Every sweep twice: as the library launches these small shapes by itself, and with the routes
-    that go through a workspace forced onto them (squared differences and the L1 gradient on the
-    fp16 matrix instruction, which by themselves only take large problems)."""
+    that go through a workspace forced onto them (squared differences, their products with
+    coefficients panel by panel, and the L1 gradient on the fp16 matrix instruction, which by
+    themselves only take large problems)."""
     if request.param == "workspace routes":
         monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
         monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
+        monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "4096")     # products in panels of 256 centres
         kermac.set_l2_mode("gram_bf16", min_k=0)
     yield
     kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
@@ -161,7 +163,7 @@ def test_fused_coefficients_random(device, seed):
     gen = torch.Generator().manual_seed(6000 + seed)
     for case in range(6):
         L = rng.choice([1, 2, 3])
-        M, N, K = rng.randint(1, 300), rng.randint(1, 300), rng.randint(1, 60)
+        M, N, K = rng.randint(1, 300), rng.randint(1, 700), rng.randint(1, 60)
         O = rng.choice([1, 3, 16, 32, 33, 70])
         name, inner_pow, outer_pow, kernel = rng.choice([
             ("laplace_l1", "ABS", "NOOP", "LAPLACE"), ("laplace_l2", "SQUARE", "SQRT", "LAPLACE"),
