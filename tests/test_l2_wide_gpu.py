@@ -6,7 +6,8 @@ relative to the float64 truth -- trusted 128 x 128 parts by the error bound of t
 distrusted parts because the direct kernel recomputes them.
 
 KERMAC_AMD_WIDE_MIN_TILES=1 sends the small shapes of these tests down the route, which by itself
-only takes problems of at least 192 tiles.
+only takes problems of at least 128 tiles of 256 x 256 (and K >= 64, several tiles in both directions
+of every batch entry, little padding: kmc_gram_workspace_bytes in include/kermac_amd.h).
 """
 import pytest
 import torch
