@@ -10,6 +10,7 @@ matrix ever reaching memory, with exactly the per-element semantics of
 from __future__ import annotations
 
 import functools
+import os
 from typing import Optional
 
 import torch
@@ -151,9 +152,10 @@ def run_kernel_coefficients(
 # reused, and kmc_matrix_times_coefficients contracts it with the coefficients of those centres.
 # The full matrix never exists; the panel (1 GiB unless KERMAC_AMD_COEFFICIENT_PANEL_BYTES says
 # otherwise, 0 switches the route off) does.  Measured, fused kernel -> panels: L = 4,
-# M = N = 16384, O = 32 at K = 256 7.5 -> 4.9 ms, at K = 1024 22.4 -> 8.9 ms; M = N = 30000,
-# K = 1024, O = 16 18.5 -> 8.4 ms.  The partial products of the panels (and of the ranges a panel
-# is cut into when the rows alone do not fill the chip) are added in a fixed order.
+# M = N = 16384, O = 32 at K = 256 7.7 -> 4.7 ms, at K = 1024 22.6 -> 8.4 ms; M = N = 30000,
+# K = 1024, O = 16 18.6 -> 7.1 ms; M = 10000, N = 100000, K = 784, O = 10 16.6 -> 8.0 ms; M = 20000,
+# N = 50000, K = 3072, O = 10 56.8 -> 17.8 ms.  The partial products of the panels (and of the
+# ranges a panel is cut into when the rows alone do not fill the chip) are added in a fixed order.
 _PANEL_BYTES = 1 << 30
 _PANEL_MAX_PARTIAL_BYTES = 512 << 20
 
@@ -168,8 +170,6 @@ def _panel_splits(M, O, L, rows):
 
 def _run_in_panels(plan, stream, device, debug):
     """The product panel by panel (above); False when this problem stays with the fused kernel."""
-    import os
-
     from .build_a_kernel import _attach_gram_workspace, _l2_current
 
     budget = int(os.environ.get("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", _PANEL_BYTES))
