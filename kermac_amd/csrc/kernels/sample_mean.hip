@@ -42,27 +42,56 @@ __device__ __forceinline__ i64 sampled_row(const SampleMeanArgs &args, int s)
     return (i64)run * (args.rows - SM_RUN) / (SM_RUNS - 1) + (s - run * SM_RUN);
 }
 
-// k contiguous (row-major panel): a workgroup owns 64 k, four groups of lanes share the rows.
-__global__ __launch_bounds__(256) void sample_mean_rows(const SampleMeanArgs args)
+// k contiguous (row-major panel): a workgroup owns 64 k, its 16 waves share the rows, and a wave
+// has eight rows under way at once (eight sums per lane, added in a fixed order at the end): the
+// panel's rows lie K floats apart, so the time is that of the loads' latency, not of their bytes.
+constexpr int SM_ROW_WAVES = 16;
+constexpr int SM_ROW_UNROLL = 8;
+
+__global__ __launch_bounds__(64 * SM_ROW_WAVES) void sample_mean_rows(const SampleMeanArgs args)
 {
-    __shared__ float partial[4][64];
+    __shared__ float partial[SM_ROW_WAVES][64];
+    __shared__ float partial_squares[SM_ROW_WAVES][64];
     const int kk = threadIdx.x & 63, group = threadIdx.x >> 6;
     const int k = blockIdx.x * 64 + kk;
     const float *x = args.x + blockIdx.y * args.bs;
-    __shared__ float partial_squares[4][64];
-    float sum = 0.0f, squares = 0.0f;
-    if (k < args.k)
-        for (int s = group; s < args.samples; s += 4) {
-            const float v = x[sampled_row(args, s) * args.ld + k];
-            sum += v;
-            squares += v * v;
+    float sum[SM_ROW_UNROLL], squares[SM_ROW_UNROLL];
+#pragma unroll
+    for (int u = 0; u < SM_ROW_UNROLL; ++u) sum[u] = squares[u] = 0.0f;
+    if (k < args.k) {
+        int s = group;
+        for (; s + (SM_ROW_UNROLL - 1) * SM_ROW_WAVES < args.samples; s += SM_ROW_UNROLL * SM_ROW_WAVES) {
+            float v[SM_ROW_UNROLL];
+#pragma unroll
+            for (int u = 0; u < SM_ROW_UNROLL; ++u) v[u] = x[sampled_row(args, s + u * SM_ROW_WAVES) * args.ld + k];
+#pragma unroll
+            for (int u = 0; u < SM_ROW_UNROLL; ++u) {
+                sum[u] += v[u];
+                squares[u] += v[u] * v[u];
+            }
         }
-    partial[group][kk] = sum;
-    partial_squares[group][kk] = squares;
+        for (; s < args.samples; s += SM_ROW_WAVES) {
+            const float v = x[sampled_row(args, s) * args.ld + k];
+            sum[0] += v;
+            squares[0] += v * v;
+        }
+    }
+    float mine = 0.0f, mine_squares = 0.0f;
+#pragma unroll
+    for (int u = 0; u < SM_ROW_UNROLL; ++u) {
+        mine += sum[u];
+        mine_squares += squares[u];
+    }
+    partial[group][kk] = mine;
+    partial_squares[group][kk] = mine_squares;
     __syncthreads();
     if (group == 0 && k < args.k_padded) {
-        const float total = ((partial[0][kk] + partial[1][kk]) + partial[2][kk]) + partial[3][kk];
-        const float total_squares = ((partial_squares[0][kk] + partial_squares[1][kk]) + partial_squares[2][kk]) + partial_squares[3][kk];
+        float total = 0.0f, total_squares = 0.0f;
+#pragma unroll
+        for (int w = 0; w < SM_ROW_WAVES; ++w) {
+            total += partial[w][kk];
+            total_squares += partial_squares[w][kk];
+        }
         const bool live = k < args.k && args.samples > 0;
         const float mean = live ? total / (float)args.samples : 0.0f;
         args.mean[blockIdx.y * args.mean_bs + k] = mean;
@@ -155,7 +184,7 @@ extern "C" int kmc_sample_mean(const float *x, int32_t majorness, int32_t rows, 
     args.samples = rows < kmc::SM_MAX_SAMPLES ? rows : kmc::SM_MAX_SAMPLES;
     hipError_t e;
     if (majorness == KMC_ROW_MAJOR)
-        e = kmc_host::launch(kmc::sample_mean_rows, dim3(k_padded / 64, l), dim3(256), static_cast<hipStream_t>(stream), args);
+        e = kmc_host::launch(kmc::sample_mean_rows, dim3(k_padded / 64, l), dim3(64 * kmc::SM_ROW_WAVES), static_cast<hipStream_t>(stream), args);
     else
         e = kmc_host::launch(kmc::sample_mean_columns, dim3(k_padded / 4, l), dim3(256), static_cast<hipStream_t>(stream), args);
     if (e != hipSuccess) return kmc_host::fail_hip(e, "sample_mean launch");
