@@ -228,6 +228,23 @@ def bench_cdist_grad(kermac, device, args, steps=None, warmup=None):
             os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"] = saved
     log(f"  on the fp32 matrix-core kernel: {fp32_ms:.2f} ms, slab max abs err / mean |truth| = {fp32_err:.2e}")
     check_parity("cdist_grad p=1 (configs[3], fp32 kernels) slab, max abs err / mean |truth|", fp32_err, 1e-4)
+    # Beside it: the same operands with p = 2 (weights d - b instead of their sign), both routes.
+    truth_l2 = torch.einsum("ok,km,nmk->onm", c.double(), a[:, ms].double(), diff)
+    side = max(2, min(steps, 5))
+    _, l2_ms = time_call(lambda: kermac.cdist_grad(a, b, c, d, out=out, p=2.0), side, 1)
+    l2_err = ((out[0][:, ns, ms].double() - truth_l2).abs().max() / truth_l2.abs().mean()).item()
+    os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"] = "0"
+    try:
+        _, l2_fp32_ms = time_call(lambda: kermac.cdist_grad(a, b, c, d, out=out, p=2.0), side, 1)
+        l2_fp32_err = ((out[0][:, ns, ms].double() - truth_l2).abs().max() / truth_l2.abs().mean()).item()
+    finally:
+        if saved is None:
+            del os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"]
+        else:
+            os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"] = saved
+    log(f"  p=2, same operands: {l2_ms:.2f} ms (slab err {l2_err:.2e}); on the fp32 matrix-core kernel {l2_fp32_ms:.2f} ms ({l2_fp32_err:.2e})")
+    check_parity("cdist_grad p=2 slab, max abs err / mean |truth|", l2_err, 1e-4)
+    check_parity("cdist_grad p=2 (fp32 kernels) slab, max abs err / mean |truth|", l2_fp32_err, 1e-4)
     # Executed matrix work on the default route: three products of fp16 pieces, 2 * O flops each per (m, n, k),
     # against the dense fp16 peak; the sign work on the vector ALU (2.5 instructions per (m, n, k)) is what bounds it.
     ops = 3.0 * 2.0 * o * m_ref * n_ref * k_ref
@@ -240,7 +257,12 @@ def bench_cdist_grad(kermac, device, args, steps=None, warmup=None):
                       "route": "a and c split once into two fp16 pieces per value, sign of d - b on the pieces, v_mfma_f32_16x16x32_f16",
                       "useful_tflops": round((2.0 * o + 3.0) * m_ref * n_ref * k_ref / kernel_ms / 1e9, 2),
                       "fp32_kernels_same_run": {"ms": round(fp32_ms, 3), "parity_max_err_over_mean": fp32_err,
-                                                "frac_of_fp32_mfma_peak": round((2.0 * o + 3.0) * m_ref * n_ref * k_ref / fp32_ms / 1e9 / 157.3, 4)}},
+                                                "frac_of_fp32_mfma_peak": round((2.0 * o + 3.0) * m_ref * n_ref * k_ref / fp32_ms / 1e9 / 157.3, 4)},
+                      "p2_same_operands": {"ms": round(l2_ms, 3), "parity_max_err_over_mean": l2_err,
+                                           "route": "e = (d - s) (c a) - (c (b - s)) a with s the row means of b: one product of "
+                                                    "(o n) x k by k x m from two fp16 pieces per value, v_mfma_f32_32x32x16_f16",
+                                           "mfma_tflops": round(3.0 * 2.0 * o * m_ref * n_ref * k_ref / l2_ms / 1e9, 2),
+                                           "fp32_kernels_ms": round(l2_fp32_ms, 3), "fp32_kernels_parity_max_err_over_mean": l2_fp32_err}},
                      args)
 
 

@@ -258,22 +258,31 @@ typedef struct kmc_norm_gradient_params {
     const float *d; int64_t d_ld; int64_t d_bs;   /* [n, m], m contiguous */
     float *e; int64_t e_ld_n; int64_t e_ld_o; int64_t e_bs; /* [o, n, m], m contiguous */
     const float *p; int64_t p_bs; float p_value;
-    /* KMC_NORM_L1 only (ignored otherwise): device memory the call may use, 256-byte aligned, of at
-     * least the size kmc_norm_gradient_workspace_bytes reports for these parameters.  With it, large
-     * problems run on the fp16 matrix instruction: a and c are split once into two fp16 pieces per
+    /* KMC_NORM_L1 and KMC_NORM_L2 (ignored otherwise): device memory the call may use, 256-byte
+     * aligned, of at least the size kmc_norm_gradient_workspace_bytes reports for these parameters.
+     * With it, large problems run on the fp16 matrix instruction.  KMC_NORM_L1: a and c are split once into two fp16 pieces per
      * value (a power-of-two scale per row m of a and per row o of c), the sign of d - b is put on
      * the pieces of a exactly, and the contraction takes 3 matrix instructions per 32 k where the
      * fp32 kernel issues 8 of twice the duration.  Error of e from the pieces below
      * 3 * 2^-22 sum_k |c a|, beside the rounding of the fp32 accumulation that both kernels have.
+     * KMC_NORM_L2 with e_ld_o = n * e_ld_n (the planes of e one matrix of o * n rows): large problems
+     * run as e = (d - s) g - p a with g[m][o] = sum_k a c, p[o n_rows + n][k] = c[o][k] (b[n][k] - s[n])
+     * and s[n] the mean of row n of b (any s gives the same e; this one keeps both terms as small
+     * as the data allows): p and a are split once into two fp16 pieces per value with a scale per
+     * row and multiplied in 256 x 256 tiles on the fp16 matrix instruction, g comes from the fp32
+     * matrix instruction; the workspace also holds p in fp32.  Error of the product from the pieces
+     * below 3 * 2^-22 sum_k |c a (b - s)|.
      * NULL, too small, or a problem for which the query reports 0: the fp32 kernels run. */
     void *workspace;
     int64_t workspace_bytes;
 } kmc_norm_gradient_params;
 
 /* Bytes of workspace that kmc_norm_kernel_gradient would use for these parameters, 0 when it would
- * not use one (another norm than L1, fewer than 3 outputs, n < 24, or fewer terms m * n * k * l
- * than 6.4e9 / min(o, 16): 4e8 at 16 outputs).  About 1.1 times the
- * bytes of a, b and c.  No counterpart in the reference. */
+ * not use one.  KMC_NORM_L1: at least 3 outputs, n >= 24 and m * n * k * l terms of at least
+ * 6.4e9 / min(o, 16) (4e8 at 16 outputs); about 1.1 times the bytes of a, b and c.  KMC_NORM_L2:
+ * when a model of both times favours the route by 15 % (tiles of 256 x 256 over m and o * n, in
+ * both directions, and a contraction of about 512 or more); about 4 (m + 2 o n) k bytes.
+ * KMC_NORM_P: never.  No counterpart in the reference. */
 int kmc_norm_gradient_workspace_bytes(const kmc_norm_gradient_params *params, int64_t *bytes);
 
 /* Stands in for launch(stream, config, cute_norm_kernel_gradient<NormType>, *args)

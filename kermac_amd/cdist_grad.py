@@ -170,10 +170,12 @@ def cdist_grad(
 
 
 def _attach_workspace(params, device):
-    """Large L1 gradients run on the fp16 matrix instruction through a workspace (include/
-    kermac_amd.h, kmc_norm_gradient_params::workspace: a and c split once into two fp16 pieces per
-    value, the sign of d - b put on the pieces of a); the library says how much it wants for this
-    call, 0 when it would not use one.  KERMAC_AMD_GRADIENT_WORKSPACE=0 keeps every call on the fp32 kernels."""
+    """Large L1 and L2 gradients run on the fp16 matrix instruction through a workspace (include/
+    kermac_amd.h, kmc_norm_gradient_params::workspace.  L1: a and c split once into two fp16 pieces
+    per value, the sign of d - b put on the pieces of a.  L2: the sum factors into
+    (d - s) (c a) - (c (b - s)) a, one product of pieces); the library says how much it wants for
+    this call, 0 when it would not use one.  KERMAC_AMD_GRADIENT_WORKSPACE=0 keeps every call on
+    the fp32 kernels."""
     if os.environ.get("KERMAC_AMD_GRADIENT_WORKSPACE", "1") in ("", "0"):
         return None
     needed = _backend.norm_gradient_workspace_bytes(params)

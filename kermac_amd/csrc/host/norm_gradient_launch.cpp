@@ -10,6 +10,8 @@ hipError_t launch_norm_gradient(int norm_type, int o_tile, const kmc::NormGradie
 int64_t norm_gradient_f16_bytes(const kmc_norm_gradient_params *p);
 hipError_t launch_norm_gradient_f16(const kmc_norm_gradient_params *p, bool a_vec, bool c_vec, bool e_vec, hipStream_t stream,
                                     bool *taken);
+int64_t norm_gradient_l2_wide_bytes(const kmc_norm_gradient_params *p);
+int launch_norm_gradient_l2_wide(const kmc_norm_gradient_params *p, hipStream_t stream, bool *taken);
 }
 
 namespace {
@@ -50,7 +52,8 @@ extern "C" int kmc_norm_gradient_workspace_bytes(const kmc_norm_gradient_params 
     if (!bytes) return fail(KMC_ERR_INVALID_ARGUMENT, "bytes: null pointer");
     int status = check(p);
     if (status != KMC_OK) return status;
-    *bytes = (p->m == 0 || p->n == 0 || p->o == 0 || p->l == 0) ? 0 : norm_gradient_f16_bytes(p);
+    if (p->m == 0 || p->n == 0 || p->o == 0 || p->l == 0) *bytes = 0;
+    else *bytes = p->norm_type == KMC_NORM_L2 ? norm_gradient_l2_wide_bytes(p) : norm_gradient_f16_bytes(p);
     return KMC_OK;
 }
 
@@ -67,6 +70,14 @@ extern "C" int kmc_norm_kernel_gradient(const kmc_norm_gradient_params *p, void 
                                                 vec_ok(p->e, p->e_ld_n, p->e_ld_o, p->e_bs, p->flags), static_cast<hipStream_t>(stream),
                                                 &taken);
         if (e != hipSuccess) return fail_hip(e, "norm_gradient_l1_f16 launches");
+        if (taken) return KMC_OK;
+    }
+    if (p->norm_type == KMC_NORM_L2 && p->workspace && p->k > 0) {
+        int ready = require_gfx950();
+        if (ready != KMC_OK) return ready;
+        bool taken = false;
+        const int launched = launch_norm_gradient_l2_wide(p, static_cast<hipStream_t>(stream), &taken);
+        if (launched != KMC_OK) return launched;
         if (taken) return KMC_OK;
     }
 

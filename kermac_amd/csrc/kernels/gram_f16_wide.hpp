@@ -89,7 +89,16 @@ struct GramWideArgs {
     i64 unscale_a_bs, unscale_b_bs;
     int rows_pad_a, rows_pad_b, slices, ranges;
     int wide_tiles_m, wide_tiles_n, wide_tiles_n_padded;
+    // GW_EPILOGUE_GRADIENT_L2 only: row r of b stands for (o, n) = (r / gradient_n, r % gradient_n) and
+    // the result is (d[n][m] - shift[n]) * g[m][o] - a[m] . b[r]
+    const float *gradient_d; i64 gradient_d_ld, gradient_d_bs;
+    const float *gradient_g; i64 gradient_g_ld, gradient_g_bs;
+    const float *gradient_shift; i64 gradient_shift_bs;
+    int gradient_n;
 };
+
+constexpr int GW_EPILOGUE_DISTANCE = 0;
+constexpr int GW_EPILOGUE_GRADIENT_L2 = 1;
 
 // The 16 values of row `row` in slice `slice`, centre subtracted; zeros where the row or k does not exist.
 __device__ __forceinline__ void gram_load_row_slice(const GramRowsArgs &args, const float *x, const float *centre, int row,
@@ -260,7 +269,11 @@ __device__ __forceinline__ bool wide_tile_of_workgroup(const GramWideArgs &args,
 // such a part are computed with the pieces in exchanged roles and differ in the last bit); the
 // part above the diagonal inside a diagonal tile is not stored from its own values at all.  A
 // distrusted part is left to the repair launch, which mirrors what it recomputes.
-template <bool SYMMETRIC>
+//
+// EPILOGUE GW_EPILOGUE_GRADIENT_L2: the same walk as a plain product of the pieces, for the gradient
+// of the L2 norm (norm_gradient_l2_wide.hpp): no norms, no trust check, the epilogue combines the
+// product with d and g as GramWideArgs says.
+template <bool SYMMETRIC, int EPILOGUE = GW_EPILOGUE_DISTANCE>
 __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs args)
 {
     __shared__ gram_chunk lds0[GW_BUFFER_CHUNKS];
@@ -432,9 +445,50 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
         return;
     }
 #endif
+    const BuildKernelArgs &kernel = args.kernel;
+    if constexpr (EPILOGUE == GW_EPILOGUE_GRADIENT_L2) {
+        // A lane holds, of every 32 x 32 tile, one row r of b (its lane number modulo 32) and 16 m in 4 runs of 4.
+        const bool full = m_valid >= GW_TILE && n_valid >= GW_TILE;
+        float *c_tile = kernel.c + batch * kernel.c_bs + (i64)n0 * kernel.c_ld + m0;
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+            const int r_local = wave_n + nt * 32 + i;
+            if (!full && r_local >= n_valid) continue;
+            const int r = n0 + r_local;
+            const int o = r / args.gradient_n, n = r - o * args.gradient_n;
+            const float unscale_b = lds_unscale_b[r_local];
+            const float shift = args.gradient_shift[batch * args.gradient_shift_bs + n];
+            const float *d_row = args.gradient_d + batch * args.gradient_d_bs + (i64)n * args.gradient_d_ld + m0;
+            const float *g_column = args.gradient_g + batch * args.gradient_g_bs + (i64)m0 * args.gradient_g_ld + o;
+            float *row = c_tile + (i64)r_local * kernel.c_ld;
+#pragma unroll
+            for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int m_local = wave_m + mt * 32 + 8 * g + 4 * h;
+                    const float4 unscale_a = *reinterpret_cast<const float4 *>(&lds_unscale_a[m_local]);
+                    const float unscales_a[4] = {unscale_a.x, unscale_a.y, unscale_a.z, unscale_a.w};
+                    float v4[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const bool exists = full || m_local + e < m_valid;
+                        const float d = exists ? d_row[m_local + e] - shift : 0.0f;
+                        const float weight = exists ? g_column[(i64)(m_local + e) * args.gradient_g_ld] : 0.0f;
+                        v4[e] = d * weight - (acc[mt][nt][4 * g + e] * unscales_a[e]) * unscale_b;
+                    }
+                    if (kernel.c_vec && (full || m_local + 3 < m_valid)) {
+                        *reinterpret_cast<float4 *>(row + m_local) = make_float4(v4[0], v4[1], v4[2], v4[3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (m_local + e < m_valid) row[m_local + e] = v4[e];
+                    }
+                }
+        }
+        return;
+    }
     // d^2 = |a|^2 + |b|^2 - 2 a.b, trust check per 128 x 128 part (the unit the repair launch
     // works in; every wave lies inside one part), epilogue, stores.
-    const BuildKernelArgs &kernel = args.kernel;
     const int outer_power = kernel.outer_power;
     const int kernel_type = kernel.kernel_type;
     float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;

@@ -9,6 +9,7 @@
 #include "../host/host_common.hpp"
 #include "launch.hpp"
 #include "gram_f16_wide.hpp"
+#include "norm_gradient_l2_wide.hpp"
 
 namespace kmc_host {
 
@@ -72,6 +73,25 @@ void place_operand(OperandRegions &r, int rows, bool broadcast, int l, const Wid
     r.unscale = place(cursor, static_cast<int64_t>(r.batches) * r.rows_pad * 4);
 }
 
+// Grid, slices and the regions of both operands in the workspace; tiles_m and tiles_n are set.
+bool place_wide(int m, int n, int k, int l, bool a_once, bool b_once, bool symmetric, WideLayout *layout)
+{
+    int padded = (layout->tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
+    if ((padded - layout->tiles_n) * 8 > layout->tiles_n) padded = layout->tiles_n;
+    if (static_cast<int64_t>(layout->tiles_m) * padded > 0x7fffffff) return false;
+    layout->tiles_n_padded = padded;
+    layout->slices = (k + kmc::BK_TILE_K - 1) / kmc::BK_TILE_K;
+    // at most 8 ranges of K per row: enough workgroups for the row kernels, few partial sums
+    layout->slices_per_range = layout->slices / 8 > 8 ? (layout->slices + 7) / 8 : 8;
+    layout->ranges = (layout->slices + layout->slices_per_range - 1) / layout->slices_per_range;
+    int64_t cursor = 0;
+    place_operand(layout->a, m, a_once, l, *layout, cursor);
+    if (symmetric) layout->b = layout->a;      // one panel, split once
+    else place_operand(layout->b, n, b_once, l, *layout, cursor);
+    layout->bytes = cursor;
+    return true;
+}
+
 bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, WideLayout *layout)
 {
     if (!(p->flags & KMC_FLAG_L2_GRAM_BF16)) return false;
@@ -83,22 +103,9 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
     const int64_t tiles = args.symmetric ? static_cast<int64_t>(layout->tiles_m) * (layout->tiles_m + 1) / 2
                                          : static_cast<int64_t>(layout->tiles_m) * layout->tiles_n;
     if (!wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k)) return false;
-    int padded = (layout->tiles_n + kmc::BK_XCDS - 1) / kmc::BK_XCDS * kmc::BK_XCDS;
-    if ((padded - layout->tiles_n) * 8 > layout->tiles_n) padded = layout->tiles_n;
-    if (static_cast<int64_t>(layout->tiles_m) * padded > 0x7fffffff) return false;
-    layout->tiles_n_padded = padded;
-    layout->slices = (args.k + kmc::BK_TILE_K - 1) / kmc::BK_TILE_K;
-    // at most 8 ranges of K per row: enough workgroups for the row kernels, few partial sums
-    layout->slices_per_range = layout->slices / 8 > 8 ? (layout->slices + 7) / 8 : 8;
-    layout->ranges = (layout->slices + layout->slices_per_range - 1) / layout->slices_per_range;
-    int64_t cursor = 0;
     // an operand that is the same for every batch entry is split once, unless the centre differs
     const bool one_centre = !args.centre || args.centre_bs == 0;
-    place_operand(layout->a, args.m, args.a_bs == 0 && one_centre, args.l, *layout, cursor);
-    if (args.symmetric) layout->b = layout->a;      // one panel, split once
-    else place_operand(layout->b, args.n, args.b_bs == 0 && one_centre, args.l, *layout, cursor);
-    layout->bytes = cursor;
-    return true;
+    return place_wide(args.m, args.n, args.k, args.l, args.a_bs == 0 && one_centre, args.b_bs == 0 && one_centre, args.symmetric, layout);
 }
 
 kmc::GramRowsArgs rows_args(const float *x, int64_t ld, int64_t bs, int rows, int majorness, bool scalar_only,
@@ -182,6 +189,148 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     }
     if (status == hipSuccess) *taken = true;
     return status;
+}
+
+// ---- the gradient of the L2 norm as one product of pieces (norm_gradient_l2_wide.hpp) ----
+
+namespace {
+
+struct GradientL2Layout {
+    WideLayout wide;                 // a: the columns m of a; b: the rows (o, n) of the products
+    int products_ld;
+    int64_t products, shift, c_transposed, g;      // byte offsets behind the regions of `wide`
+    int64_t bytes;
+};
+
+// The route pays where a model of both times says so by 15 %, in microseconds, fitted to sweeps:
+//   fp32 kernels   30 + terms * t(o) with terms = m n k l and t(o) = 0.077, 0.10, 0.126, 0.137 ps for 1 .. 4
+//                  outputs, 0.028 o up to 8 (vector kernels), 0.27 up to 16, 0.56 up to 32, 0.0175 o beyond
+//                  (matrix-core kernels: a run of outputs costs what its 16 or 32 columns cost);
+//   this route     200 + 1.5e-6 (o n + m) k l for the products and the two splits, and for the walk
+//                  6.3e-9 per multiply-add of the padded tiles (1.7 us per 256 x 256 x 16 step of a CU with the
+//                  chip full) but not less than 0.056 k (a CU alone walks a step in 0.9 us).
+// Examples (fp32 / this route, measured): 8192 x 512 x 16 x 8192 2.7; o = 1 .. 8 there 2.8 .. 4.0; n = 64 1.75,
+// n = 32 0.96, n = 8 0.81; m = 1024 1.55, m = 512 0.86; k = 512 1.35, k = 256 0.92, k = 64 0.40;
+// 10000 x 1000 x 10 x 784 2.6.  KERMAC_AMD_GRADIENT_L2_MIN_TERMS replaces the rule by a number of terms
+// (read on every call, so that a test can send small shapes down the route).
+bool gradient_l2_pays(const kmc_norm_gradient_params *p, int64_t tiles_m, int64_t tiles_n)
+{
+    const char *text = std::getenv("KERMAC_AMD_GRADIENT_L2_MIN_TERMS");
+    const double forced = text ? std::atof(text) : 0.0;
+    const double terms = static_cast<double>(p->m) * p->n * p->k * p->l;
+    if (forced > 0.0) return terms >= forced;
+    const int o = p->o;
+    const double per_term = o == 1 ? 0.077 : o == 2 ? 0.10 : o == 3 ? 0.126 : o == 4 ? 0.137 : o <= 8 ? 0.028 * o
+                          : o <= 16 ? 0.27 : o <= 32 ? 0.56 : 0.0175 * o;
+    const double fp32_us = 30.0 + terms * per_term * 1e-6;
+    const double padded = static_cast<double>(tiles_m) * tiles_n * kmc::GW_TILE * kmc::GW_TILE * p->k * p->l;
+    const double walk_us = padded * 6.3e-9 > 0.056 * p->k ? padded * 6.3e-9 : 0.056 * p->k;
+    const double route_us = 200.0 + 1.5e-6 * (static_cast<double>(o) * p->n + p->m) * p->k * p->l + walk_us;
+    return 1.15 * route_us < fp32_us;
+}
+
+bool gradient_l2_layout(const kmc_norm_gradient_params *p, GradientL2Layout *layout)
+{
+    if (p->norm_type != KMC_NORM_L2 || p->m < 1 || p->n < 1 || p->o < 1 || p->k < 1 || p->l < 1) return false;
+    // row r = o * n_rows + n of the product is row n of plane o of e
+    if (p->o > 1 && p->e_ld_o != static_cast<int64_t>(p->n) * p->e_ld_n) return false;
+    const int64_t rows = static_cast<int64_t>(p->o) * p->n;
+    if (rows > 0x7fffffff - kmc::GW_TILE) return false;
+    WideLayout &wide = layout->wide;
+    wide.tiles_m = (p->m + kmc::GW_TILE - 1) / kmc::GW_TILE;
+    wide.tiles_n = static_cast<int>((rows + kmc::GW_TILE - 1) / kmc::GW_TILE);
+    if (!gradient_l2_pays(p, wide.tiles_m, wide.tiles_n)) return false;
+    if (!place_wide(p->m, static_cast<int>(rows), p->k, p->l, p->a_bs == 0, false, false, &wide)) return false;
+    int64_t cursor = wide.bytes;
+    layout->products_ld = (p->k + 3) / 4 * 4;
+    layout->products = place(cursor, static_cast<int64_t>(p->l) * rows * layout->products_ld * 4);
+    layout->shift = place(cursor, static_cast<int64_t>(p->l) * p->n * 4);
+    layout->c_transposed = place(cursor, static_cast<int64_t>(p->l) * p->k * p->o * 4);
+    layout->g = place(cursor, static_cast<int64_t>(p->l) * p->m * p->o * 4);
+    layout->bytes = cursor;
+    return true;
+}
+
+}  // namespace
+
+int64_t norm_gradient_l2_wide_bytes(const kmc_norm_gradient_params *p)
+{
+    GradientL2Layout layout;
+    return gradient_l2_layout(p, &layout) ? layout.bytes : 0;
+}
+
+// `*taken` says whether the route applied (and the launches were made); if not, nothing was launched.
+int launch_norm_gradient_l2_wide(const kmc_norm_gradient_params *p, hipStream_t stream, bool *taken)
+{
+    *taken = false;
+    GradientL2Layout layout;
+    if (!p->workspace || !gradient_l2_layout(p, &layout) || p->workspace_bytes < layout.bytes ||
+        (reinterpret_cast<uintptr_t>(p->workspace) & (REGION_ALIGN - 1)) != 0)
+        return KMC_OK;
+    char *workspace = static_cast<char *>(p->workspace);
+    const WideLayout &wide = layout.wide;
+    const int rows = p->o * p->n;
+    const bool scalar_only = (p->flags & KMC_FLAG_FORCE_SCALAR_ACCESS) != 0;
+
+    kmc::GradientL2PrepareArgs prepare = {};
+    prepare.b = p->b; prepare.b_ld = p->b_ld; prepare.b_bs = p->b_bs;
+    prepare.c = p->c; prepare.c_ld = p->c_ld; prepare.c_bs = p->c_bs;
+    prepare.products = reinterpret_cast<float *>(workspace + layout.products);
+    prepare.products_ld = layout.products_ld; prepare.products_bs = static_cast<int64_t>(rows) * layout.products_ld;
+    prepare.shift = reinterpret_cast<float *>(workspace + layout.shift); prepare.shift_bs = p->n;
+    prepare.c_transposed = reinterpret_cast<float *>(workspace + layout.c_transposed);
+    prepare.c_transposed_ld = p->o; prepare.c_transposed_bs = static_cast<int64_t>(p->k) * p->o;
+    prepare.n = p->n; prepare.o = p->o; prepare.k = p->k;
+    hipError_t status = launch(kmc::gradient_l2_products, dim3(p->n, p->l), dim3(kmc::GL2_THREADS), stream, prepare);
+    if (status != hipSuccess) return fail_hip(status, "gradient_l2_products launch");
+    status = launch(kmc::gradient_l2_transpose_c, dim3((p->k + kmc::GL2_THREADS - 1) / kmc::GL2_THREADS, p->l), dim3(kmc::GL2_THREADS), stream, prepare);
+    if (status != hipSuccess) return fail_hip(status, "gradient_l2_transpose_c launch");
+
+    // g[m][o] = sum_k a[k][m] c[o][k]: a is a stored panel with m contiguous
+    float *g = reinterpret_cast<float *>(workspace + layout.g);
+    kmc_matrix_coefficients_params weights = {};
+    weights.m = p->m; weights.n = p->k; weights.o = p->o; weights.l = p->l;
+    weights.matrix = p->a; weights.matrix_ld = p->a_ld; weights.matrix_bs = p->a_bs;
+    weights.coef = prepare.c_transposed; weights.coef_ld = prepare.c_transposed_ld; weights.coef_bs = prepare.c_transposed_bs;
+    weights.out = g; weights.out_ld = p->o; weights.out_bs = static_cast<int64_t>(p->m) * p->o;
+    const int contracted = kmc_matrix_times_coefficients(&weights, stream);
+    if (contracted != KMC_OK) return contracted;
+
+    // no centre: the shift of b is in the products already
+    kmc::BuildKernelArgs walk = {};
+    walk.m = p->m; walk.n = rows; walk.k = p->k; walk.l = p->l;
+    const kmc::GramRowsArgs rows_a = rows_args(p->a, p->a_ld, p->a_bs, p->m, KMC_COL_MAJOR, scalar_only, walk, wide, wide.a, workspace);
+    const kmc::GramRowsArgs rows_b = rows_args(prepare.products, prepare.products_ld, prepare.products_bs, rows, KMC_ROW_MAJOR, scalar_only,
+                                               walk, wide, wide.b, workspace);
+    status = launch_gram_rows(rows_a, wide.a.batches, stream);
+    if (status == hipSuccess) status = launch_gram_rows(rows_b, wide.b.batches, stream);
+    if (status != hipSuccess) return fail_hip(status, "gram_row_stats / gram_f16_split launch");
+
+    kmc::GramWideArgs product = {};
+    product.kernel = walk;
+    product.kernel.c = p->e; product.kernel.c_ld = p->e_ld_n; product.kernel.c_bs = p->e_bs;
+    product.kernel.c_vec = !scalar_only && aligned16(p->e) && p->e_ld_n % 4 == 0 && p->e_bs % 4 == 0;
+    product.pieces_a = rows_a.pieces; product.pieces_b = rows_b.pieces;
+    product.pieces_a_bs = wide.a.batches > 1 ? wide.a.pieces_bs : 0;
+    product.pieces_b_bs = wide.b.batches > 1 ? wide.b.pieces_bs : 0;
+    product.squares_a = rows_a.squares; product.squares_b = rows_b.squares;
+    product.stats_a_bs = wide.a.batches > 1 ? wide.a.stats_bs : 0;
+    product.stats_b_bs = wide.b.batches > 1 ? wide.b.stats_bs : 0;
+    product.unscale_a = rows_a.unscale; product.unscale_b = rows_b.unscale;
+    product.unscale_a_bs = wide.a.batches > 1 ? wide.a.rows_pad : 0;
+    product.unscale_b_bs = wide.b.batches > 1 ? wide.b.rows_pad : 0;
+    product.rows_pad_a = wide.a.rows_pad; product.rows_pad_b = wide.b.rows_pad;
+    product.slices = wide.slices; product.ranges = wide.ranges;
+    product.wide_tiles_m = wide.tiles_m; product.wide_tiles_n = wide.tiles_n; product.wide_tiles_n_padded = wide.tiles_n_padded;
+    product.gradient_d = p->d; product.gradient_d_ld = p->d_ld; product.gradient_d_bs = p->d_bs;
+    product.gradient_g = g; product.gradient_g_ld = p->o; product.gradient_g_bs = weights.out_bs;
+    product.gradient_shift = prepare.shift; product.gradient_shift_bs = prepare.shift_bs;
+    product.gradient_n = p->n;
+    const dim3 grid(static_cast<unsigned>(wide.tiles_m) * wide.tiles_n_padded, p->l, 1);
+    status = launch(kmc::gram_f16_wide<false, kmc::GW_EPILOGUE_GRADIENT_L2>, grid, dim3(kmc::GW_THREADS), stream, product);
+    if (status != hipSuccess) return fail_hip(status, "gram_f16_wide (gradient) launch");
+    *taken = true;
+    return KMC_OK;
 }
 
 }  // namespace kmc_host

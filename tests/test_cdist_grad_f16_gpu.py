@@ -59,7 +59,8 @@ def test_when_the_route_applies(device, monkeypatch):
     c = torch.empty(16, 2048, device=device)
     d = torch.empty(512, 4096, device=device)
     assert workspace_bytes(a, b, c, d) > 0                                   # 4.3e9 terms
-    assert workspace_bytes(a, b, c, d, p=2.0) == 0 and workspace_bytes(a, b, c, d, p=1.3) == 0
+    assert workspace_bytes(a, b, c, d, p=1.3) == 0
+    assert workspace_bytes(a, b, c, d, p=2.0) not in (0, workspace_bytes(a, b, c, d))         # the L2 norm has a route of its own
     assert workspace_bytes(a[:, :256], b[:64], c, d[:64, :256]) == 0         # 3.4e7 terms
     assert workspace_bytes(a, b, c[:2], d) == 0                              # two outputs: the vector kernel
     needed = workspace_bytes(a, b, c, d)

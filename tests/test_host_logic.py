@@ -499,7 +499,14 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
         return _backend.norm_gradient_workspace_bytes(grad)
 
     assert gradient(8192, 512, 16, 8192) > 4 * 8192 * 8192                           # the pieces of a alone
-    assert gradient(8192, 512, 16, 8192, norm_type=1) == 0 and gradient(8192, 512, 16, 8192, norm_type=2) == 0
+    assert gradient(8192, 512, 16, 8192, norm_type=2) == 0
+    # the L2 norm: one product of (o n) x k by k x m on the fp16 matrix instruction, by a model of both times
+    monkeypatch.delenv("KERMAC_AMD_GRADIENT_L2_MIN_TERMS", raising=False)
+    assert gradient(8192, 512, 16, 8192, norm_type=1) > 3 * 4 * 8192 * 8192          # c b in fp32 and in pieces, the pieces of a
+    assert gradient(8192, 512, 16, 256, norm_type=1) == 0                            # a short contraction
+    assert gradient(8192, 8, 16, 8192, norm_type=1) == 0                             # 32 x 1 tiles
+    assert gradient(512, 512, 16, 8192, norm_type=1) == 0                            # 2 x 32 tiles
+    assert gradient(8192, 512, 1, 8192, norm_type=1) > 0                             # one output: the fp32 kernel is slow there
     assert gradient(8192, 512, 2, 8192) == 0                                         # two outputs: the vector kernel
     assert gradient(1024, 64, 16, 1024) == 0                                         # 6.7e7 terms
     assert gradient(8192, 16, 16, 8192) == 0                                         # half of every tile of 32 columns unused

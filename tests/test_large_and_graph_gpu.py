@@ -178,12 +178,13 @@ def test_operators_replay_from_a_hip_graph(device):
 
 def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
     """The routes that go through a workspace allocated by the Python layer (squared differences on
-    the fp16 matrix instruction: centre, row statistics, split, product, repair; the L1 gradient on
-    the fp16 matrix instruction) captured into one graph: the workspace comes from the graph's memory
+    the fp16 matrix instruction: centre, row statistics, split, product, repair; the L1 and L2
+    gradients on the fp16 matrix instruction) captured into one graph: the workspace comes from the graph's memory
     pool, the decision whether to subtract the centre is taken on the device, and every replay on
     new values equals the eager result bit for bit."""
     monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
     monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
+    monkeypatch.setenv("KERMAC_AMD_GRADIENT_L2_MIN_TERMS", "1")
     monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "4096")         # panels of 256 centres: three here
     g = torch.Generator().manual_seed(77)
     M, N, K, O = 600, 520, 96, 16
@@ -197,6 +198,7 @@ def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
     out_p2 = torch.empty(N, M, device=device)
     out_self = torch.empty(M, M, device=device)
     out_grad = torch.empty(O, K, M, device=device)
+    out_grad_l2 = torch.empty(O, K, M, device=device)
     coefficients = torch.randn(N, 5, generator=g).to(device)
     out_product = torch.empty(1, M, 5, device=device)
 
@@ -208,8 +210,9 @@ def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
             kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, a_store.t(), b_store.t(), out=out_product,
                               bandwidth=10.0, coefficients=coefficients)
         kermac.cdist_grad(weights, centres, classes, samples, out=out_grad, p=1.0)
+        kermac.cdist_grad(weights, centres, classes, samples, out=out_grad_l2, p=2.0)
 
-    outs = (out_p2, out_self, out_grad, out_product)
+    outs = (out_p2, out_self, out_grad, out_product, out_grad_l2)
     side = torch.cuda.Stream(device=device)
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -231,7 +234,7 @@ def test_workspace_routes_replay_from_a_hip_graph(device, monkeypatch):
         graph.replay()
         torch.cuda.synchronize()
         del scratch
-        for name, e, o in zip(("p2", "p2 self", "grad", "product in panels"), eager, outs):
+        for name, e, o in zip(("p2", "p2 self", "grad", "product in panels", "L2 grad"), eager, outs):
             assert torch.equal(e, o), f"replay {replay}: {name} differs from the eager result"
     truth = oracle.cdist(a_store.t().cpu(), b_store.t().cpu(), p=2.0)[0]
     assert_close_to_truth(out_p2.t(), truth, rtol=1e-5, atol=1e-30, what="graph replay vs oracle")

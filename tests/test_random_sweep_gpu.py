@@ -23,11 +23,12 @@ pytestmark = pytest.mark.gpu
 def routes(request, monkeypatch):
     """Every sweep twice: as the library launches these small shapes by itself, and with the routes
     that go through a workspace forced onto them (squared differences, their products with
-    coefficients panel by panel, and the L1 gradient on the fp16 matrix instruction, which by
-    themselves only take large problems)."""
+    coefficients panel by panel, and the L1 and L2 gradients on the fp16 matrix instruction, which
+    by themselves only take large problems)."""
     if request.param == "workspace routes":
         monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
         monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
+        monkeypatch.setenv("KERMAC_AMD_GRADIENT_L2_MIN_TERMS", "1")
         monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "4096")     # products in panels of 256 centres
         kermac.set_l2_mode("gram_bf16", min_k=0)
     yield
