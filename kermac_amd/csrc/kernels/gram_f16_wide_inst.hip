@@ -198,7 +198,8 @@ namespace {
 struct GradientL2Layout {
     WideLayout wide;                 // a: the columns m of a; b: the rows (o, n) of the products
     int products_ld;
-    int64_t products, shift, c_transposed, g;      // byte offsets behind the regions of `wide`
+    int g_parts;                     // ranges of k that g is summed in (partial products, then their sum)
+    int64_t products, shift, c_transposed, g, g_partial;      // byte offsets behind the regions of `wide`
     int64_t bytes;
 };
 
@@ -235,7 +236,7 @@ bool gradient_l2_layout(const kmc_norm_gradient_params *p, GradientL2Layout *lay
     // row r = o * n_rows + n of the product is row n of plane o of e
     if (p->o > 1 && p->e_ld_o != static_cast<int64_t>(p->n) * p->e_ld_n) return false;
     const int64_t rows = static_cast<int64_t>(p->o) * p->n;
-    if (rows > 0x7fffffff - kmc::GW_TILE) return false;
+    if (rows > 0x7fffffff - kmc::GW_TILE || (p->o + kmc::GL2_OUTPUTS - 1) / kmc::GL2_OUTPUTS > 65535) return false;
     WideLayout &wide = layout->wide;
     wide.tiles_m = (p->m + kmc::GW_TILE - 1) / kmc::GW_TILE;
     wide.tiles_n = static_cast<int>((rows + kmc::GW_TILE - 1) / kmc::GW_TILE);
@@ -247,6 +248,13 @@ bool gradient_l2_layout(const kmc_norm_gradient_params *p, GradientL2Layout *lay
     layout->shift = place(cursor, static_cast<int64_t>(p->l) * p->n * 4);
     layout->c_transposed = place(cursor, static_cast<int64_t>(p->l) * p->k * p->o * 4);
     layout->g = place(cursor, static_cast<int64_t>(p->l) * p->m * p->o * 4);
+    // kmc_matrix_times_coefficients wants a workgroup per CU: 128 columns m and 32 outputs each
+    const int64_t workgroups = static_cast<int64_t>((p->m + 127) / 128) * ((p->o + 31) / 32) * p->l;
+    int parts = workgroups >= 256 ? 1 : static_cast<int>((256 + workgroups - 1) / workgroups);
+    if (parts > p->k / 512) parts = p->k / 512 > 1 ? p->k / 512 : 1;
+    if (static_cast<int64_t>(parts) * p->l > 65535) parts = 1;
+    layout->g_parts = parts;
+    layout->g_partial = parts > 1 ? place(cursor, static_cast<int64_t>(parts) * p->l * p->m * p->o * 4) : 0;
     layout->bytes = cursor;
     return true;
 }
@@ -281,7 +289,8 @@ int launch_norm_gradient_l2_wide(const kmc_norm_gradient_params *p, hipStream_t 
     prepare.c_transposed = reinterpret_cast<float *>(workspace + layout.c_transposed);
     prepare.c_transposed_ld = p->o; prepare.c_transposed_bs = static_cast<int64_t>(p->k) * p->o;
     prepare.n = p->n; prepare.o = p->o; prepare.k = p->k;
-    hipError_t status = launch(kmc::gradient_l2_products, dim3(p->n, p->l), dim3(kmc::GL2_THREADS), stream, prepare);
+    hipError_t status = launch(kmc::gradient_l2_products, dim3(p->n, (p->o + kmc::GL2_OUTPUTS - 1) / kmc::GL2_OUTPUTS, p->l),
+                               dim3(kmc::GL2_THREADS), stream, prepare);
     if (status != hipSuccess) return fail_hip(status, "gradient_l2_products launch");
     status = launch(kmc::gradient_l2_transpose_c, dim3((p->k + kmc::GL2_THREADS - 1) / kmc::GL2_THREADS, p->l), dim3(kmc::GL2_THREADS), stream, prepare);
     if (status != hipSuccess) return fail_hip(status, "gradient_l2_transpose_c launch");
@@ -293,8 +302,22 @@ int launch_norm_gradient_l2_wide(const kmc_norm_gradient_params *p, hipStream_t 
     weights.matrix = p->a; weights.matrix_ld = p->a_ld; weights.matrix_bs = p->a_bs;
     weights.coef = prepare.c_transposed; weights.coef_ld = prepare.c_transposed_ld; weights.coef_bs = prepare.c_transposed_bs;
     weights.out = g; weights.out_ld = p->o; weights.out_bs = static_cast<int64_t>(p->m) * p->o;
+    if (layout.g_parts > 1) {
+        weights.out = reinterpret_cast<float *>(workspace + layout.g_partial);
+        weights.n_splits = layout.g_parts;
+        weights.out_split_stride = static_cast<int64_t>(p->l) * weights.out_bs;
+    }
     const int contracted = kmc_matrix_times_coefficients(&weights, stream);
     if (contracted != KMC_OK) return contracted;
+    if (layout.g_parts > 1) {
+        kmc::GradientL2SumArgs sum = {};
+        sum.partial = weights.out; sum.sum = g;
+        sum.count = static_cast<int64_t>(p->l) * weights.out_bs; sum.stride = weights.out_split_stride;
+        sum.parts = layout.g_parts;
+        status = launch(kmc::gradient_l2_sum_parts, dim3(static_cast<unsigned>((sum.count + kmc::GL2_THREADS - 1) / kmc::GL2_THREADS)),
+                        dim3(kmc::GL2_THREADS), stream, sum);
+        if (status != hipSuccess) return fail_hip(status, "gradient_l2_sum_parts launch");
+    }
 
     // no centre: the shift of b is in the products already
     kmc::BuildKernelArgs walk = {};

@@ -35,12 +35,16 @@ struct GradientL2PrepareArgs {
 };
 
 constexpr int GL2_THREADS = 256;
+constexpr int GL2_OUTPUTS = 4;       // rows of p per workgroup
 
-// One workgroup per row n of b: its mean (sums in a fixed order), then the o rows of p that belong to it.
+// One workgroup per row n of b and four outputs: the mean of the row (sums in a fixed order, the
+// same in every workgroup of the row), then the rows of p that belong to it.
 __global__ __launch_bounds__(GL2_THREADS) void gradient_l2_products(const GradientL2PrepareArgs args)
 {
     __shared__ float partial[GL2_THREADS];
-    const int n = blockIdx.x, batch = blockIdx.y;
+    const int n = blockIdx.x, batch = blockIdx.z;
+    const int o_begin = blockIdx.y * GL2_OUTPUTS;
+    const int o_end = o_begin + GL2_OUTPUTS < args.o ? o_begin + GL2_OUTPUTS : args.o;
     const float *b_row = args.b + batch * args.b_bs + (i64)n * args.b_ld;
     float sum = 0.0f;
     for (int k = threadIdx.x; k < args.k; k += GL2_THREADS) sum += b_row[k];
@@ -53,14 +57,31 @@ __global__ __launch_bounds__(GL2_THREADS) void gradient_l2_products(const Gradie
     const float mean = partial[0] / (float)args.k;
     // not-a-number or infinite rows: no shift (the product then carries them as the fp32 kernels would)
     const float shift = (mean - mean == 0.0f) ? mean : 0.0f;
-    if (threadIdx.x == 0) args.shift[batch * args.shift_bs + n] = shift;
+    if (threadIdx.x == 0 && blockIdx.y == 0) args.shift[batch * args.shift_bs + n] = shift;
     const float *c = args.c + batch * args.c_bs;
     float *products = args.products + batch * args.products_bs;
     for (int k = threadIdx.x; k < args.k; k += GL2_THREADS) {
         const float centred = b_row[k] - shift;
-        for (int o = 0; o < args.o; ++o)
+        for (int o = o_begin; o < o_end; ++o)
             products[((i64)o * args.n + n) * args.products_ld + k] = c[(i64)o * args.c_ld + k] * centred;
     }
+}
+
+// g = the sum of `parts` partial products, in their order (kmc_matrix_times_coefficients with n_splits)
+struct GradientL2SumArgs {
+    const float *partial;
+    float *sum;
+    i64 count, stride;
+    int parts;
+};
+
+__global__ __launch_bounds__(GL2_THREADS) void gradient_l2_sum_parts(const GradientL2SumArgs args)
+{
+    const i64 at = (i64)blockIdx.x * GL2_THREADS + threadIdx.x;
+    if (at >= args.count) return;
+    float total = args.partial[at];
+    for (int part = 1; part < args.parts; ++part) total += args.partial[part * args.stride + at];
+    args.sum[at] = total;
 }
 
 // c_transposed[k][o] = c[o][k]
