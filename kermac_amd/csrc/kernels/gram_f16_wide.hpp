@@ -97,6 +97,8 @@ struct GramWideArgs {
     int gradient_n;
 };
 
+constexpr int GW_MAX_RANGES = 9;      // ranges of K per row: ceil(slices / 8) up to 71 slices, 8 beyond
+
 constexpr int GW_EPILOGUE_DISTANCE = 0;
 constexpr int GW_EPILOGUE_GRADIENT_L2 = 1;
 
@@ -306,8 +308,14 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
         const int r = of_a ? tid : tid - GW_TILE;
         const float *partial = of_a ? args.squares_a + batch * args.stats_a_bs + m0 + r : args.squares_b + batch * args.stats_b_bs + n0 + r;
         const int pitch = of_a ? args.rows_pad_a : args.rows_pad_b;
+        // all loads first, then the sum in range order: a loop would wait for each load in turn,
+        // eight memory latencies before the first copy of the walk is issued
+        float parts[GW_MAX_RANGES];
+#pragma unroll
+        for (int range = 0; range < GW_MAX_RANGES; range++) parts[range] = range < args.ranges ? partial[(i64)range * pitch] : 0.0f;
         float norm = 0.0f;
-        for (int range = 0; range < args.ranges; range++) norm += partial[(i64)range * pitch];
+#pragma unroll
+        for (int range = 0; range < GW_MAX_RANGES; range++) norm += range < args.ranges ? parts[range] : 0.0f;
         (of_a ? lds_norm_a : lds_norm_b)[r] = norm;
         (of_a ? lds_unscale_a : lds_unscale_b)[r] =
             of_a ? args.unscale_a[batch * args.unscale_a_bs + m0 + r] : args.unscale_b[batch * args.unscale_b_bs + n0 + r];

@@ -84,6 +84,7 @@ bool place_wide(int m, int n, int k, int l, bool a_once, bool b_once, bool symme
     // at most 8 ranges of K per row: enough workgroups for the row kernels, few partial sums
     layout->slices_per_range = layout->slices / 8 > 8 ? (layout->slices + 7) / 8 : 8;
     layout->ranges = (layout->slices + layout->slices_per_range - 1) / layout->slices_per_range;
+    if (layout->ranges > kmc::GW_MAX_RANGES) return false;       // 9 at most by the two lines above
     int64_t cursor = 0;
     place_operand(layout->a, m, a_once, l, *layout, cursor);
     if (symmetric) layout->b = layout->a;      // one panel, split once
