@@ -480,6 +480,31 @@ def main():
         per_p["2.0_a_against_itself"] = {"ms": round(k_ms, 3), "parity_max_rel_err": e, "rtol": 1e-5, "l2_mode": kermac.get_l2_mode(),
                                          "note": "symmetric result on the workspace route: the 256 x 256 tiles on and below the diagonal"}
 
+        # Beside the distances: the same operands through run_kernel with the inner operator DOT (a linear
+        # kernel matrix, a @ b.T), on the route through the workspace and on the direct kernel.
+        log("timing the sum of products (inner operator DOT)")
+        dot = kermac.KernelDescriptor(kermac.InnerOperator.DOT, kermac.PowerType.NOOP, kermac.PowerType.NOOP, kermac.KernelType.NONE)
+
+        def dot_error():
+            truth = a[:64].double() @ b[:96].double().t()
+            scale = a[:64].abs().double() @ b[:96].abs().double().t()
+            return ((out[:64, :96].double() - truth).abs() / scale).max().item()
+
+        _, dot_ms = time_call(lambda: kermac.run_kernel(dot, a, b, out=out), side_steps, 1)
+        dot_err = dot_error()
+        with kermac.l2_mode("direct"):
+            _, dot_direct_ms = time_call(lambda: kermac.run_kernel(dot, a, b, out=out), side_steps, 1)
+            dot_direct_err = dot_error()
+        log(f"  {dot_ms:.2f} ms kernel (max err / sum |a b| {dot_err:.2e}); direct kernel {dot_direct_ms:.2f} ms ({dot_direct_err:.2e})")
+        check_parity("sum of products, max abs err / sum_k |a b|", dot_err, 1e-6)
+        check_parity("sum of products (direct kernel), max abs err / sum_k |a b|", dot_direct_err, 1e-6)
+        per_p["sum_of_products"] = {"ms": round(dot_ms, 3), "parity_max_err_over_sum_of_absolute_terms": dot_err,
+                                    "mfma_tflops": round(3 * 2.0 * M * N * K / dot_ms / 1e9, 2),
+                                    "direct_kernel_ms": round(dot_direct_ms, 3),
+                                    "direct_kernel_parity_max_err_over_sum_of_absolute_terms": dot_direct_err,
+                                    "note": "run_kernel with inner operator DOT: two fp16 pieces per value on the 256 x 256 walk; "
+                                            "no trust check (nothing cancels in a product)"}
+
         # The two other configurations of the path, timed in this same run so that the default invocation
         # covers them: each entry is the line `--workload <name>` prints on its own.
         del out_store, out

@@ -103,7 +103,15 @@ enum kmc_flags {
      * `a` unchanged since; it is not made again.  For callers that build the matrix panel by panel
      * of `b` (the split of `a` is a quarter of the cost of a panel of 2048 rows of b).  Anything
      * else in those fields of the previous call gives a wrong result, not an error. */
-    KMC_FLAG_GRAM_A_KEPT = 64
+    KMC_FLAG_GRAM_A_KEPT = 64,
+    /* kmc_build_kernel, inner_operator DOT with inner_power NOOP (sum_k a b: linear and polynomial
+     * kernels), with gram_workspace: large problems are multiplied on the fp16 matrix instruction
+     * from two fp16 pieces per value and a scale per row, in the 256 x 256 tiles of the route that
+     * KMC_FLAG_L2_GRAM_BF16 describes (kmc_gram_workspace_bytes says which, and how much memory it
+     * wants).  Error below 3 * 2^-22 sum_k |a b|, the size of the rounding of an fp32 sum of
+     * k >= 100 terms; nothing cancels, so nothing is checked or repaired.  Without a workspace, or
+     * for a problem the query reports 0 for, the direct kernel runs. */
+    KMC_FLAG_DOT_PIECES = 128
 };
 
 /*
@@ -161,7 +169,7 @@ typedef struct kmc_build_kernel_params {
      * as it is; kmc_sample_mean writes all of this).  NULL: nothing is subtracted. */
     const float *gram_centre;
     int64_t gram_centre_bs;
-    /* With KMC_FLAG_L2_GRAM_BF16 only (ignored otherwise): device memory the call may use, 256-byte
+    /* With KMC_FLAG_L2_GRAM_BF16 or KMC_FLAG_DOT_PIECES (ignored otherwise): device memory the call may use, 256-byte
      * aligned, of at least the size kmc_gram_workspace_bytes reports for these parameters.  With
      * it, large problems take a faster route in three steps (statistics per row, both operands
      * split once into two fp16 pieces per value in the order the matrix instruction reads them,
@@ -174,7 +182,8 @@ typedef struct kmc_build_kernel_params {
 } kmc_build_kernel_params;
 
 /* Bytes of gram_workspace that kmc_build_kernel would use for these parameters, 0 when it would
- * not use one (no KMC_FLAG_L2_GRAM_BF16, or a problem too small to gain: fewer than 128 tiles of
+ * not use one (neither KMC_FLAG_L2_GRAM_BF16 with squared differences nor KMC_FLAG_DOT_PIECES with
+ * products, or a problem too small to gain: fewer than 128 tiles of
  * 256 x 256 over the batch, k < 64, tiles * k below 147456, fewer tiles within a batch entry than
  * tiles_m * tiles_n >= 2.5 * (tiles_m + tiles_n), or more than 20 % of the tiles' area padding; of
  * a panel against itself the tiles on and below the diagonal count, and the panel is split once).  About 1.1 times the bytes of the

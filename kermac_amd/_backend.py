@@ -29,6 +29,10 @@ ERR_JIT = 4
 COL_MAJOR = 0
 ROW_MAJOR = 1
 
+# enum kmc_inner_operator, enum kmc_power_type (the values the Python mirror tests for)
+OP_DOT = 1
+POW_NOOP = 0
+
 FLAG_FORCE_SCALAR_ACCESS = 1
 FLAG_NEGATE_DIFF = 2
 FLAG_L2_GRAM = 4
@@ -36,6 +40,7 @@ FLAG_GENERIC_POWER = 8
 FLAG_NO_SYMMETRY = 16
 FLAG_L2_GRAM_BF16 = 32
 FLAG_GRAM_A_KEPT = 64
+FLAG_DOT_PIECES = 128
 
 _float_p = c_void_p  # device pointers are passed as integers
 

@@ -427,6 +427,13 @@ def _plan_run_kernel(
             if l2["mode"] == "gram_bf16" or (l2_auto and stats_c is not None):
                 params.flags |= _backend.FLAG_L2_GRAM_BF16
             params.gram_trust = _gram_trust(K, l2)
+    elif (l2["mode"] in ("auto", "gram_bf16") and d._inner_operator is InnerOperator.DOT
+            and d._inner_power is PowerType.NOOP and K >= l2["min_k"] and stats_c is not None):
+        # sums of products (linear and polynomial kernels): large ones on the fp16 matrix instruction from two
+        # fp16 pieces per value, when the library has a use for the workspace that run_kernel offers it
+        l2_auto = l2["mode"] == "auto"
+        if not l2_auto or float(L) * M * N * K >= _L2_AUTO_MIN_TERMS:
+            params.flags |= _backend.FLAG_DOT_PIECES
     params.m, params.n, params.k, params.l = M, N, K, L
     params.a, params.a_ld, params.a_bs = a.data_ptr(), stats_a.leading_dimension_stride, stats_a.batch_stride
     params.b, params.b_ld, params.b_bs = b.data_ptr(), stats_b.leading_dimension_stride, stats_b.batch_stride
@@ -530,15 +537,23 @@ def run_kernel(
                 print(f"(Kermac Debug) Launching kernel: {function_name}")
             _backend.build_kernel_jit(function, block, stream)
 
-    matrix_core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16
+    matrix_core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16 | _backend.FLAG_DOT_PIECES
     if plan.l2_auto and params.flags & matrix_core:
         # a grid that the direct kernel would cut over k (a small result over a long contraction)
         # stays with it: the matrix-core kernels are launched uncut
+        asked = params.flags & matrix_core
         params.flags &= ~matrix_core
         if _cut_over_contraction(params) is None:
-            params.flags |= matrix_core
+            params.flags |= asked
+    if params.flags & _backend.FLAG_DOT_PIECES:
+        # products have no matrix-core kernel beside the route through the workspace: a call the
+        # library has no use for a workspace for is an ordinary call of the direct kernel
+        workspace = _attach_gram_workspace(params, a.device)
+        if workspace is None:
+            params.flags &= ~_backend.FLAG_DOT_PIECES
+        plan.keepalive.append(workspace)
     cut = _cut_over_contraction(params)
-    if params.flags & matrix_core:
+    if params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
         plan.keepalive.append(_attach_gram_centre(params, stream, a.device))
         plan.keepalive.append(_attach_gram_workspace(params, a.device))
     if cut is None:
@@ -638,7 +653,7 @@ def _choose_cut(tiles, K, mirrored, plane_bytes):
 
 def _cut_over_contraction(params):
     """(ranges of k, k per range), or None when the launch goes out as it is."""
-    if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
+    if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16 | _backend.FLAG_DOT_PIECES):
         return None
     tiles = -(-params.m // 128) * -(-params.n // 128)
     if tiles == 0 or params.k < _CUT_MIN_K or not launch_cuts_enabled():

@@ -103,7 +103,7 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
         if (p->l < 1 || p->k < 1 || before_last >= p->k_total || before_last + p->k < p->k_total)
             return fail(KMC_ERR_INVALID_ARGUMENT, "k_total=%d is not covered by l=%d ranges of k=%d, the last one not empty",
                         p->k_total, p->l, p->k);
-        if (p->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16))
+        if (p->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16 | KMC_FLAG_DOT_PIECES))
             return fail(KMC_ERR_INVALID_ARGUMENT, "k_total cannot be combined with the matrix-core flags");
     }
     args->k_total = p->k_total;
@@ -214,6 +214,16 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
     status = require_gfx950();
     if (status != KMC_OK) return status;
     const dim3 grid(static_cast<unsigned>(args.grid_width), args.l, 1);
+    if (params->flags & KMC_FLAG_DOT_PIECES) {
+        if (params->inner_operator != KMC_OP_DOT || params->inner_power != KMC_POW_NOOP)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_DOT_PIECES needs inner_operator DOT and inner_power NOOP");
+        if (params->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16))
+            return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_DOT_PIECES cannot be combined with KMC_FLAG_L2_GRAM");
+        bool wide = false;
+        hipError_t g = launch_gram_f16_wide(params, args, static_cast<hipStream_t>(stream), &wide);
+        if (g != hipSuccess) return fail_hip(g, "gram_f16_wide launches");
+        if (wide) return KMC_OK;
+    }
     if (params->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16)) {
         if (params->inner_operator != KMC_OP_DIFF || params->inner_power != KMC_POW_SQUARE)
             return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L2_GRAM needs inner_operator DIFF and inner_power SQUARE");

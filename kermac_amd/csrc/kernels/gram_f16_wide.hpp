@@ -101,6 +101,7 @@ constexpr int GW_MAX_RANGES = 9;      // ranges of K per row: ceil(slices / 8) u
 
 constexpr int GW_EPILOGUE_DISTANCE = 0;
 constexpr int GW_EPILOGUE_GRADIENT_L2 = 1;
+constexpr int GW_EPILOGUE_DOT = 2;
 
 // The 16 values of row `row` in slice `slice`, centre subtracted; zeros where the row or k does not exist.
 __device__ __forceinline__ void gram_load_row_slice(const GramRowsArgs &args, const float *x, const float *centre, int row,
@@ -275,6 +276,10 @@ __device__ __forceinline__ bool wide_tile_of_workgroup(const GramWideArgs &args,
 // EPILOGUE GW_EPILOGUE_GRADIENT_L2: the same walk as a plain product of the pieces, for the gradient
 // of the L2 norm (norm_gradient_l2_wide.hpp): no norms, no trust check, the epilogue combines the
 // product with d and g as GramWideArgs says.
+//
+// EPILOGUE GW_EPILOGUE_DOT: the inner operator DOT (sum_k a b): the product of the pieces is the
+// value itself, nothing cancels, so there is no trust check and no repair; outer power, kernel
+// function, regularised diagonal and the stores, mirrored ones included, are those of the distance.
 template <bool SYMMETRIC, int EPILOGUE = GW_EPILOGUE_DISTANCE>
 __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs args)
 {
@@ -543,13 +548,18 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
             for (int e = 0; e < 4; e++)
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++) {
-                    const float norms = norms_a[e] + norm_b[nt];
-                    const float d2 = norms + (acc[mt][nt][4 * g + e] * unscales_a[e]) * unscale_b[nt];
-                    // not a number (overflowing squares, NaN data): not trusted either
-                    bool bad = !(d2 >= trust * norms);
-                    if (!full) bad = bad && m_local + e < m_valid && n_local[nt] < n_valid;
-                    distrusted |= __builtin_amdgcn_ballot_w64(bad);
-                    acc[mt][nt][4 * g + e] = fmaxf(d2, 0.0f);
+                    if constexpr (EPILOGUE == GW_EPILOGUE_DOT) {
+                        // unscale_b carries the factor -2 of the distance
+                        acc[mt][nt][4 * g + e] = (acc[mt][nt][4 * g + e] * unscales_a[e]) * (-0.5f * unscale_b[nt]);
+                    } else {
+                        const float norms = norms_a[e] + norm_b[nt];
+                        const float d2 = norms + (acc[mt][nt][4 * g + e] * unscales_a[e]) * unscale_b[nt];
+                        // not a number (overflowing squares, NaN data): not trusted either
+                        bool bad = !(d2 >= trust * norms);
+                        if (!full) bad = bad && m_local + e < m_valid && n_local[nt] < n_valid;
+                        distrusted |= __builtin_amdgcn_ballot_w64(bad);
+                        acc[mt][nt][4 * g + e] = fmaxf(d2, 0.0f);
+                    }
                 }
         }
     auto for_each = [&](auto &&f) {

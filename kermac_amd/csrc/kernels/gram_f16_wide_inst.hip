@@ -95,8 +95,9 @@ bool place_wide(int m, int n, int k, int l, bool a_once, bool b_once, bool symme
 
 bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, WideLayout *layout)
 {
-    if (!(p->flags & KMC_FLAG_L2_GRAM_BF16)) return false;
-    if (p->inner_operator != KMC_OP_DIFF || p->inner_power != KMC_POW_SQUARE) return false;
+    const bool squared_differences = (p->flags & KMC_FLAG_L2_GRAM_BF16) && p->inner_operator == KMC_OP_DIFF && p->inner_power == KMC_POW_SQUARE;
+    const bool products = (p->flags & KMC_FLAG_DOT_PIECES) && p->inner_operator == KMC_OP_DOT && p->inner_power == KMC_POW_NOOP;
+    if (!squared_differences && !products) return false;
     if (args.m < 1 || args.n < 1 || args.l < 1) return false;
     layout->tiles_m = (args.m + kmc::GW_TILE - 1) / kmc::GW_TILE;
     layout->tiles_n = (args.n + kmc::GW_TILE - 1) / kmc::GW_TILE;
@@ -105,7 +106,8 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
                                          : static_cast<int64_t>(layout->tiles_m) * layout->tiles_n;
     if (!wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k)) return false;
     // an operand that is the same for every batch entry is split once, unless the centre differs
-    const bool one_centre = !args.centre || args.centre_bs == 0;
+    // (products have no centre: the caller's parameter block carries none into `args`)
+    const bool one_centre = products || !args.centre || args.centre_bs == 0;
     return place_wide(args.m, args.n, args.k, args.l, args.a_bs == 0 && one_centre, args.b_bs == 0 && one_centre, args.symmetric, layout);
 }
 
@@ -181,12 +183,15 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     wide.rows_pad_a = layout.a.rows_pad; wide.rows_pad_b = layout.b.rows_pad;
     wide.slices = layout.slices; wide.ranges = layout.ranges;
     wide.wide_tiles_m = layout.tiles_m; wide.wide_tiles_n = layout.tiles_n; wide.wide_tiles_n_padded = layout.tiles_n_padded;
+    const bool products = p->inner_operator == KMC_OP_DOT;
     if (args.symmetric) {
         const dim3 grid(static_cast<unsigned>(layout.tiles_m) * (layout.tiles_m + 1) / 2, args.l, 1);
-        status = launch(kmc::gram_f16_wide<true>, grid, dim3(kmc::GW_THREADS), stream, wide);
+        status = products ? launch(kmc::gram_f16_wide<true, kmc::GW_EPILOGUE_DOT>, grid, dim3(kmc::GW_THREADS), stream, wide)
+                          : launch(kmc::gram_f16_wide<true>, grid, dim3(kmc::GW_THREADS), stream, wide);
     } else {
         const dim3 grid(static_cast<unsigned>(layout.tiles_m) * layout.tiles_n_padded, args.l, 1);
-        status = launch(kmc::gram_f16_wide<false>, grid, dim3(kmc::GW_THREADS), stream, wide);
+        status = products ? launch(kmc::gram_f16_wide<false, kmc::GW_EPILOGUE_DOT>, grid, dim3(kmc::GW_THREADS), stream, wide)
+                          : launch(kmc::gram_f16_wide<false>, grid, dim3(kmc::GW_THREADS), stream, wide);
     }
     if (status == hipSuccess) *taken = true;
     return status;

@@ -119,8 +119,11 @@ def run_kernel_coefficients(
     if matrix_core:
         from .build_a_kernel import _attach_gram_centre
         plan.keepalive.append(_attach_gram_centre(kernel, stream, a.device))
-        if aot and _run_in_panels(plan, stream, a.device, debug):
+        if aot and _run_in_panels(plan, stream, a.device, debug, _backend.FLAG_L2_GRAM_BF16):
             return plan.out
+    elif (_products_in_panels(plan) and _backend.build_kernel_has_variant(kernel.inner_operator, kernel.inner_power)
+            and _run_in_panels(plan, stream, a.device, debug, _backend.FLAG_DOT_PIECES)):
+        return plan.out
     ranges = _centre_ranges(plan, three_resident=aot and not matrix_core and plan.O <= 32)
     partial = None
     if ranges > 1:
@@ -145,7 +148,7 @@ def run_kernel_coefficients(
     return plan.out
 
 
-# Squared differences on the matrix cores: the route of kmc_build_kernel through a workspace
+# Squared differences and sums of products on the matrix cores: the route of kmc_build_kernel through a workspace
 # (operands split once into fp16 pieces, 256 x 256 tiles) builds the kernel matrix several times
 # faster than the fused kernel walks it, so a large product is taken panel by panel instead: the
 # kernel matrix of all rows against a few thousand centres is written into a buffer that is
@@ -168,8 +171,23 @@ def _panel_splits(M, O, L, rows):
     return min(max(splits, -(-rows // 4096)), max(1, 65535 // L))
 
 
-def _run_in_panels(plan, stream, device, debug):
-    """The product panel by panel (above); False when this problem stays with the fused kernel."""
+def _products_in_panels(plan):
+    """Sums of products (linear and polynomial kernels) have the same route: as run_kernel decides
+    for a stored matrix, large ones in the l2 modes "auto" and "gram_bf16"."""
+    from .build_a_kernel import _L2_AUTO_MIN_TERMS, _l2_current
+
+    kernel = plan.params.kernel
+    if kernel.inner_operator != _backend.OP_DOT or kernel.inner_power != _backend.POW_NOOP:
+        return False
+    l2 = _l2_current()
+    if l2["mode"] not in ("auto", "gram_bf16") or plan.K < l2["min_k"]:
+        return False
+    return l2["mode"] != "auto" or float(plan.L) * plan.M * plan.N * plan.K >= _L2_AUTO_MIN_TERMS
+
+
+def _run_in_panels(plan, stream, device, debug, route):
+    """The product panel by panel (above); False when this problem stays with the fused kernel.
+    `route`: the flag of kmc_build_kernel's route through a workspace for this descriptor."""
     from .build_a_kernel import _attach_gram_workspace, _l2_current
 
     budget = int(os.environ.get("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", _PANEL_BYTES))
@@ -184,7 +202,7 @@ def _run_in_panels(plan, stream, device, debug):
     panels = -(-N // rows)
     params = plan.params
     block = _backend.BuildKernelParams.from_buffer_copy(params.kernel)
-    block.flags |= _backend.FLAG_L2_GRAM_BF16
+    block.flags |= route
     block.n, block.c, block.c_ld, block.c_bs = rows, 256, ld, rows * ld      # c: any address, for the query
     if _backend.gram_workspace_bytes(block) == 0:
         return False                                             # panels of this shape would not take the fast route
