@@ -108,8 +108,10 @@ enum kmc_flags {
      * kernels), with gram_workspace: large problems are multiplied on the fp16 matrix instruction
      * from two fp16 pieces per value and a scale per row, in the 256 x 256 tiles of the route that
      * KMC_FLAG_L2_GRAM_BF16 describes (kmc_gram_workspace_bytes says which, and how much memory it
-     * wants).  Error below 3 * 2^-22 sum_k |a b|, the size of the rounding of an fp32 sum of
-     * k >= 100 terms; nothing cancels, so nothing is checked or repaired.  Without a workspace, or
+     * wants).  Error below 3 * 2^-22 sum_k |a b| + k * 2^-38 max|a[m]| max|b[n]| (a value below
+     * 2^-28 of the largest of its row is kept to 2^-40 of that largest one, not to 2^-22 of
+     * itself): the size of the rounding of an fp32 sum of k >= 100 terms; nothing cancels, so
+     * nothing is checked or repaired.  Without a workspace, or
      * for a problem the query reports 0 for, the direct kernel runs. */
     KMC_FLAG_DOT_PIECES = 128
 };
@@ -280,7 +282,7 @@ typedef struct kmc_norm_gradient_params {
      * as the data allows): p and a are split once into two fp16 pieces per value with a scale per
      * row and multiplied in 256 x 256 tiles on the fp16 matrix instruction, g comes from the fp32
      * matrix instruction; the workspace also holds p in fp32.  Error of the product from the pieces
-     * below 3 * 2^-22 sum_k |c a (b - s)|.
+     * below 3 * 2^-22 sum_k |c a (b - s)| + k * 2^-38 max_k|a[k][m]| max_k|p[r][k]|.
      * NULL, too small, or a problem for which the query reports 0: the fp32 kernels run. */
     void *workspace;
     int64_t workspace_bytes;
