@@ -540,10 +540,17 @@ def run_kernel(
     matrix_core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16 | _backend.FLAG_DOT_PIECES
     if plan.l2_auto and params.flags & matrix_core:
         # a grid that the direct kernel would cut over k (a small result over a long contraction)
-        # stays with it: the matrix-core kernels are launched uncut
+        # stays with it, unless the route through a workspace takes the call: its 256 x 256 walk is
+        # launched uncut and is the faster of the two from 64 tiles on (4096 x 4096 over K = 4096:
+        # 0.53 ms against 2.4 ms cut), the one-step matrix-core kernels are not
+        # (2048 x 2048 over K = 4096: 0.27 ms on the one-step matrix-core kernel, whose 256 tiles of 128 x 128
+        # give every CU one, against 0.65 ms cut; 1536 x 1536, 144 tiles: 0.25 against 0.38; 1024 x 1024 over
+        # K = 32768, 64 tiles: 10 ms against 1.4)
         asked = params.flags & matrix_core
         params.flags &= ~matrix_core
-        if _cut_over_contraction(params) is None:
+        one_step_fills_the_chip = (asked & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16)
+                                   and -(-params.m // 128) * -(-params.n // 128) >= 128)
+        if _cut_over_contraction(params) is None or one_step_fills_the_chip or _workspace_route_applies(params, asked):
             params.flags |= asked
     if params.flags & _backend.FLAG_DOT_PIECES:
         # products have no matrix-core kernel beside the route through the workspace: a call the
@@ -579,6 +586,18 @@ def _attach_gram_centre(params, stream, device):
                          centre.data_ptr(), width, stream)
     params.gram_centre, params.gram_centre_bs = centre.data_ptr(), (width if batches > 1 else 0)
     return centre
+
+
+def _workspace_route_applies(params, flags):
+    """Whether kmc_build_kernel would take this call through a workspace, given these matrix-core flags."""
+    if os.environ.get("KERMAC_AMD_L2_WORKSPACE", "1") in ("", "0"):
+        return False
+    kept = params.flags
+    params.flags |= flags
+    try:
+        return _backend.gram_workspace_bytes(params) > 0
+    finally:
+        params.flags = kept
 
 
 def _attach_gram_workspace(params, device):

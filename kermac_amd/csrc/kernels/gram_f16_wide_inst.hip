@@ -44,11 +44,17 @@ struct WideLayout {
 //     1290 x 1290 (6 x 6 tiles, 30 % padding) 0.86.  The rule asks for at most 20 % padding.
 // KERMAC_AMD_WIDE_MIN_TILES = t replaces the rule by "at least t tiles" (read on every call, so that
 // a test can send small shapes down the route).
-bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t tiles, int k)
+// Sums of products have no one-step matrix-core kernel to fall back to: the alternative is the direct
+// kernel, which the route beats much earlier (direct / route time: 64 tiles 1.04 .. 1.42 at K = 1024,
+// 0.82 .. 1.04 at K = 512; 256 tiles 1.25 at K = 256, 0.86 at K = 128; 1024 tiles 1.17 .. 1.35 at K = 128,
+// 0.91 .. 1.02 at K = 64; 64 batch entries of 2 x 2 tiles 1.5, 118 x 2 tiles 1.9).
+bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t tiles, int k, bool products)
 {
     const char *text = std::getenv("KERMAC_AMD_WIDE_MIN_TILES");
     const int forced = text ? std::atoi(text) : 0;
     if (forced > 0) return tiles >= forced && k >= 1;
+    if (products)
+        return k >= 128 && tiles >= 64 && tiles * k >= 65536 && 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
     if (k < 64 || tiles < 128 || tiles * k < 147456) return false;
     if (2 * tiles_m * tiles_n < 5 * (tiles_m + tiles_n)) return false;
     return 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
@@ -104,7 +110,7 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
     // a panel against itself: the tiles on and below the diagonal
     const int64_t tiles = args.symmetric ? static_cast<int64_t>(layout->tiles_m) * (layout->tiles_m + 1) / 2
                                          : static_cast<int64_t>(layout->tiles_m) * layout->tiles_n;
-    if (!wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k)) return false;
+    if (!wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k, products)) return false;
     // an operand that is the same for every batch entry is split once, unless the centre differs
     // (products have no centre: the caller's parameter block carries none into `args`)
     const bool one_centre = products || !args.centre || args.centre_bs == 0;

@@ -268,6 +268,17 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
     with kermac.l2_mode("direct"):
         assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0])
     assert_close_to_truth(got, oracle.cdist(x.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, what="auto, long contraction")
+    # results the direct path would cut over k, but large enough for the matrix cores uncut: 256 tiles of
+    # 128 x 128 fill the chip on the one-step kernel, 144 tiles of 256 x 256 take the route through a workspace
+    for rows, depth in ((2048, 2048), (3000, 2048)):
+        x = torch.randn(rows, depth, generator=g).to(device)
+        y = torch.randn(rows, depth, generator=g).to(device)
+        assert module._cut_over_contraction(planned(rows, rows, depth, kermac.kernel_descriptor_l1_norm).params) is not None
+        got = kermac.cdist(x, y, p=2.0)[0]
+        with kermac.l2_mode("gram_bf16"):
+            assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0]), f"{rows} x {rows} x {depth}: expected the matrix cores"
+        truth = torch.cdist(x[:64].double(), y[:64].double(), p=2.0)
+        assert_close_to_truth(got[:64, :64], truth, rtol=1e-5, what="auto, uncut on the matrix cores")
     # a large problem in auto mode equals the explicit split-bf16 mode, near-duplicate tiles included
     g = torch.Generator().manual_seed(6)
     points = torch.randn(4400, 256, generator=g)
