@@ -186,7 +186,7 @@ typedef struct kmc_build_kernel_params {
 /* Bytes of gram_workspace that kmc_build_kernel would use for these parameters, 0 when it would
  * not use one (neither KMC_FLAG_L2_GRAM_BF16 with squared differences nor KMC_FLAG_DOT_PIECES with
  * products, or a problem too small to gain: fewer than 128 tiles of
- * 256 x 256 over the batch, k < 64, tiles * k below 147456, fewer tiles within a batch entry than
+ * 256 x 256 over the batch, k < 64, tiles * k below 147456 with fewer than 768 tiles, fewer tiles within a batch entry than
  * tiles_m * tiles_n >= 2.5 * (tiles_m + tiles_n), or more than 20 % of the tiles' area padding; of
  * a panel against itself the tiles on and below the diagonal count, and the panel is split once).  About 1.1 times the bytes of the
  * operands.  No counterpart in the reference. */

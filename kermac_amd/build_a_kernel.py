@@ -417,11 +417,11 @@ def _plan_run_kernel(
     l2_auto = False
     if (l2["mode"] != "direct" and d._inner_operator is InnerOperator.DIFF
             and d._inner_power is PowerType.SQUARE and K >= l2["min_k"]):
-        # "auto" leaves small problems (launches that take a few tens of microseconds: the two extra
-        # launches of the matrix-core path would show) to the direct kernel, and run_kernel gives it
-        # the calls whose grid it would rather cut over k
+        # "auto": a stored matrix is a candidate for the matrix cores from min_k on, and run_kernel decides
+        # (_auto_matrix_core_flags); the fused coefficient product takes its matrix-core variant from
+        # 5e8 terms on
         l2_auto = l2["mode"] == "auto"
-        if not l2_auto or float(L) * M * N * K >= _L2_AUTO_MIN_TERMS:
+        if not l2_auto or stats_c is not None or float(L) * M * N * K >= _L2_AUTO_MIN_TERMS:
             # also for the fused coefficient product (no out matrix here): it has a matrix-core variant too
             params.flags |= _backend.FLAG_L2_GRAM
             if l2["mode"] == "gram_bf16" or (l2_auto and stats_c is not None):
@@ -432,8 +432,7 @@ def _plan_run_kernel(
         # sums of products (linear and polynomial kernels): large ones on the fp16 matrix instruction from two
         # fp16 pieces per value, when the library has a use for the workspace that run_kernel offers it
         l2_auto = l2["mode"] == "auto"
-        if not l2_auto or float(L) * M * N * K >= _L2_AUTO_MIN_TERMS:
-            params.flags |= _backend.FLAG_DOT_PIECES
+        params.flags |= _backend.FLAG_DOT_PIECES
     params.m, params.n, params.k, params.l = M, N, K, L
     params.a, params.a_ld, params.a_bs = a.data_ptr(), stats_a.leading_dimension_stride, stats_a.batch_stride
     params.b, params.b_ld, params.b_bs = b.data_ptr(), stats_b.leading_dimension_stride, stats_b.batch_stride
@@ -539,19 +538,9 @@ def run_kernel(
 
     matrix_core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16 | _backend.FLAG_DOT_PIECES
     if plan.l2_auto and params.flags & matrix_core:
-        # a grid that the direct kernel would cut over k (a small result over a long contraction)
-        # stays with it, unless the route through a workspace takes the call: its 256 x 256 walk is
-        # launched uncut and is the faster of the two from 64 tiles on (4096 x 4096 over K = 4096:
-        # 0.53 ms against 2.4 ms cut), the one-step matrix-core kernels are not
-        # (2048 x 2048 over K = 4096: 0.27 ms on the one-step matrix-core kernel, whose 256 tiles of 128 x 128
-        # give every CU one, against 0.65 ms cut; 1536 x 1536, 144 tiles: 0.25 against 0.38; 1024 x 1024 over
-        # K = 32768, 64 tiles: 10 ms against 1.4)
         asked = params.flags & matrix_core
         params.flags &= ~matrix_core
-        one_step_fills_the_chip = (asked & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16)
-                                   and -(-params.m // 128) * -(-params.n // 128) >= 128)
-        if _cut_over_contraction(params) is None or one_step_fills_the_chip or _workspace_route_applies(params, asked):
-            params.flags |= asked
+        params.flags |= _auto_matrix_core_flags(params, asked)
     if params.flags & _backend.FLAG_DOT_PIECES:
         # products have no matrix-core kernel beside the route through the workspace: a call the
         # library has no use for a workspace for is an ordinary call of the direct kernel
@@ -586,6 +575,45 @@ def _attach_gram_centre(params, stream, device):
                          centre.data_ptr(), width, stream)
     params.gram_centre, params.gram_centre_bs = centre.data_ptr(), (width if batches > 1 else 0)
     return centre
+
+
+# The l2 mode "auto", from sweeps of the public call over shapes, batches and storage orders
+# (microseconds, direct / matrix cores):
+#   * the route through a workspace wherever the library takes it (kmc_gram_workspace_bytes: large
+#     problems from K = 64 on; 10000 x 10000 x 96 413 / 304, 4096 x 4096 x 4096 2400 cut / 530, 4096 x 4096 x 20000
+#     12500 / 2300), sums of products nowhere else (they have no one-step kernel);
+#   * the one-step kernels from K = 192 on (128 x 128 x 200 65 / 37, 8 x 256 x 256 x 512 141 / 54, 2000 x 2000 x 200
+#     71 / 52; at K = 64 .. 160 the direct kernel is as fast or faster: 4096 x 4096 x 64 59 / 83, 1000 x 30000 x 128
+#     178 / 233, 8 x 1000 x 1000 x 160 67 / 81), unless the direct path would cut the call over k and the
+#     grid is below 128 tiles (1024 x 1024 x 32768: 1400 cut / 10000; 1536 x 1536 x 4096 380 cut / 250), or the
+#     contraction is so long that they trust nothing they compute (K > 18000: every tile would be redone);
+#   * of the one-step kernels the fp32 one for K >= 384 on 128 to 768 tiles (2000 x 2000 x 784 fp32 135 / split 171,
+#     8 x 1000 x 1000 x 3072 634 / 855), the split one otherwise (K = 200: 47 .. 55 / 37 .. 44; 4096 x 4096 x 512 212 / 161;
+#     8 x 256 x 256 x 512, 32 tiles, 69 / 55).
+_AUTO_ONE_STEP_MIN_K = 192
+_AUTO_FP32_MIN_K = 384
+_AUTO_FP32_MIN_TILES = 128
+_AUTO_FP32_MAX_TILES = 768
+
+
+def _auto_matrix_core_flags(params, asked):
+    """Which of the matrix-core flags `asked` (those the descriptor allows) this call gets in the l2 mode "auto"."""
+    if _workspace_route_applies(params, asked):
+        return asked
+    if not asked & _backend.FLAG_L2_GRAM or params.k < _AUTO_ONE_STEP_MIN_K or params.gram_trust >= 1.0:
+        return 0
+    tiles = -(-params.m // 128) * -(-params.n // 128)
+    if tiles < 128:
+        kept = params.flags
+        params.flags &= ~asked                  # the question is what the direct path would do
+        try:
+            if _cut_over_contraction(params) is not None:
+                return 0
+        finally:
+            params.flags = kept
+    if params.k >= _AUTO_FP32_MIN_K and _AUTO_FP32_MIN_TILES <= tiles * params.l <= _AUTO_FP32_MAX_TILES:
+        return _backend.FLAG_L2_GRAM
+    return asked
 
 
 def _workspace_route_applies(params, flags):

@@ -55,7 +55,9 @@ bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t t
     if (forced > 0) return tiles >= forced && k >= 1;
     if (products)
         return k >= 128 && tiles >= 64 && tiles * k >= 65536 && 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
-    if (k < 64 || tiles < 128 || tiles * k < 147456) return false;
+    // (from 768 tiles on the route is as fast as the one-step kernel also for the shortest contractions
+    // it takes, 8192 x 8192 x 64 180 us against 187, and ahead of the direct kernel, 236)
+    if (k < 64 || tiles < 128 || (tiles * k < 147456 && tiles < 768)) return false;
     if (2 * tiles_m * tiles_n < 5 * (tiles_m + tiles_n)) return false;
     return 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
 }
@@ -177,6 +179,12 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
 
     kmc::GramWideArgs wide = {};
     wide.kernel = args;
+    // The caller's trust rule grows with sqrt(k) (the error of a sum of k terms against the norms) and
+    // passes 1 near k = 18000, where it would send every part to the repair launch -- whose own
+    // fp32 sum over k is no better by then (measured at k = 20000 .. 200000: this walk, which rounds once
+    // per 16 k, 4e-7 .. 2e-6 of d for points as far apart as their norms, the direct kernel 5e-6 .. 4e-5).
+    // With a product worth half the norms the two are equally good, so that is where the rule stops.
+    if (wide.kernel.gram_trust > 0.5f) wide.kernel.gram_trust = 0.5f;
     wide.pieces_a = rows_a.pieces; wide.pieces_b = rows_b.pieces;
     wide.pieces_a_bs = layout.a.batches > 1 ? layout.a.pieces_bs : 0;
     wide.pieces_b_bs = layout.b.batches > 1 ? layout.b.pieces_bs : 0;

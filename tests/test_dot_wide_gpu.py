@@ -115,8 +115,8 @@ def test_which_calls_take_the_route(device, monkeypatch):
     for mode, expected in (("direct", False), ("gram", False), ("gram_bf16", True)):
         with kermac.l2_mode(mode):
             assert (bytes_wanted() > 0) == expected, mode
-    small = plan_of(DOT, a[:300], b[:300])
-    assert not small.params.flags & _backend.FLAG_DOT_PIECES                  # 4.6e7 terms: the direct kernel
+    small = plan_of(DOT, a[:300], b[:300])                                    # 4 tiles: the direct kernel
+    assert module._auto_matrix_core_flags(small.params, small.params.flags & _backend.FLAG_DOT_PIECES) == 0
 
 
 def test_without_a_workspace_the_direct_kernel_runs(device, pieces):

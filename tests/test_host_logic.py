@@ -285,6 +285,10 @@ def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
         plan = _plan_run_kernel(descriptor, a, b, None, kw.get("p"), None, None, kw.get("bandwidth"), None, None, 0, 0,
                                 False, require_device=False)
         return plan.params.flags, plan.params.gram_trust
+    # the default mode "auto" marks a stored matrix of squared differences as a candidate; run_kernel decides
+    assert flags(kermac.kernel_descriptor_l2_norm)[0] & _backend.FLAG_L2_GRAM
+    assert flags(kermac.kernel_descriptor_l1_norm)[0] & _backend.FLAG_L2_GRAM == 0
+    kermac.set_l2_mode("direct")
     assert flags(kermac.kernel_descriptor_l2_norm)[0] & _backend.FLAG_L2_GRAM == 0
     kermac.set_l2_mode("gram")
     try:
@@ -314,6 +318,44 @@ def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
     params.inner_power, params.flags, params.l = 1, _backend.FLAG_L2_GRAM, 1
     params.m = params.n = params.k = 0
     _backend.build_kernel(params, 0)          # empty problem: accepted, nothing launched
+
+
+def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
+    """The l2 mode "auto" decides from the parameter block (and the library's answer about its
+    workspace route, which needs no device): the route through a workspace where the library takes
+    it, the one-step kernels from K = 192 on (the fp32 one for long contractions over few tiles),
+    the direct kernel for short contractions, for grids it would rather cut over k, and for
+    contractions so long that the one-step kernels would trust nothing."""
+    from kermac_amd import build_a_kernel as module
+    for name in ("KERMAC_AMD_WIDE_MIN_TILES", "KERMAC_AMD_L2_WORKSPACE", "KERMAC_AMD_NO_CUT"):
+        monkeypatch.delenv(name, raising=False)
+    core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16
+
+    def chosen(m, n, k, l=1, dot=False):
+        params = _backend.BuildKernelParams()
+        params.inner_operator, params.inner_power, params.outer_power = (1, 0, 0) if dot else (0, 2, 3)
+        params.m, params.n, params.k, params.l = m, n, k, l
+        params.a, params.a_ld, params.a_bs = 4096, m, m * k
+        params.b, params.b_ld, params.b_bs = 4096 + 4 * m * k * l, n, n * k
+        params.c, params.c_ld, params.c_bs = 256, m, m * n
+        params.gram_trust = module._gram_trust(k, {"trust": None})
+        return module._auto_matrix_core_flags(params, _backend.FLAG_DOT_PIECES if dot else core)
+
+    assert chosen(128, 128, 200) == core                         # one step, split pieces
+    assert chosen(2000, 2000, 784) == _backend.FLAG_L2_GRAM      # one step, fp32: a long contraction over 256 tiles
+    assert chosen(4096, 4096, 512) == core                       # 1024 tiles: split pieces
+    assert chosen(4096, 4096, 64) == 0 and chosen(1000, 30000, 160) == 0
+    assert chosen(10000, 10000, 96) == core                      # the library's workspace route
+    assert chosen(4096, 4096, 4096) == core                      # ... also where the direct path would cut over k
+    assert chosen(4096, 4096, 20000) == core                     # ... and for contractions the one-step kernels would not trust
+    assert chosen(2000, 2000, 20000) == 0
+    assert chosen(1024, 1024, 32768) == 0                        # 64 tiles: cut over k by the direct path
+    assert chosen(1536, 1536, 4096) == _backend.FLAG_L2_GRAM     # 144 tiles: uncut on the matrix cores
+    assert chosen(256, 256, 512, l=8) == core
+    assert chosen(8192, 4096, 512, dot=True) == _backend.FLAG_DOT_PIECES
+    assert chosen(300, 300, 512, dot=True) == 0
+    monkeypatch.setenv("KERMAC_AMD_L2_WORKSPACE", "0")
+    assert chosen(8192, 4096, 512, dot=True) == 0 and chosen(10000, 10000, 96) == 0 and chosen(10000, 10000, 256) == core
 
 
 def interpret_grad_params(p: _backend.NormGradientParams):

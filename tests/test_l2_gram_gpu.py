@@ -249,12 +249,19 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
         b = torch.empty(N, K, device=device)
         return module._plan_run_kernel(descriptor, a, b, None, kw.get("p"), None, None, kw.get("bandwidth"), None, None, 0, 0, False)
 
+    def chosen(M, N, K, descriptor=kermac.kernel_descriptor_l2_norm, **kw):
+        plan = planned(M, N, K, descriptor, **kw)
+        asked = plan.params.flags & core
+        return module._auto_matrix_core_flags(plan.params, asked) if plan.l2_auto and asked else 0
+
     big = planned(8000, 8000, 128)
     assert big.l2_auto and big.params.flags & core == core and big.params.gram_trust > 0
-    assert planned(500, 500, 128).params.flags & core == 0                       # 3.2e7 terms: direct
+    assert chosen(8000, 8000, 128) == core                                       # the route through a workspace
+    assert chosen(500, 500, 128) == 0                                            # a short contraction: direct
+    assert chosen(500, 500, 256) == core                                         # one step, from K = 192 on
     assert planned(16000, 16000, 32).params.flags & core == 0                    # K below min_k: direct
     assert planned(8000, 8000, 128, kermac.kernel_descriptor_l1_norm).params.flags & core == 0
-    assert planned(8000, 8000, 128, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0).params.flags & core == core
+    assert chosen(8000, 8000, 128, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0) == core
     a = torch.empty(8000, 128, device=device)
     fused = _plan_run_kernel_coefficients(kermac.kernel_descriptor_laplace_l2, a, a, torch.empty(8000, 8, device=device), None,
                                           None, None, None, 2.0, None, None, 0, 0)
@@ -263,19 +270,20 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
     g = torch.Generator().manual_seed(5)
     x = torch.randn(400, 40000, generator=g).to(device)
     y = torch.randn(380, 40000, generator=g).to(device)
-    assert planned(400, 380, 40000).params.flags & core == core
+    assert planned(400, 380, 40000).params.flags & core == core and chosen(400, 380, 40000) == 0
     got = kermac.cdist(x, y, p=2.0)[0]
     with kermac.l2_mode("direct"):
         assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0])
     assert_close_to_truth(got, oracle.cdist(x.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, what="auto, long contraction")
     # results the direct path would cut over k, but large enough for the matrix cores uncut: 256 tiles of
     # 128 x 128 fill the chip on the one-step kernel, 144 tiles of 256 x 256 take the route through a workspace
-    for rows, depth in ((2048, 2048), (3000, 2048)):
+    # (of the one-step kernels the fp32 one here: a long contraction over 256 tiles)
+    for rows, depth, mode in ((2048, 2048, "gram"), (3000, 2048, "gram_bf16")):
         x = torch.randn(rows, depth, generator=g).to(device)
         y = torch.randn(rows, depth, generator=g).to(device)
         assert module._cut_over_contraction(planned(rows, rows, depth, kermac.kernel_descriptor_l1_norm).params) is not None
         got = kermac.cdist(x, y, p=2.0)[0]
-        with kermac.l2_mode("gram_bf16"):
+        with kermac.l2_mode(mode):
             assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0]), f"{rows} x {rows} x {depth}: expected the matrix cores"
         truth = torch.cdist(x[:64].double(), y[:64].double(), p=2.0)
         assert_close_to_truth(got[:64, :64], truth, rtol=1e-5, what="auto, uncut on the matrix cores")

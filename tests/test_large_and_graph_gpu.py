@@ -7,6 +7,7 @@ import pytest
 import torch
 
 import kermac_amd as kermac
+from kermac_amd import _backend
 from oracle import oracle
 from tests.helpers import assert_close_to_truth
 
@@ -271,9 +272,12 @@ def test_cut_launches_replay_from_a_hip_graph(device):
     long_b = torch.rand(90, 3000, generator=g).to(device)
     out_long = torch.empty(150, 90, device=device)
     from kermac_amd import build_a_kernel as kernel_module
-    assert kernel_module._cut_over_contraction(
-        kernel_module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, long_a, long_b, out_long, None, None, None, None,
-                                       None, None, 0, 0, False).params) is not None
+    planned = kernel_module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, long_a, long_b, out_long, None, None, None, None,
+                                             None, None, 0, 0, False).params
+    matrix_cores = planned.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16)
+    assert matrix_cores and kernel_module._auto_matrix_core_flags(planned, matrix_cores) == 0      # two tiles: the direct path
+    planned.flags &= ~matrix_cores
+    assert kernel_module._cut_over_contraction(planned) is not None                                # ... which cuts it over k
 
     def run_all():
         kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x, z, out=out_fused, bandwidth=2.0, coefficients=coef)
