@@ -589,8 +589,12 @@ def _attach_gram_centre(params, stream, device):
 #     contraction is so long that they trust nothing they compute (K > 18000: every tile would be redone);
 #   * of the one-step kernels the fp32 one for K >= 384 on 128 to 768 tiles (2000 x 2000 x 784 fp32 135 / split 171,
 #     8 x 1000 x 1000 x 3072 634 / 855), the split one otherwise (K = 200: 47 .. 55 / 37 .. 44; 4096 x 4096 x 512 212 / 161;
-#     8 x 256 x 256 x 512, 32 tiles, 69 / 55).
+#     8 x 256 x 256 x 512, 32 tiles, 69 / 55);
+#   * the numbers above are for operands with k contiguous, as torch allocates them.  With the rows contiguous
+#     (the kernels' own order) the split kernel stages faster: it is taken from K = 128 on (5000 x 5000 x 128 155 /
+#     119, 30000 x 1500 x 128 242 / 165) and instead of the fp32 one (2500 x 2500 x 1024 fp32 198 / split 137).
 _AUTO_ONE_STEP_MIN_K = 192
+_AUTO_ONE_STEP_MIN_K_ROWS_CONTIGUOUS = 128
 _AUTO_FP32_MIN_K = 384
 _AUTO_FP32_MIN_TILES = 128
 _AUTO_FP32_MAX_TILES = 768
@@ -600,7 +604,10 @@ def _auto_matrix_core_flags(params, asked):
     """Which of the matrix-core flags `asked` (those the descriptor allows) this call gets in the l2 mode "auto"."""
     if _workspace_route_applies(params, asked):
         return asked
-    if not asked & _backend.FLAG_L2_GRAM or params.k < _AUTO_ONE_STEP_MIN_K or params.gram_trust >= 1.0:
+    # operands with the rows contiguous (m or n, the kernels' own order) stage faster in the split kernel
+    rows_contiguous = params.a_majorness == _backend.COL_MAJOR and params.b_majorness == _backend.COL_MAJOR
+    one_step_min_k = _AUTO_ONE_STEP_MIN_K_ROWS_CONTIGUOUS if rows_contiguous else _AUTO_ONE_STEP_MIN_K
+    if not asked & _backend.FLAG_L2_GRAM or params.k < one_step_min_k or params.gram_trust >= 1.0:
         return 0
     tiles = -(-params.m // 128) * -(-params.n // 128)
     if tiles < 128:
@@ -611,7 +618,7 @@ def _auto_matrix_core_flags(params, asked):
                 return 0
         finally:
             params.flags = kept
-    if params.k >= _AUTO_FP32_MIN_K and _AUTO_FP32_MIN_TILES <= tiles * params.l <= _AUTO_FP32_MAX_TILES:
+    if not rows_contiguous and params.k >= _AUTO_FP32_MIN_K and _AUTO_FP32_MIN_TILES <= tiles * params.l <= _AUTO_FP32_MAX_TILES:
         return _backend.FLAG_L2_GRAM
     return asked
 

@@ -331,12 +331,13 @@ def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
         monkeypatch.delenv(name, raising=False)
     core = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16
 
-    def chosen(m, n, k, l=1, dot=False):
+    def chosen(m, n, k, l=1, dot=False, rows_contiguous=False):
         params = _backend.BuildKernelParams()
+        params.a_majorness = params.b_majorness = _backend.COL_MAJOR if rows_contiguous else _backend.ROW_MAJOR
         params.inner_operator, params.inner_power, params.outer_power = (1, 0, 0) if dot else (0, 2, 3)
         params.m, params.n, params.k, params.l = m, n, k, l
-        params.a, params.a_ld, params.a_bs = 4096, m, m * k
-        params.b, params.b_ld, params.b_bs = 4096 + 4 * m * k * l, n, n * k
+        params.a, params.a_ld, params.a_bs = 4096, (m if rows_contiguous else k), m * k
+        params.b, params.b_ld, params.b_bs = 4096 + 4 * m * k * l, (n if rows_contiguous else k), n * k
         params.c, params.c_ld, params.c_bs = 256, m, m * n
         params.gram_trust = module._gram_trust(k, {"trust": None})
         return module._auto_matrix_core_flags(params, _backend.FLAG_DOT_PIECES if dot else core)
@@ -352,6 +353,9 @@ def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
     assert chosen(1024, 1024, 32768) == 0                        # 64 tiles: cut over k by the direct path
     assert chosen(1536, 1536, 4096) == _backend.FLAG_L2_GRAM     # 144 tiles: uncut on the matrix cores
     assert chosen(256, 256, 512, l=8) == core
+    # operands stored with the rows contiguous: the split kernel from K = 128 on, and instead of the fp32 one
+    assert chosen(5000, 5000, 128, rows_contiguous=True) == core and chosen(5000, 5000, 128) == 0
+    assert chosen(2500, 2500, 1024, rows_contiguous=True) == core and chosen(2500, 2500, 1024) == _backend.FLAG_L2_GRAM
     assert chosen(8192, 4096, 512, dot=True) == _backend.FLAG_DOT_PIECES
     assert chosen(300, 300, 512, dot=True) == 0
     monkeypatch.setenv("KERMAC_AMD_L2_WORKSPACE", "0")
