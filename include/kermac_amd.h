@@ -188,7 +188,9 @@ typedef struct kmc_build_kernel_params {
  * products, or a problem too small to gain: fewer than 128 tiles of
  * 256 x 256 over the batch, k < 64, tiles * k below 147456 with fewer than 768 tiles, fewer tiles within a batch entry than
  * tiles_m * tiles_n >= 2.5 * (tiles_m + tiles_n), or more than 20 % of the tiles' area padding; of
- * a panel against itself the tiles on and below the diagonal count, and the panel is split once).  About 1.1 times the bytes of the
+ * a panel against itself the tiles on and below the diagonal count, and the panel is split once;
+ * squared differences of operands that both have k contiguous take the route from 48 tiles, k = 256 and
+ * tiles * k = 36864 on, whatever the shape of a batch entry).  About 1.1 times the bytes of the
  * operands.  No counterpart in the reference. */
 int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes);
 

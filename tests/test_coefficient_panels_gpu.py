@@ -187,7 +187,7 @@ def test_which_calls_go_in_panels(device, monkeypatch, capsys):
     assert in_panels()                                               # 8 x 32 tiles, 1.7e10 terms
     assert in_panels(kermac.kernel_descriptor_laplace_l2)
     assert not in_panels(kermac.kernel_descriptor_laplace_l1)
-    assert not in_panels(rows=a[:512])                               # 2 x 32 tiles: the split is not earned back
+    assert not in_panels(rows=a[:256])                               # 1 x 32 tiles: the split is not earned back
     monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "0")
     assert not in_panels()
     monkeypatch.delenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES")

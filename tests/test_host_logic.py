@@ -343,19 +343,21 @@ def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
         return module._auto_matrix_core_flags(params, _backend.FLAG_DOT_PIECES if dot else core)
 
     assert chosen(128, 128, 200) == core                         # one step, split pieces
-    assert chosen(2000, 2000, 784) == _backend.FLAG_L2_GRAM      # one step, fp32: a long contraction over 256 tiles
+    assert chosen(1500, 1500, 784) == _backend.FLAG_L2_GRAM      # one step, fp32: a long contraction over 144 tiles
+    assert chosen(2000, 2000, 784) == core                       # 64 tiles of 256 x 256, k contiguous: the workspace route
     assert chosen(4096, 4096, 512) == core                       # 1024 tiles: split pieces
     assert chosen(4096, 4096, 64) == 0 and chosen(1000, 30000, 160) == 0
     assert chosen(10000, 10000, 96) == core                      # the library's workspace route
     assert chosen(4096, 4096, 4096) == core                      # ... also where the direct path would cut over k
     assert chosen(4096, 4096, 20000) == core                     # ... and for contractions the one-step kernels would not trust
-    assert chosen(2000, 2000, 20000) == 0
+    assert chosen(1500, 1500, 20000) == 0
     assert chosen(1024, 1024, 32768) == 0                        # 64 tiles: cut over k by the direct path
     assert chosen(1536, 1536, 4096) == _backend.FLAG_L2_GRAM     # 144 tiles: uncut on the matrix cores
     assert chosen(256, 256, 512, l=8) == core
     # operands stored with the rows contiguous: the split kernel from K = 128 on, and instead of the fp32 one
     assert chosen(5000, 5000, 128, rows_contiguous=True) == core and chosen(5000, 5000, 128) == 0
-    assert chosen(2500, 2500, 1024, rows_contiguous=True) == core and chosen(2500, 2500, 1024) == _backend.FLAG_L2_GRAM
+    assert chosen(1500, 1500, 1024, rows_contiguous=True) == core and chosen(1500, 1500, 1024) == _backend.FLAG_L2_GRAM
+    assert chosen(2000, 2000, 784, rows_contiguous=True) == core              # the split one-step kernel there
     assert chosen(8192, 4096, 512, dot=True) == _backend.FLAG_DOT_PIECES
     assert chosen(300, 300, 512, dot=True) == 0
     monkeypatch.setenv("KERMAC_AMD_L2_WORKSPACE", "0")

@@ -275,10 +275,10 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
     with kermac.l2_mode("direct"):
         assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0])
     assert_close_to_truth(got, oracle.cdist(x.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, what="auto, long contraction")
-    # results the direct path would cut over k, but large enough for the matrix cores uncut: 256 tiles of
-    # 128 x 128 fill the chip on the one-step kernel, 144 tiles of 256 x 256 take the route through a workspace
-    # (of the one-step kernels the fp32 one here: a long contraction over 256 tiles)
-    for rows, depth, mode in ((2048, 2048, "gram"), (3000, 2048, "gram_bf16")):
+    # results the direct path would cut over k, but large enough for the matrix cores uncut: 144 tiles of
+    # 128 x 128 on the one-step kernel (36 of 256 x 256 are too few for the route through a workspace; of the
+    # one-step kernels the fp32 one here: a long contraction with k contiguous), 144 tiles of 256 x 256 on that route
+    for rows, depth, mode in ((1500, 2048, "gram"), (3000, 2048, "gram_bf16")):
         x = torch.randn(rows, depth, generator=g).to(device)
         y = torch.randn(rows, depth, generator=g).to(device)
         assert module._cut_over_contraction(planned(rows, rows, depth, kermac.kernel_descriptor_l1_norm).params) is not None

@@ -67,8 +67,12 @@ def test_when_the_route_applies(device, monkeypatch):
         assert workspace_bytes(a, b, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0) > 0
         assert workspace_bytes(a, b, kermac.kernel_descriptor_l1_norm) == 0
         assert 0 < workspace_bytes(a, a) < 0.6 * workspace_bytes(a, a.clone())   # 406 tiles of the triangle; one panel, split once
-        assert workspace_bytes(a[:3500], a[:3500]) == 0                          # 14 * 15 / 2 = 105 tiles of the triangle
-        assert workspace_bytes(a[:2500], b[:2500]) == 0                          # 100 tiles
+        assert workspace_bytes(a[:2500], b[:2500]) > 0                           # 100 tiles, k contiguous: from 48 tiles on
+        assert workspace_bytes(a[:1500], b[:1500]) == 0                          # 36 tiles
+        at, bt = torch.empty(512, 7000, device=device).t(), torch.empty(512, 4000, device=device).t()
+        assert workspace_bytes(at, bt) > 0                                       # rows contiguous: from 128 tiles on
+        assert workspace_bytes(at[:3500], at[:3500]) == 0                        # 14 * 15 / 2 = 105 tiles of the triangle
+        assert workspace_bytes(at[:2500], bt[:2500]) == 0                        # 100 tiles
         assert workspace_bytes(a[:, :32], b[:, :32]) == 0                        # k < 64
         assert workspace_bytes(a[:, :128], b[:, :128]) == 0                      # 320 tiles at k = 128
         assert workspace_bytes(a[:2500].expand(3, 2500, 512), b[:2500].expand(3, 2500, 512)) > 0    # 300 over the batch
