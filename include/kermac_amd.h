@@ -113,7 +113,13 @@ enum kmc_flags {
      * itself): the size of the rounding of an fp32 sum of k >= 100 terms; nothing cancels, so
      * nothing is checked or repaired.  Without a workspace, or
      * for a problem the query reports 0 for, the direct kernel runs. */
-    KMC_FLAG_DOT_PIECES = 128
+    KMC_FLAG_DOT_PIECES = 128,
+    /* With KMC_FLAG_L2_GRAM_BF16 or KMC_FLAG_DOT_PIECES: the route through gram_workspace for a
+     * problem of any size (k >= 1), also where kmc_gram_workspace_bytes would report 0 because the
+     * one-step kernels are faster.  For callers whose alternative is not those kernels: the
+     * product of a kernel matrix with coefficients taken panel by panel competes with the fused
+     * kernel of kmc_kernel_times_coefficients, which walks the matrix several times more slowly. */
+    KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE = 256
 };
 
 /*
@@ -190,7 +196,8 @@ typedef struct kmc_build_kernel_params {
  * tiles_m * tiles_n >= 2.5 * (tiles_m + tiles_n), or more than 20 % of the tiles' area padding; of
  * a panel against itself the tiles on and below the diagonal count, and the panel is split once;
  * squared differences of operands that both have k contiguous take the route from 48 tiles, k = 256 and
- * tiles * k = 36864 on, whatever the shape of a batch entry).  About 1.1 times the bytes of the
+ * tiles * k = 36864 on, whatever the shape of a batch entry, unless m or n is at most 128;
+ * KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE sets the size rules aside).  About 1.1 times the bytes of the
  * operands.  No counterpart in the reference. */
 int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes);
 

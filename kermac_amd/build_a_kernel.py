@@ -198,7 +198,7 @@ def _hyper_parameter(name, value, L, device, require_device):
 #   launches are bound by the result stores, and the direct kernel has the cheaper
 #   epilogue and no repair launch (M = N = 30000, K = 16: 1.2 ms against 2.4 .. 2.6 ms).
 _L2_DEFAULT_MIN_K = 64
-_L2_AUTO_MIN_TERMS = 5e8          # "auto": below L * M * N * K terms the direct kernel is launched
+_L2_AUTO_MIN_TERMS = 5e8          # "auto", coefficient products: a bound of L * M * N * K terms in their rules
 _L2_MODES = ("direct", "gram", "gram_bf16", "auto")
 # The process-wide setting, and per host thread what `l2_mode(...)` blocks have put on top
 # of it: two threads can evaluate squared differences in different modes at the same time.
@@ -417,16 +417,14 @@ def _plan_run_kernel(
     l2_auto = False
     if (l2["mode"] != "direct" and d._inner_operator is InnerOperator.DIFF
             and d._inner_power is PowerType.SQUARE and K >= l2["min_k"]):
-        # "auto": a stored matrix is a candidate for the matrix cores from min_k on, and run_kernel decides
-        # (_auto_matrix_core_flags); the fused coefficient product takes its matrix-core variant from
-        # 5e8 terms on
+        # "auto": a candidate for the matrix cores from min_k on; run_kernel decides for a stored matrix
+        # (_auto_matrix_core_flags), run_kernel_coefficients for the coefficient product (no out matrix
+        # here), whose fused kernel has a matrix-core variant too
         l2_auto = l2["mode"] == "auto"
-        if not l2_auto or stats_c is not None or float(L) * M * N * K >= _L2_AUTO_MIN_TERMS:
-            # also for the fused coefficient product (no out matrix here): it has a matrix-core variant too
-            params.flags |= _backend.FLAG_L2_GRAM
-            if l2["mode"] == "gram_bf16" or (l2_auto and stats_c is not None):
-                params.flags |= _backend.FLAG_L2_GRAM_BF16
-            params.gram_trust = _gram_trust(K, l2)
+        params.flags |= _backend.FLAG_L2_GRAM
+        if l2["mode"] == "gram_bf16" or (l2_auto and stats_c is not None):
+            params.flags |= _backend.FLAG_L2_GRAM_BF16
+        params.gram_trust = _gram_trust(K, l2)
     elif (l2["mode"] in ("auto", "gram_bf16") and d._inner_operator is InnerOperator.DOT
             and d._inner_power is PowerType.NOOP and K >= l2["min_k"] and stats_c is not None):
         # sums of products (linear and polynomial kernels): large ones on the fp16 matrix instruction from two
@@ -589,7 +587,8 @@ def _attach_gram_centre(params, stream, device):
 #     contraction is so long that they trust nothing they compute (K > 18000: every tile would be redone);
 #   * of the one-step kernels the fp32 one for K >= 384 on 128 to 768 tiles (2000 x 2000 x 784 fp32 135 / split 171,
 #     8 x 1000 x 1000 x 3072 634 / 855), the split one otherwise (K = 200: 47 .. 55 / 37 .. 44; 4096 x 4096 x 512 212 / 161;
-#     8 x 256 x 256 x 512, 32 tiles, 69 / 55);
+#     8 x 256 x 256 x 512, 32 tiles, 69 / 55), and for a single row of 128 tiles or more (4 x 100 x 50000
+#     x 784 fp32 558 / split 857, at K = 256 252 / 340);
 #   * the numbers above are for operands with k contiguous, as torch allocates them.  With the rows contiguous
 #     (the kernels' own order) the split kernel stages faster: it is taken from K = 128 on (5000 x 5000 x 128 155 /
 #     119, 30000 x 1500 x 128 242 / 165) and instead of the fp32 one (2500 x 2500 x 1024 fp32 198 / split 137).
@@ -618,8 +617,11 @@ def _auto_matrix_core_flags(params, asked):
                 return 0
         finally:
             params.flags = kept
-    if not rows_contiguous and params.k >= _AUTO_FP32_MIN_K and _AUTO_FP32_MIN_TILES <= tiles * params.l <= _AUTO_FP32_MAX_TILES:
-        return _backend.FLAG_L2_GRAM
+    if not rows_contiguous:
+        if params.k >= _AUTO_FP32_MIN_K and _AUTO_FP32_MIN_TILES <= tiles * params.l <= _AUTO_FP32_MAX_TILES:
+            return _backend.FLAG_L2_GRAM
+        if min(params.m, params.n) <= 128 and tiles * params.l >= _AUTO_FP32_MIN_TILES:      # one long row of tiles
+            return _backend.FLAG_L2_GRAM
     return asked
 
 

@@ -54,13 +54,14 @@ struct WideLayout {
 // and whatever the shape of a batch entry (one-step / route time: 64 tiles 1.2 at K = 784, 1.5 at K = 3072, also
 // as 16 entries of 2 x 2 tiles with a third of the tiles padding; 144 tiles 1.1 at K = 256, 1.8 at K = 784;
 // 2 x 118 tiles 1.07 at K = 256, 1.3 at K = 784; 36 tiles 0.9 / 1.2; 32 tiles as 8 entries of 2 x 2 0.75 / 0.8;
-// K = 128 never above 1).
+// K = 128 never above 1).  Not for a dimension that half a tile holds, where the 128 x 128 tiles of the
+// one-step kernels waste half as much (100 x 50000: 0.87 at K = 784, 4 entries 0.73; 128 x 20000 0.8).
 bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t tiles, int k, bool products, bool k_contiguous)
 {
     const char *text = std::getenv("KERMAC_AMD_WIDE_MIN_TILES");
     const int forced = text ? std::atoi(text) : 0;
     if (forced > 0) return tiles >= forced && k >= 1;
-    if (k_contiguous && !products && k >= 256 && tiles >= 48 && tiles * k >= 36864) return true;
+    if (k_contiguous && !products && k >= 256 && tiles >= 48 && tiles * k >= 36864 && m > kmc::GW_TILE / 2 && n > kmc::GW_TILE / 2) return true;
     if (products)
         return k >= 128 && tiles >= 64 && tiles * k >= 65536 && 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
     // (from 768 tiles on the route is as fast as the one-step kernel also for the shortest contractions
@@ -121,7 +122,8 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
     const int64_t tiles = args.symmetric ? static_cast<int64_t>(layout->tiles_m) * (layout->tiles_m + 1) / 2
                                          : static_cast<int64_t>(layout->tiles_m) * layout->tiles_n;
     const bool k_contiguous = p->a_majorness == KMC_ROW_MAJOR && p->b_majorness == KMC_ROW_MAJOR;
-    if (!wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k, products, k_contiguous)) return false;
+    const bool asked_for = (p->flags & KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE) && args.k >= 1;
+    if (!asked_for && !wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k, products, k_contiguous)) return false;
     // an operand that is the same for every batch entry is split once, unless the centre differs
     // (products have no centre: the caller's parameter block carries none into `args`)
     const bool one_centre = products || !args.centre || args.centre_bs == 0;

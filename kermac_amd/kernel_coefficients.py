@@ -21,7 +21,7 @@ from .module_cache.module_cache import ModuleCache, kernel_coefficients_function
 
 
 class _CoefPlan:
-    __slots__ = ("params", "out", "keepalive", "L", "M", "N", "K", "O")
+    __slots__ = ("params", "out", "keepalive", "L", "M", "N", "K", "O", "l2_auto")
 
 
 def _plan_run_kernel_coefficients(
@@ -92,6 +92,7 @@ def _plan_run_kernel_coefficients(
     plan.params, plan.out = params, out
     plan.keepalive = base.keepalive + [coefficients, out]
     plan.L, plan.M, plan.N, plan.K, plan.O = L, M, N, K, O
+    plan.l2_auto = base.l2_auto
     return plan
 
 
@@ -118,12 +119,18 @@ def run_kernel_coefficients(
     matrix_core = bool(kernel.flags & _backend.FLAG_L2_GRAM)
     if matrix_core:
         from .build_a_kernel import _attach_gram_centre
-        plan.keepalive.append(_attach_gram_centre(kernel, stream, a.device))
-        if aot and _run_in_panels(plan, stream, a.device, debug, _backend.FLAG_L2_GRAM_BF16):
+        panels = _panel_shape(plan, _backend.FLAG_L2_GRAM_BF16) if aot else None
+        if panels is None and plan.l2_auto and not _auto_fused_on_matrix_cores(plan):
+            kernel.flags &= ~(_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16)
+            matrix_core = False
+        else:
+            plan.keepalive.append(_attach_gram_centre(kernel, stream, a.device))
+            if panels is not None and _run_in_panels(plan, panels, stream, a.device, debug):
+                return plan.out
+    elif _products_in_panels(plan) and _backend.build_kernel_has_variant(kernel.inner_operator, kernel.inner_power):
+        panels = _panel_shape(plan, _backend.FLAG_DOT_PIECES)
+        if panels is not None and _run_in_panels(plan, panels, stream, a.device, debug):
             return plan.out
-    elif (_products_in_panels(plan) and _backend.build_kernel_has_variant(kernel.inner_operator, kernel.inner_power)
-            and _run_in_panels(plan, stream, a.device, debug, _backend.FLAG_DOT_PIECES)):
-        return plan.out
     ranges = _centre_ranges(plan, three_resident=aot and not matrix_core and plan.O <= 32)
     partial = None
     if ranges > 1:
@@ -185,31 +192,110 @@ def _products_in_panels(plan):
     return l2["mode"] != "auto" or float(plan.L) * plan.M * plan.N * plan.K >= _L2_AUTO_MIN_TERMS
 
 
-def _run_in_panels(plan, stream, device, debug, route):
-    """The product panel by panel (above); False when this problem stays with the fused kernel.
-    `route`: the flag of kmc_build_kernel's route through a workspace for this descriptor."""
-    from .build_a_kernel import _attach_gram_workspace, _l2_current
+# The matrix-core variant of the fused kernel holds 32 coefficient columns per workgroup where the
+# direct one holds up to 64: with more than 32 columns it computes every distance once more often
+# than the direct kernel and loses what the matrix instruction gains (O = 40: 1.3 .. 1.5 times
+# slower at K = 128 and 256, level at K = 784 and beyond), unless the problem is so small that
+# the additional workgroups find idle CUs (500 x 500 x 256: 71 us against 98).  With at most 32
+# columns it is ahead from K = 192 on at any size (500 x 500 x 256: 71 us against 96), from 5e8
+# terms on also at K = 128; at K = 64 the direct kernel is ahead everywhere (10000 x 10000: 393
+# us against 479).
+_AUTO_FUSED_MIN_K = 128
+_AUTO_FUSED_ANY_SIZE_MIN_K = 192
+_AUTO_FUSED_MAX_COLUMNS = 32
+_AUTO_FUSED_SMALL_ELEMENTS = 4e6
+
+
+def _auto_fused_on_matrix_cores(plan):
+    """l2 mode "auto", a product that stays with the fused kernel: its matrix-core variant or the direct one."""
+    from .build_a_kernel import _L2_AUTO_MIN_TERMS
+
+    elements = float(plan.L) * plan.M * plan.N
+    if plan.K < _AUTO_FUSED_MIN_K:
+        return False
+    if plan.O > _AUTO_FUSED_MAX_COLUMNS:
+        return plan.K >= _AUTO_FUSED_ANY_SIZE_MIN_K and elements <= _AUTO_FUSED_SMALL_ELEMENTS
+    return plan.K >= _AUTO_FUSED_ANY_SIZE_MIN_K or elements * plan.K >= _L2_AUTO_MIN_TERMS
+
+
+# The rule of kmc_gram_workspace_bytes weighs the route through a workspace against the one-step kernels
+# of a stored matrix.  Here the alternative is the fused kernel, which walks the matrix several times
+# more slowly, so in "auto" squared differences are taken in panels (KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE) also
+# for (fused kernel / panels, the faster of the fused variants):
+#   - long contractions of any number of tiles (K = 3072: 4 tiles 1.4, 16 tiles 1.35, 64 tiles 1.3 .. 1.4,
+#     with O = 40 1.4 .. 2.0; K = 784: 0.95 .. 1.05);
+#   - from 192 tiles on at K >= 256 whatever the storage order (256 tiles 1.06 .. 1.24, 316 tiles 1.3;
+#     64 tiles 0.6);
+#   - more than 32 coefficient columns, where both fused variants pay for them, from K = 784 and 64 tiles
+#     on (64 tiles 1.3, 100 x 50000 1.2 .. 1.3, K = 3072 1.5 .. 2.0), even with most of the tiles padding.
+# The first two need 60 % of the tiles' area used (100 rows against 50000 centres, O = 32: 0.8 .. 0.95).
+# Contractions below 128 stay with the fused kernel (K = 64: 0.83 .. 1.1 at any size).
+_AUTO_PANEL_MIN_K = 128
+_AUTO_PANEL_LONG_K = 1536
+_AUTO_PANEL_MID_K, _AUTO_PANEL_MID_TILES = 256, 192
+_AUTO_PANEL_WIDE_K, _AUTO_PANEL_WIDE_TILES = 784, 64
+_AUTO_PANEL_MIN_USED = 0.6
+
+
+def _auto_panels_of_any_size(plan):
+    tiles_m, tiles_n = -(-plan.M // 256), -(-plan.N // 256)
+    tiles = tiles_m * tiles_n * plan.L
+    used = plan.M * plan.N / (65536.0 * tiles_m * tiles_n)
+    if plan.O > _AUTO_FUSED_MAX_COLUMNS and plan.K >= _AUTO_PANEL_WIDE_K and tiles >= _AUTO_PANEL_WIDE_TILES:
+        return True
+    if used < _AUTO_PANEL_MIN_USED:
+        return False
+    return plan.K >= _AUTO_PANEL_LONG_K or (plan.K >= _AUTO_PANEL_MID_K and tiles >= _AUTO_PANEL_MID_TILES)
+
+
+def _panel_shape(plan, route):
+    """(rows, panels, ld, splits, flags) of the product panel by panel (above); None when this problem
+    stays with the fused kernel.  `route`: the flag of kmc_build_kernel's route through a workspace
+    for this descriptor; `flags`: what the calls for the panels add to the caller's.  No device call."""
+    from .build_a_kernel import _l2_current
 
     budget = int(os.environ.get("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", _PANEL_BYTES))
     L, M, N, O = plan.L, plan.M, plan.N, plan.O
     # l2 mode "gram" asks for the fp32 matrix instruction; the panels are built from fp16 pieces
-    if budget <= 0 or 0 in (L, M, N, O, plan.K) or _l2_current()["mode"] not in ("auto", "gram_bf16"):
-        return False
+    mode = _l2_current()["mode"]
+    if budget <= 0 or 0 in (L, M, N, O, plan.K) or mode not in ("auto", "gram_bf16"):
+        return None
+    if mode == "auto" and plan.K < _AUTO_PANEL_MIN_K:
+        return None
     ld = -(-M // 4) * 4                                          # rows of the panel start on 16 bytes
     rows = min(N, max(256, budget // (4 * L * ld) // 256 * 256))
     panels = -(-N // rows)
     rows = min(N, -(-(-(-N // panels)) // 256) * 256)             # panels of equal size, whole tiles
     panels = -(-N // rows)
-    params = plan.params
-    block = _backend.BuildKernelParams.from_buffer_copy(params.kernel)
+    block = _backend.BuildKernelParams.from_buffer_copy(plan.params.kernel)
     block.flags |= route
     block.n, block.c, block.c_ld, block.c_bs = rows, 256, ld, rows * ld      # c: any address, for the query
     if _backend.gram_workspace_bytes(block) == 0:
-        return False                                             # panels of this shape would not take the fast route
+        # panels of this shape would not take the fast route by themselves
+        if mode != "auto" or route != _backend.FLAG_L2_GRAM_BF16 or not _auto_panels_of_any_size(plan):
+            return None
+        route |= _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
+        block.flags |= route
+        if _backend.gram_workspace_bytes(block) == 0:
+            return None
     splits = _panel_splits(M, O, L, rows)
     parts = panels * splits
     if parts > 1 and 4 * parts * L * M * O > _PANEL_MAX_PARTIAL_BYTES:
-        return False
+        return None
+    return rows, panels, ld, splits, route
+
+
+def _run_in_panels(plan, shape, stream, device, debug):
+    """The product in the panels of `shape` (_panel_shape); False when memory for them is missing."""
+    from .build_a_kernel import _attach_gram_workspace
+
+    rows, panels, ld, splits, route = shape
+    L, M, N, O = plan.L, plan.M, plan.N, plan.O
+    parts = panels * splits
+    params = plan.params
+    block = _backend.BuildKernelParams.from_buffer_copy(params.kernel)
+    block.flags |= route
+    block.n, block.c_ld, block.c_bs = rows, ld, rows * ld
     try:
         panel = torch.empty(L * rows * ld, dtype=torch.float32, device=device)
         partial = torch.empty((parts, L, M, O), dtype=torch.float32, device=device) if parts > 1 else None

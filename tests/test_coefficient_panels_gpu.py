@@ -218,3 +218,25 @@ def test_headline_shape_gaussian(device, capsys):
         d2 = torch.cdist(x[l, :, rows].t().double(), z.t().double(), p=2.0) ** 2
         truth = torch.exp(-d2 / (2 * 9.0 ** 2)) @ coef[l].double()
         assert_close_to_truth(out[l, rows], truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"gaussian slab batch {l}")
+
+
+@pytest.mark.parametrize("M,N,K,O,k_contiguous", [(500, 480, 1600, 5, True), (500, 480, 1600, 5, False),      # a long contraction, 4 tiles
+                                                  (100, 16500, 800, 40, True),                               # 65 tiles, more than 32 columns
+                                                  (2100, 6000, 256, 3, False)])                              # 216 tiles
+def test_auto_mode_takes_panels_where_the_fused_kernel_is_the_slower_one(device, capsys, M, N, K, O, k_contiguous):
+    """The default mode asks for the route through a workspace (KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE) for
+    products that the library's own rule, made for stored matrices, leaves to the one-step kernels."""
+    assert kermac.get_l2_mode() == "auto"
+    g = torch.Generator().manual_seed(M + N + K + O)
+    a = make_operand(1, M, K, not k_contiguous, device, g, batch=False)
+    b = make_operand(1, N, K, not k_contiguous, device, g, batch=False)
+    coef = torch.randn(N, O, generator=g).to(device)
+    bandwidth = float(K) ** 0.5
+    got = kermac.run_kernel(GAUSSIAN, a, b, coefficients=coef, bandwidth=bandwidth, debug=True)
+    assert PANELS in capsys.readouterr().out
+    squared = torch.cdist(a.double(), b.double(), p=2.0) ** 2                 # float64 on the device: the larger cases take the CPU oracle too long
+    truth = torch.exp(-squared / (2 * bandwidth ** 2)) @ coef.double()
+    assert_close_to_truth(got[0], truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"auto panels {M}x{N}x{K}x{O}")
+    with kermac.l2_mode("gram_bf16"):           # the explicit mode follows the library's rule: the fused kernel
+        kermac.run_kernel(GAUSSIAN, a, b, coefficients=coef, bandwidth=bandwidth, debug=True)
+        assert PANELS not in capsys.readouterr().out

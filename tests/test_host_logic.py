@@ -343,6 +343,7 @@ def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
         return module._auto_matrix_core_flags(params, _backend.FLAG_DOT_PIECES if dot else core)
 
     assert chosen(128, 128, 200) == core                         # one step, split pieces
+    assert chosen(100, 50000, 256, l=4) == _backend.FLAG_L2_GRAM   # one long row of tiles: fp32
     assert chosen(1500, 1500, 784) == _backend.FLAG_L2_GRAM      # one step, fp32: a long contraction over 144 tiles
     assert chosen(2000, 2000, 784) == core                       # 64 tiles of 256 x 256, k contiguous: the workspace route
     assert chosen(4096, 4096, 512) == core                       # 1024 tiles: split pieces
@@ -429,7 +430,8 @@ def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
         lines.append(f'  printf("{c_name} size %zu\\n", sizeof(struct {c_name}));')
         for field, _ in binding._fields_:
             lines.append(f'  printf("{c_name} {field} %zu\\n", offsetof(struct {c_name}, {field}));')
-    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16"):
+    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16", "GRAM_A_KEPT",
+                 "DOT_PIECES", "GRAM_WORKSPACE_ANY_SIZE"):
         lines.append(f'  printf("flag {flag} %d\\n", (int)KMC_FLAG_{flag});')
     lines += ['  printf("err WRONG_DEVICE %d\\n", (int)KMC_ERR_WRONG_DEVICE);', "  return 0;", "}"]
     source = tmp_path / "probe.c"
@@ -445,7 +447,8 @@ def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
         assert reported[(c_name, "size")] == ctypes.sizeof(binding), c_name
         for field, _ in binding._fields_:
             assert reported[(c_name, field)] == getattr(binding, field).offset, f"{c_name}.{field}"
-    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16"):
+    for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16", "GRAM_A_KEPT",
+                 "DOT_PIECES", "GRAM_WORKSPACE_ANY_SIZE"):
         assert reported[("flag", flag)] == getattr(_backend, f"FLAG_{flag}")
     assert reported[("err", "WRONG_DEVICE")] == _backend.ERR_WRONG_DEVICE
 
@@ -512,12 +515,13 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     monkeypatch.delenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", raising=False)
     fake = 4096
 
-    def squared_differences(m, n, k, l=1, flags=_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16, same=False):
+    def squared_differences(m, n, k, l=1, flags=_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16, same=False, k_contiguous=False):
         params = _backend.BuildKernelParams()
         params.inner_operator, params.inner_power, params.outer_power = 0, 2, 3      # DIFF, SQUARE, SQRT
         params.m, params.n, params.k, params.l = m, n, k, l
-        params.a, params.a_ld, params.a_bs = fake, m, m * k
-        params.b, params.b_ld, params.b_bs = (fake if same else fake + 4 * m * k * l), n, n * k
+        params.a, params.a_ld, params.a_bs = fake, (k if k_contiguous else m), m * k
+        params.b, params.b_ld, params.b_bs = (fake if same else fake + 4 * m * k * l), (k if k_contiguous else n), n * k
+        params.a_majorness = params.b_majorness = _backend.ROW_MAJOR if k_contiguous else _backend.COL_MAJOR
         params.c_ld, params.c_bs = m, m * n                                          # c stays null: not allocated yet
         params.flags = flags
         return _backend.gram_workspace_bytes(params)
@@ -535,6 +539,18 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert squared_differences(1290, 1290, 1024, l=8) == 0                           # 6 x 6 tiles, 30 % of them padding
     assert squared_differences(1280, 1280, 1024, l=8) > 0
     assert squared_differences(0, 8192, 512) == 0
+    # both operands with k contiguous: from 48 tiles on at k >= 256, whatever the shape of a batch entry,
+    # unless half a tile holds a dimension
+    assert squared_differences(2048, 2048, 1024, k_contiguous=True) > 0
+    assert squared_differences(512, 512, 1024, l=16, k_contiguous=True) > 0
+    assert squared_differences(1500, 1500, 512, k_contiguous=True) == 0              # 36 tiles
+    assert squared_differences(2048, 2048, 128, k_contiguous=True) == 0
+    assert squared_differences(128, 50000, 1024, k_contiguous=True) == 0 and squared_differences(129, 50000, 1024, k_contiguous=True) > 0
+    # the caller's own rule
+    any_size = _backend.FLAG_L2_GRAM_BF16 | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
+    assert squared_differences(300, 200, 5, flags=any_size) > 0
+    assert squared_differences(300, 200, 0, flags=any_size) == 0
+    assert squared_differences(300, 200, 5, flags=_backend.FLAG_L2_GRAM | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE) == 0
     monkeypatch.setenv("KERMAC_AMD_WIDE_MIN_TILES", "1")
     assert squared_differences(300, 200, 5) > 0
 
@@ -561,6 +577,58 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert gradient(2048, 128, 4, 2048) == 0 and gradient(2048, 128, 16, 2048) > 0   # 5.4e8 terms: enough for 16 outputs, not for 4
     monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
     assert gradient(3, 2, 1, 5) > 0
+
+
+def test_auto_mode_of_the_coefficient_product_without_a_gpu(monkeypatch):
+    """l2 mode "auto", run_kernel(..., coefficients=...) of squared differences: panels where the
+    library's rule or the rule for this product takes them, else the matrix-core variant of the
+    fused kernel or the direct one, by K, the number of coefficient columns and the size."""
+    from kermac_amd import kernel_coefficients as module
+    for name in ("KERMAC_AMD_WIDE_MIN_TILES", "KERMAC_AMD_COEFFICIENT_PANEL_BYTES"):
+        monkeypatch.delenv(name, raising=False)
+    assert kermac.get_l2_mode() == "auto"
+    any_size = _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
+
+    def plan(M, N, K, O, L=1, k_contiguous=True, descriptor=kermac.kernel_descriptor_laplace_l2):
+        a = torch.empty(L, M, K) if k_contiguous else torch.empty(L, K, M).transpose(1, 2)
+        b = torch.empty(L, N, K) if k_contiguous else torch.empty(L, K, N).transpose(1, 2)
+        return module._plan_run_kernel_coefficients(descriptor, a, b, torch.empty(L, N, O), None, None, None, None, 2.0,
+                                                    None, None, 0, 0, require_device=False)
+
+    def chosen(*shape, **kw):
+        p = plan(*shape, **kw)
+        assert p.l2_auto and p.params.kernel.flags & _backend.FLAG_L2_GRAM
+        panels = module._panel_shape(p, _backend.FLAG_L2_GRAM_BF16)
+        if panels is not None:
+            return "panels, any size" if panels[4] & any_size else "panels"
+        return "fused, matrix cores" if module._auto_fused_on_matrix_cores(p) else "fused, direct"
+
+    assert chosen(4096, 4096, 256, 32) == "panels"
+    assert chosen(4096, 4096, 256, 32, k_contiguous=False) == "panels, any size"       # 256 tiles
+    assert chosen(4096, 4096, 128, 32, k_contiguous=False) == "fused, matrix cores"    # 256 tiles at K = 128: no panels; 2.1e9 terms
+    assert chosen(4096, 4096, 128, 32, L=4, k_contiguous=False) == "panels"            # 1024 tiles
+    assert chosen(10000, 10000, 64, 32) == "fused, direct"                             # K below 128
+    assert chosen(500, 500, 256, 32) == "fused, matrix cores"
+    assert chosen(500, 500, 128, 32) == "fused, direct"                                # 3.2e7 terms
+    assert chosen(500, 500, 256, 40) == "fused, matrix cores"                          # a small problem: the second chunk of columns runs beside the first
+    assert chosen(500, 500, 3072, 8) == "panels, any size"                             # a long contraction
+    assert chosen(2000, 2000, 784, 32, k_contiguous=False) == "fused, matrix cores"    # 64 tiles
+    assert chosen(2000, 2000, 784, 40, k_contiguous=False) == "panels, any size"
+    assert chosen(100, 50000, 784, 32) == "fused, matrix cores"                        # 61 % of every tile padding
+    assert chosen(100, 50000, 784, 40) == "panels, any size"
+    assert chosen(100, 50000, 256, 40) == "fused, direct"
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "0")
+    assert chosen(4096, 4096, 256, 32) == "fused, matrix cores"
+    assert chosen(4096, 4096, 256, 40) == "fused, direct"
+    monkeypatch.delenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES")
+    with kermac.l2_mode("gram_bf16"):                                                   # the explicit mode: the library's rule alone
+        p = plan(4096, 4096, 256, 32, k_contiguous=False)
+        assert not p.l2_auto and module._panel_shape(p, _backend.FLAG_L2_GRAM_BF16) is None
+        p = plan(8192, 8192, 256, 32, k_contiguous=False)
+        assert module._panel_shape(p, _backend.FLAG_L2_GRAM_BF16)[4] == _backend.FLAG_L2_GRAM_BF16
+    with kermac.l2_mode("direct"):
+        assert plan(4096, 4096, 256, 32).params.kernel.flags & _backend.FLAG_L2_GRAM == 0
+    assert plan(4096, 4096, 256, 32, descriptor=kermac.kernel_descriptor_laplace_l1).params.kernel.flags & _backend.FLAG_L2_GRAM == 0
 
 
 def test_matrix_times_coefficients_checks_its_arguments_before_any_device_call():
