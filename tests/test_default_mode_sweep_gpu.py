@@ -1,0 +1,81 @@
+"""A seeded sweep of mid-size calls in the default l2 mode, no route forced: sizes from a few
+hundred to twenty thousand rows, contractions from 64 to 3200, 1 to 70 coefficient columns, both
+storage orders, padded rows, operands shared by the batch.  Every call takes whatever the rules
+pick for it (direct kernel, one-step matrix-core kernels, the route through a workspace, the cut
+over k, the fused coefficient kernel in either variant, panels), and the result is checked
+against float64 arithmetic on the device (torch.cdist and matmul in float64; the CPU oracle would
+take minutes at these sizes).  Tolerance as everywhere: rtol 1e-5, for sums with coefficients
+plus an absolute floor proportional to the typical magnitude of the sum.
+"""
+import random
+
+import pytest
+import torch
+
+import kermac_amd as kermac
+
+pytestmark = pytest.mark.gpu
+
+GAUSSIAN = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP,
+                                   kermac.KernelType.GAUSSIAN)
+PRODUCTS = kermac.KernelDescriptor(kermac.InnerOperator.DOT, kermac.PowerType.NOOP, kermac.PowerType.NOOP,
+                                   kermac.KernelType.NONE)
+
+
+def operand(rng, device, L, rows, K, col_major, shared):
+    shape = (K, rows) if col_major else (rows, K)
+    if not shared:
+        shape = (L,) + shape
+    pad = rng.choice((0, 0, 4, 3))
+    t = torch.randn(shape[:-1] + (shape[-1] + pad,), device=device)[..., :shape[-1]]
+    return t.transpose(-1, -2) if col_major else t
+
+
+def test_mid_size_calls_as_the_rules_route_them(device):
+    assert kermac.get_l2_mode() == "auto"
+    rng = random.Random(11)
+    torch.manual_seed(11)
+    done = 0
+    while done < 60:
+        L = rng.choice((1, 1, 1, 2, 3))
+        M = rng.choice((rng.randint(60, 300), rng.randint(300, 1500), rng.randint(1500, 5000)))
+        N = rng.choice((rng.randint(100, 600), rng.randint(600, 3000), rng.randint(3000, 20000)))
+        K = rng.choice((rng.randint(64, 200), rng.randint(200, 400), rng.randint(700, 900), rng.randint(1500, 3200)))
+        O = rng.choice((1, 7, 32, 40, 70))
+        if L * M * N * K > 3e10 or L * M * N > 6e7:
+            continue
+        done += 1
+        col_major = rng.random() < 0.4
+        kind = rng.choice(("distances", "gaussian x coefficients", "gaussian x coefficients", "laplace x coefficients", "products"))
+        a = operand(rng, device, L, M, K, col_major, rng.random() < 0.2)
+        b = operand(rng, device, L, N, K, col_major if rng.random() < 0.8 else not col_major, rng.random() < 0.2)
+        what = f"case {done}: {kind}, L={L} M={M} N={N} K={K} O={O}, a {tuple(a.shape)} {a.stride()}, b {tuple(b.shape)} {b.stride()}"
+        print(what, flush=True)
+        with_coefficients = kind.endswith("coefficients")
+        batch = L if with_coefficients or a.dim() == 3 or b.dim() == 3 else 1         # two shared operands: one matrix
+        a64 = (a if a.dim() == 3 else a.unsqueeze(0).expand(batch, -1, -1)).double()
+        b64 = (b if b.dim() == 3 else b.unsqueeze(0).expand(batch, -1, -1)).double()
+        bandwidth = float(K) ** 0.5
+        if kind == "distances":
+            got, truth, atol = kermac.cdist(a, b, p=2.0), torch.cdist(a64, b64, p=2.0), 0.0
+        elif kind == "products":
+            got, truth = kermac.run_kernel(PRODUCTS, a, b), a64 @ b64.transpose(1, 2)
+            atol = 1e-5 * float((a64.abs() @ b64.abs().transpose(1, 2)).mean())
+        else:
+            coef = torch.randn(L, N, O + 1, device=device)[..., :O] / N ** 0.5
+            if kind == "gaussian x coefficients":
+                got = kermac.run_kernel(GAUSSIAN, a, b, coefficients=coef, bandwidth=bandwidth)
+                matrix = torch.exp(-torch.cdist(a64, b64, p=2.0) ** 2 / (2 * bandwidth ** 2))
+            else:
+                got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, a, b, coefficients=coef, bandwidth=bandwidth,
+                                        regularization=0.25, regularization_offset_x=3, regularization_offset_y=1)
+                matrix = torch.exp(-torch.cdist(a64, b64, p=2.0) / bandwidth)
+                m = torch.arange(M, device=device)
+                n = m - 2                                      # the elements with offset_x + n == offset_y + m
+                keep = (n >= 0) & (n < N)
+                matrix[:, m[keep], n[keep]] = 1.25
+            truth = matrix @ coef.double()
+            atol = 1e-5 * float(truth.abs().mean()) * 10
+        assert got.shape == truth.shape, what
+        excess = (got.double() - truth).abs() - (1e-5 * truth.abs() + atol)       # compared on the device: up to 6e7 elements
+        assert bool(torch.isfinite(got).all()) and float(excess.max()) <= 0.0, f"{what}: {float(excess.max()):.3e} beyond the tolerance"
