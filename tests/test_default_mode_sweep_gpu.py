@@ -79,3 +79,41 @@ def test_mid_size_calls_as_the_rules_route_them(device):
         assert got.shape == truth.shape, what
         excess = (got.double() - truth).abs() - (1e-5 * truth.abs() + atol)       # compared on the device: up to 6e7 elements
         assert bool(torch.isfinite(got).all()) and float(excess.max()) <= 0.0, f"{what}: {float(excess.max()):.3e} beyond the tolerance"
+
+
+def test_mid_size_gradients_as_the_rules_route_them(device):
+    """cdist_grad for p = 1 and p = 2 at sizes on both sides of the rules that send a gradient to
+    the fp16 matrix instruction: e[o, n, m] = sum_k c[o, k] a[k, m] w(d[n, m] - b[n, k]), with
+    w = sign for p = 1 and the identity for p = 2, in float64 on the device.  Tolerance of the
+    gradient tests: |got - truth| <= 1e-5 |truth| + 1e-4 mean |truth| (a signed sum of K terms)."""
+    rng = random.Random(12)
+    torch.manual_seed(12)
+    done = 0
+    while done < 24:
+        L = rng.choice((1, 1, 2))
+        M = rng.choice((rng.randint(100, 700), rng.randint(700, 3000), rng.randint(3000, 9000)))
+        N = rng.choice((rng.randint(8, 40), rng.randint(40, 200), rng.randint(200, 600)))
+        O = rng.choice((1, 2, 3, 10, 16, 24, 40))
+        K = rng.choice((rng.randint(64, 300), rng.randint(300, 1500), rng.randint(1500, 9000)))
+        p = rng.choice((1.0, 2.0))
+        if L * M * N * O * K > 6e11 or L * M * N * O > 1.5e8:
+            continue
+        done += 1
+        a = torch.rand(L, K, M, device=device) - 0.3
+        b = torch.randn(L, N, K, device=device)
+        c = torch.randn(L, O, K, device=device)
+        d = torch.randn(L, N, M, device=device)
+        what = f"gradient case {done}: p={p} L={L} M={M} N={N} O={O} K={K}"
+        print(what, flush=True)
+        got = kermac.cdist_grad(a, b, c, d, p=p)
+        assert got.shape == (L, O, N, M), what
+        a64, b64, c64, d64 = a.double(), b.double(), c.double(), d.double()
+        if p == 2.0:
+            truth = d64[:, None] * (c64 @ a64)[:, :, None, :] - torch.einsum("lok,lnk,lkm->lonm", c64, b64, a64)
+        else:
+            truth = torch.empty(L, O, N, M, dtype=torch.float64, device=device)
+            for n in range(N):
+                sign = torch.copysign(torch.ones((), dtype=torch.float64, device=device), d64[:, n, None, :] - b64[:, n, :, None])
+                truth[:, :, n, :] = c64 @ (a64 * sign)           # [L, O, K] @ [L, K, M]
+        excess = (got.double() - truth).abs() - (1e-5 * truth.abs() + 1e-4 * float(truth.abs().mean()))
+        assert bool(torch.isfinite(got).all()) and float(excess.max()) <= 0.0, f"{what}: {float(excess.max()):.3e} beyond the tolerance"
