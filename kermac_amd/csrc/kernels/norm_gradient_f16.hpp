@@ -19,15 +19,15 @@
 // a2 c2 below 2^-22 |a c|: the error of E from the pieces is below 3 * 2^-22 sum_k |c a|, the size
 // of the rounding of an fp32 accumulation over a few terms, beside the fp32 accumulation itself.
 //
-// Workgroup: 4 waves, 64 m x 32 n x 16 o; wave w owns the 8 n  8w .. 8w + 7  and all 64 m as 4 row
-// blocks of 16.  Per 32 k it reads the pieces of C (2 x 16 bytes per lane) and of its A rows
+// Workgroup: 4 waves, 64 m x 32 n x 16 o (for more than 16 outputs 64 m x 16 n x 32 o, below); wave w
+// owns the 8 (4) n  8w .. 8w + 7  and all 64 m as 4 row blocks of 16.  Per 32 k it reads the pieces of C (2 x 16 bytes per lane) and of its A rows
 // (8 x 16 bytes), and per n the 8 values of B that match its 8 k (2 x 16 bytes, the same for the
 // 16 lanes of a row block).  B is copied once into a padded array in the workspace (rows to 32,
 // k to 32 plus what the walk copies ahead), so that everything the walk touches exists and all of
 // it arrives in LDS by global_load_lds_dwordx4, three steps in three buffers, as in
 // gram_f16_wide.hpp (the copies are inline instructions for the reason given there).
 //
-// Measured at M = K = 8192, N = 512, O = 16: 3.86 ms for this kernel and 0.33 ms for the row kernels
+// Measured at M = K = 8192, N = 512, O = 16: 3.86 ms (O = 32 on the second shape: 5.4 ms) for this kernel and 0.33 ms for the row kernels
 // against 9.85 ms on the fp32 kernels.  Counters: 2.5 vector instructions per (m, n, k) (the
 // compiler fuses AND and XOR into v_bitop3_b32), the matrix pipeline busy 46 % and the vector
 // pipeline about 44 % of the elapsed cycles, hardly ever together, shader clock 1.75 GHz.  Tried
@@ -45,19 +45,29 @@ namespace kmc {
 typedef float ngf_float4 __attribute__((ext_vector_type(4)));
 
 constexpr int NGF_TILE_M = 64;
-constexpr int NGF_TILE_N = 32;
-constexpr int NGF_TILE_O = 16;
-constexpr int NGF_WAVE_N = 8;
 constexpr int NGF_STEP_K = 32;                 // two slices of the split
 constexpr int NGF_THREADS = 256;
 constexpr int NGF_AHEAD = 3;                   // steps copied ahead of the walk
-constexpr int NGF_A_CHUNKS = 8 * NGF_TILE_M;   // per step: 8 runs (slice, piece, half) of 64 rows
-constexpr int NGF_C_CHUNKS = 8 * NGF_TILE_O;
-constexpr int NGF_B_CHUNKS = NGF_TILE_N * NGF_STEP_K / 4;
-constexpr int NGF_BUFFER_CHUNKS = NGF_A_CHUNKS + NGF_C_CHUNKS + NGF_B_CHUNKS;      // 14 KB
+constexpr int NGF_N_PAD = 32;                  // rows of the padded copy of B come in whole multiples of this
+
+// Two shapes of the workgroup's tile, 64 m in both: 32 n x 16 o (O_BLOCKS = 1) and 16 n x 32 o
+// (O_BLOCKS = 2).  The signed pieces of A are made once per (m, n, k) and meet every block of 16
+// outputs, so with more than 16 outputs the second shape halves the vector work per result, which
+// is what bounds the first (17 to 32 outputs: one pass instead of two passes of 16).
+template <int O_BLOCKS>
+struct GradientF16Tile {
+    static constexpr int TILE_N = 32 / O_BLOCKS;
+    static constexpr int TILE_O = 16 * O_BLOCKS;
+    static constexpr int WAVE_N = TILE_N / 4;
+    static constexpr int A_CHUNKS = 8 * NGF_TILE_M;    // per step: 8 runs (slice, piece, half) of 64 rows
+    static constexpr int C_CHUNKS = 8 * TILE_O;
+    static constexpr int B_CHUNKS = TILE_N * NGF_STEP_K / 4;
+    static constexpr int BUFFER_CHUNKS = A_CHUNKS + C_CHUNKS + B_CHUNKS;      // 14 KB
+};
 
 struct NormGradientF16Args {
-    NormGradientArgs g;                        // extents, d, e, strides, o_chunks (of NGF_TILE_O); a, b, c are not read
+    NormGradientArgs g;                        // extents, d, e, strides, o_chunks (of the tile's outputs); a, b, c are not read
+    int o_begin;                               // the launch covers the outputs from here on
     const gram_chunk *pieces_a, *pieces_c;     // gram_f16_split of A (rows m) and of C (rows o)
     i64 pieces_a_bs, pieces_c_bs;              // per batch entry, in chunks
     const float *unscale_a, *unscale_c;
@@ -86,11 +96,14 @@ __global__ __launch_bounds__(256) void gradient_pad_b(const GradientPadArgs args
     *reinterpret_cast<float4 *>(args.padded + batch * args.padded_bs + (i64)n * args.k_pad + quad * 4) = make_float4(v[0], v[1], v[2], v[3]);
 }
 
+template <int O_BLOCKS>
 __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const NormGradientF16Args args)
 {
-    __shared__ gram_chunk lds0[NGF_BUFFER_CHUNKS];
-    __shared__ gram_chunk lds1[NGF_BUFFER_CHUNKS];
-    __shared__ gram_chunk lds2[NGF_BUFFER_CHUNKS];
+    using Tile = GradientF16Tile<O_BLOCKS>;
+    constexpr int WAVE_N = Tile::WAVE_N;
+    __shared__ gram_chunk lds0[Tile::BUFFER_CHUNKS];
+    __shared__ gram_chunk lds1[Tile::BUFFER_CHUNKS];
+    __shared__ gram_chunk lds2[Tile::BUFFER_CHUNKS];
 
     const NormGradientArgs &g = args.g;
     const int tid = threadIdx.x;
@@ -99,9 +112,9 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
     const int q = lane >> 4;     // 8 k of a step (operands), row quad (result)
     const int r = lane & 15;     // row m (T) / column o (C, result)
     const int batch = blockIdx.z / g.o_chunks;
-    const int o0 = (blockIdx.z % g.o_chunks) * NGF_TILE_O;
+    const int o0 = args.o_begin + (blockIdx.z % g.o_chunks) * Tile::TILE_O;
     const int m0 = blockIdx.x * NGF_TILE_M;
-    const int n0 = blockIdx.y * NGF_TILE_N;
+    const int n0 = blockIdx.y * Tile::TILE_N;
 
     auto buffer = [&](auto which) -> gram_chunk * {
         constexpr int B = decltype(which)::value;
@@ -110,11 +123,12 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
         else return lds2;
     };
 
-    // Copies per step: A 8 runs of 64 chunks (one per wave and run: 2 per wave), C 8 runs of 16
-    // chunks (2 copies of 4 runs; waves 0 and 2 issue the first, 1 and 3 the second: the same bytes
-    // twice, so that every wave has the same number of copies under way), B 32 rows of 128 bytes
-    // (8 rows per copy, one per wave).  A run (slice, piece, half) of a step starts at chunk
-    // ((2 step + slice) * 4 + 2 piece + half) * rows_pad of an operand's pieces.
+    // Copies per step, four per wave.  A: 8 runs of 64 chunks, two per wave.  C: 8 runs of 16 or 32
+    // chunks: with 16, two copies of 4 runs (waves 0 and 2 issue the first, 1 and 3 the second: the
+    // same bytes twice, so that every wave has the same number of copies under way); with 32, one
+    // copy of 2 runs per wave.  B: rows of 128 bytes, 8 per copy: with 32 rows one copy per wave,
+    // with 16 rows waves 2 and 3 repeat the copies of waves 0 and 1.  A run (slice, piece, half) of
+    // a step starts at chunk ((2 step + slice) * 4 + 2 piece + half) * rows_pad of an operand's pieces.
     typedef const __attribute__((address_space(1))) void *global_address;
     typedef __attribute__((address_space(3))) void *lds_address;
     const gram_chunk *src[4];
@@ -130,15 +144,18 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
             advance[j] = (i64)8 * args.rows_pad_a;
             dst[j] = run * NGF_TILE_M;
         }
-        const int c_run = 4 * (wave & 1) + q;
-        src[2] = pieces_c + (i64)c_run * args.rows_pad_c + r;
+        const int c_copy = O_BLOCKS == 1 ? (wave & 1) : wave;                   // 64 chunks of the step's C each
+        const int c_run = O_BLOCKS == 1 ? 4 * c_copy + q : 2 * c_copy + (lane >> 5);
+        const int c_row = O_BLOCKS == 1 ? r : (lane & 31);
+        src[2] = pieces_c + (i64)c_run * args.rows_pad_c + c_row;
         advance[2] = (i64)8 * args.rows_pad_c;
-        dst[2] = NGF_A_CHUNKS + 64 * (wave & 1);
-        // 8 rows of B per wave: lane -> row lane / 8, 16 bytes number lane % 8 of the step's 128
-        const float *b_row = args.b_padded + batch * args.b_padded_bs + (i64)(n0 + 8 * wave + (lane >> 3)) * args.k_pad + 4 * (lane & 7);
+        dst[2] = Tile::A_CHUNKS + 64 * c_copy;
+        // 8 rows of B per copy: lane -> row lane / 8, 16 bytes number lane % 8 of the step's 128
+        const int b_copy = O_BLOCKS == 1 ? wave : (wave & 1);
+        const float *b_row = args.b_padded + batch * args.b_padded_bs + (i64)(n0 + 8 * b_copy + (lane >> 3)) * args.k_pad + 4 * (lane & 7);
         src[3] = reinterpret_cast<const gram_chunk *>(b_row);
         advance[3] = NGF_STEP_K / 4;
-        dst[3] = NGF_A_CHUNKS + NGF_C_CHUNKS + 64 * wave;
+        dst[3] = Tile::A_CHUNKS + Tile::C_CHUNKS + 64 * b_copy;
     }
     auto copy_step = [&](auto into) {
 #pragma unroll
@@ -152,13 +169,13 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
         }
     };
 
-    // D[m, n] of this lane's rows, for the 8 n of the wave.
-    float dval[NGF_WAVE_N][4];
+    // D[m, n] of this lane's rows, for the n of the wave.
+    float dval[WAVE_N][4];
     {
         const float *d_base = g.d + batch * g.d_bs;
 #pragma unroll
-        for (int nb = 0; nb < NGF_WAVE_N; nb++) {
-            const int n = n0 + NGF_WAVE_N * wave + nb;
+        for (int nb = 0; nb < WAVE_N; nb++) {
+            const int n = n0 + WAVE_N * wave + nb;
 #pragma unroll
             for (int mb = 0; mb < 4; mb++) {
                 const int m = m0 + 16 * mb + r;
@@ -169,29 +186,34 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
     // the copies are not counted by the compiler: nothing it loads may be under way beside them
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
-    ngf_float4 acc[NGF_WAVE_N][4];
+    ngf_float4 acc[WAVE_N][4][O_BLOCKS];
 #pragma unroll
-    for (int nb = 0; nb < NGF_WAVE_N; nb++)
+    for (int nb = 0; nb < WAVE_N; nb++)
 #pragma unroll
-        for (int mb = 0; mb < 4; mb++) acc[nb][mb] = ngf_float4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int ob = 0; ob < O_BLOCKS; ob++) acc[nb][mb][ob] = ngf_float4{0.0f, 0.0f, 0.0f, 0.0f};
 
     // lane (q, r): its 8 k are slice q / 2, half q % 2 of the step
     const int run_of_lane = 4 * (q >> 1) + (q & 1);      // + 2 piece
     auto step = [&](auto which) {
         const gram_chunk *lds = buffer(which);
-        gram_half8 fc[GW_PIECES], fa[4][GW_PIECES];
+        gram_half8 fc[O_BLOCKS][GW_PIECES], fa[4][GW_PIECES];
 #pragma unroll
-        for (int p = 0; p < GW_PIECES; p++) fc[p] = __builtin_bit_cast(gram_half8, lds[NGF_A_CHUNKS + (run_of_lane + 2 * p) * NGF_TILE_O + r]);
+        for (int ob = 0; ob < O_BLOCKS; ob++)
+#pragma unroll
+            for (int p = 0; p < GW_PIECES; p++)
+                fc[ob][p] = __builtin_bit_cast(gram_half8, lds[Tile::A_CHUNKS + (run_of_lane + 2 * p) * Tile::TILE_O + 16 * ob + r]);
 #pragma unroll
         for (int mb = 0; mb < 4; mb++)
 #pragma unroll
             for (int p = 0; p < GW_PIECES; p++)
                 fa[mb][p] = __builtin_bit_cast(gram_half8, lds[(run_of_lane + 2 * p) * NGF_TILE_M + 16 * mb + r]);
-        const float4 *b_rows = reinterpret_cast<const float4 *>(lds + NGF_A_CHUNKS + NGF_C_CHUNKS);
+        const float4 *b_rows = reinterpret_cast<const float4 *>(lds + Tile::A_CHUNKS + Tile::C_CHUNKS);
 #pragma unroll
-        for (int nb = 0; nb < NGF_WAVE_N; nb++) {
-            const float4 b_low = b_rows[(NGF_WAVE_N * wave + nb) * (NGF_STEP_K / 4) + 2 * q];
-            const float4 b_high = b_rows[(NGF_WAVE_N * wave + nb) * (NGF_STEP_K / 4) + 2 * q + 1];
+        for (int nb = 0; nb < WAVE_N; nb++) {
+            const float4 b_low = b_rows[(WAVE_N * wave + nb) * (NGF_STEP_K / 4) + 2 * q];
+            const float4 b_high = b_rows[(WAVE_N * wave + nb) * (NGF_STEP_K / 4) + 2 * q + 1];
             const float bk[8] = {b_low.x, b_low.y, b_low.z, b_low.w, b_high.x, b_high.y, b_high.z, b_high.w};
 #pragma unroll
             for (int mb = 0; mb < 4; mb++) {
@@ -207,9 +229,12 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
                     t2[pair] ^= flip;
                 }
                 const gram_half8 h1 = __builtin_bit_cast(gram_half8, t1), h2 = __builtin_bit_cast(gram_half8, t2);
-                acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h2, fc[0], acc[nb][mb], 0, 0, 0);
-                acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[1], acc[nb][mb], 0, 0, 0);
-                acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[0], acc[nb][mb], 0, 0, 0);
+#pragma unroll
+                for (int ob = 0; ob < O_BLOCKS; ob++) acc[nb][mb][ob] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h2, fc[ob][0], acc[nb][mb][ob], 0, 0, 0);
+#pragma unroll
+                for (int ob = 0; ob < O_BLOCKS; ob++) acc[nb][mb][ob] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[ob][1], acc[nb][mb][ob], 0, 0, 0);
+#pragma unroll
+                for (int ob = 0; ob < O_BLOCKS; ob++) acc[nb][mb][ob] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[ob][0], acc[nb][mb][ob], 0, 0, 0);
             }
         }
         // the wave's own copies of the next step have arrived (the four of the step after it may
@@ -234,27 +259,31 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
-    // acc[nb][mb][j]: m = m0 + 16 mb + 4 q + j, o = o0 + r, n = n0 + 8 wave + nb
-    const int o = o0 + r;
-    const float unscale_c = args.unscale_c[batch * args.unscale_c_bs + o];
-    float *e_base = g.e + batch * g.e_bs + (i64)o * g.e_ld_o;
+    // acc[nb][mb][ob][j]: m = m0 + 16 mb + 4 q + j, o = o0 + 16 ob + r, n = n0 + WAVE_N wave + nb
 #pragma unroll
-    for (int mb = 0; mb < 4; mb++) {
-        const int m = m0 + 16 * mb + 4 * q;
-        const float4 unscale_a = *reinterpret_cast<const float4 *>(args.unscale_a + batch * args.unscale_a_bs + m);
+    for (int ob = 0; ob < O_BLOCKS; ob++) {
+        const int o = o0 + 16 * ob + r;
+        const float unscale_c = args.unscale_c[batch * args.unscale_c_bs + o];
+        float *e_base = g.e + batch * g.e_bs + (i64)o * g.e_ld_o;
 #pragma unroll
-        for (int nb = 0; nb < NGF_WAVE_N; nb++) {
-            const int n = n0 + NGF_WAVE_N * wave + nb;
-            if (n >= g.n || o >= g.o) continue;
-            const float v[4] = {acc[nb][mb][0] * unscale_a.x * unscale_c, acc[nb][mb][1] * unscale_a.y * unscale_c,
-                                acc[nb][mb][2] * unscale_a.z * unscale_c, acc[nb][mb][3] * unscale_a.w * unscale_c};
-            float *dst = e_base + (i64)n * g.e_ld_n + m;
-            if (g.e_vec && m + 3 < g.m) {
-                *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-            } else {
+        for (int mb = 0; mb < 4; mb++) {
+            const int m = m0 + 16 * mb + 4 * q;
+            const float4 unscale_a = *reinterpret_cast<const float4 *>(args.unscale_a + batch * args.unscale_a_bs + m);
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (m + j < g.m) dst[j] = v[j];
+            for (int nb = 0; nb < WAVE_N; nb++) {
+                const int n = n0 + WAVE_N * wave + nb;
+                if (n >= g.n || o >= g.o) continue;
+                const ngf_float4 sum = acc[nb][mb][ob];
+                const float v[4] = {sum[0] * unscale_a.x * unscale_c, sum[1] * unscale_a.y * unscale_c,
+                                    sum[2] * unscale_a.z * unscale_c, sum[3] * unscale_a.w * unscale_c};
+                float *dst = e_base + (i64)n * g.e_ld_n + m;
+                if (g.e_vec && m + 3 < g.m) {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (m + j < g.m) dst[j] = v[j];
+                }
             }
         }
     }

@@ -77,7 +77,7 @@ bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)
     layout->slices_alloc = 2 * (layout->steps + kmc::NGF_AHEAD);
     layout->slices_per_range = layout->slices / 8 > 8 ? (layout->slices + 7) / 8 : 8;
     layout->ranges = (layout->slices + layout->slices_per_range - 1) / layout->slices_per_range;
-    layout->n_pad = (p->n + kmc::NGF_TILE_N - 1) / kmc::NGF_TILE_N * kmc::NGF_TILE_N;
+    layout->n_pad = (p->n + kmc::NGF_N_PAD - 1) / kmc::NGF_N_PAD * kmc::NGF_N_PAD;
     layout->k_pad = kmc::NGF_STEP_K * (layout->steps + kmc::NGF_AHEAD);
     int64_t cursor = 0;
     place_rows(layout->a, p->m, p->a_bs == 0 ? 1 : p->l, *layout, cursor);
@@ -86,8 +86,9 @@ bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)
     layout->b_padded_bs = static_cast<int64_t>(layout->n_pad) * layout->k_pad;
     layout->b_padded = place(cursor, layout->b_batches * layout->b_padded_bs * 4);
     layout->bytes = cursor;
-    const int64_t grid_z = static_cast<int64_t>(p->l) * ((p->o + kmc::NGF_TILE_O - 1) / kmc::NGF_TILE_O);
-    if (grid_z > 65535 || layout->n_pad / kmc::NGF_TILE_N > 65535 || layout->n_pad > 65535) return false;
+    // blockIdx.z = batch entry x chunk of outputs, blockIdx.y = tile of at least 16 n
+    const int64_t grid_z = static_cast<int64_t>(p->l) * (p->o / 32 + 1);
+    if (grid_z > 65535 || layout->n_pad / 16 > 65535) return false;
     return true;
 }
 
@@ -148,7 +149,6 @@ hipError_t launch_norm_gradient_f16(const kmc_norm_gradient_params *p, bool a_ve
     args.g.m = p->m; args.g.n = p->n; args.g.o = p->o; args.g.k = p->k; args.g.l = p->l;
     args.g.d = p->d; args.g.d_ld = p->d_ld; args.g.d_bs = p->d_bs;
     args.g.e = p->e; args.g.e_ld_n = p->e_ld_n; args.g.e_ld_o = p->e_ld_o; args.g.e_bs = p->e_bs;
-    args.g.o_chunks = (p->o + kmc::NGF_TILE_O - 1) / kmc::NGF_TILE_O;
     args.g.e_vec = e_vec;
     args.pieces_a = rows_a.pieces; args.pieces_c = rows_c.pieces;
     args.pieces_a_bs = layout.a.batches > 1 ? layout.a.pieces_bs : 0;
@@ -160,9 +160,25 @@ hipError_t launch_norm_gradient_f16(const kmc_norm_gradient_params *p, bool a_ve
     args.b_padded_bs = layout.b_batches > 1 ? layout.b_padded_bs : 0;
     args.rows_pad_a = layout.a.rows_pad; args.rows_pad_c = layout.c.rows_pad;
     args.k_pad = layout.k_pad; args.steps = layout.steps;
-    const dim3 grid((p->m + kmc::NGF_TILE_M - 1) / kmc::NGF_TILE_M, layout.n_pad / kmc::NGF_TILE_N,
-                    static_cast<unsigned>(p->l) * args.g.o_chunks);
-    status = launch(kmc::norm_gradient_l1_f16, grid, dim3(kmc::NGF_THREADS), stream, args);
+    // Outputs in chunks of 32 on the 16 n x 32 o tile; what is left, if at most 16, on the 32 n x 16 o tile.
+    const int wide_chunks = p->o > 16 ? p->o / 32 + (p->o % 32 > 16 ? 1 : 0) : 0;
+    const int wide_outputs = wide_chunks * 32 < p->o ? wide_chunks * 32 : (wide_chunks ? p->o : 0);
+    const unsigned tiles_m = (p->m + kmc::NGF_TILE_M - 1) / kmc::NGF_TILE_M;
+    if (wide_chunks) {
+        using Tile = kmc::GradientF16Tile<2>;
+        args.o_begin = 0;
+        args.g.o_chunks = wide_chunks;
+        const dim3 grid(tiles_m, (p->n + Tile::TILE_N - 1) / Tile::TILE_N, static_cast<unsigned>(p->l) * wide_chunks);
+        status = launch(kmc::norm_gradient_l1_f16<2>, grid, dim3(kmc::NGF_THREADS), stream, args);
+        if (status != hipSuccess) return status;
+    }
+    if (wide_outputs < p->o) {
+        using Tile = kmc::GradientF16Tile<1>;
+        args.o_begin = wide_outputs;
+        args.g.o_chunks = 1;
+        const dim3 grid(tiles_m, (p->n + Tile::TILE_N - 1) / Tile::TILE_N, static_cast<unsigned>(p->l));
+        status = launch(kmc::norm_gradient_l1_f16<1>, grid, dim3(kmc::NGF_THREADS), stream, args);
+    }
     if (status == hipSuccess) *taken = true;
     return status;
 }
