@@ -131,6 +131,12 @@ def run_kernel_coefficients(
         panels = _panel_shape(plan, _backend.FLAG_DOT_PIECES)
         if panels is not None and _run_in_panels(plan, panels, stream, a.device, debug):
             return plan.out
+    if (plan.O > _FUSED_COLUMNS_PER_WALK and float(plan.L) * plan.M * plan.N >= _MANY_COLUMNS_MIN_ELEMENTS
+            and _backend.build_kernel_has_variant(kernel.inner_operator, kernel.inner_power)):
+        # any descriptor: the fused kernel would walk the matrix once per 64 columns
+        panels = _panel_shape(plan, 0)
+        if panels is not None and _run_in_panels(plan, panels, stream, a.device, debug):
+            return plan.out
     ranges = _centre_ranges(plan, three_resident=aot and not matrix_core and plan.O <= 32)
     partial = None
     if ranges > 1:
@@ -166,7 +172,16 @@ def run_kernel_coefficients(
 # K = 1024, O = 16 18.6 -> 7.1 ms; M = 10000, N = 100000, K = 784, O = 10 16.6 -> 8.0 ms; M = 20000,
 # N = 50000, K = 3072, O = 10 56.8 -> 17.8 ms.  The partial products of the panels (and of the
 # ranges a panel is cut into when the rows alone do not fill the chip) are added in a fixed order.
+#
+# The same two steps serve every descriptor when there are more than 64 coefficient columns: the fused
+# kernel holds at most 64 per walk of the kernel matrix and walks it ceil(O / 64) times, while a panel
+# built once by kmc_build_kernel (whatever kernel this descriptor and l2 mode launch for a stored
+# matrix) is contracted with all columns at 4 bytes of traffic per element.  Laplace kernel on L1
+# distances, L = 4, M = N = 16384, K = 256: O = 65 .. 128 22.1 -> 11.8 .. 12.0 ms, O = 256 44.0 -> 14.6 ms,
+# O = 1000 176 -> 30.7 ms; p = 1.3 norm, M = 1000, N = 20000, K = 784, O = 300: 15.1 -> 3.2 ms.
 _PANEL_BYTES = 1 << 30
+_FUSED_COLUMNS_PER_WALK = 64
+_MANY_COLUMNS_MIN_ELEMENTS = 1e6        # below, the three launches cost what the second walk does (500 x 500, O = 100: 54 against 41 us)
 _PANEL_MAX_PARTIAL_BYTES = 512 << 20
 
 
@@ -256,11 +271,11 @@ def _panel_shape(plan, route):
 
     budget = int(os.environ.get("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", _PANEL_BYTES))
     L, M, N, O = plan.L, plan.M, plan.N, plan.O
-    # l2 mode "gram" asks for the fp32 matrix instruction; the panels are built from fp16 pieces
-    mode = _l2_current()["mode"]
-    if budget <= 0 or 0 in (L, M, N, O, plan.K) or mode not in ("auto", "gram_bf16"):
+    if budget <= 0 or 0 in (L, M, N, O, plan.K):
         return None
-    if mode == "auto" and plan.K < _AUTO_PANEL_MIN_K:
+    # l2 mode "gram" asks for the fp32 matrix instruction; the panels of a route are built from fp16 pieces
+    mode = _l2_current()["mode"]
+    if route and (mode not in ("auto", "gram_bf16") or (mode == "auto" and plan.K < _AUTO_PANEL_MIN_K)):
         return None
     ld = -(-M // 4) * 4                                          # rows of the panel start on 16 bytes
     rows = min(N, max(256, budget // (4 * L * ld) // 256 * 256))
@@ -270,7 +285,7 @@ def _panel_shape(plan, route):
     block = _backend.BuildKernelParams.from_buffer_copy(plan.params.kernel)
     block.flags |= route
     block.n, block.c, block.c_ld, block.c_bs = rows, 256, ld, rows * ld      # c: any address, for the query
-    if _backend.gram_workspace_bytes(block) == 0:
+    if route and _backend.gram_workspace_bytes(block) == 0:
         # panels of this shape would not take the fast route by themselves
         if mode != "auto" or route != _backend.FLAG_L2_GRAM_BF16 or not _auto_panels_of_any_size(plan):
             return None
@@ -279,9 +294,8 @@ def _panel_shape(plan, route):
         if _backend.gram_workspace_bytes(block) == 0:
             return None
     splits = _panel_splits(M, O, L, rows)
-    parts = panels * splits
-    if parts > 1 and 4 * parts * L * M * O > _PANEL_MAX_PARTIAL_BYTES:
-        return None
+    if panels * splits > 1 and 4 * panels * splits * L * M * O > _PANEL_MAX_PARTIAL_BYTES:
+        splits = 0              # too many partial products to keep: every panel is added to the result as it comes
     return rows, panels, ld, splits, route
 
 
@@ -291,7 +305,7 @@ def _run_in_panels(plan, shape, stream, device, debug):
 
     rows, panels, ld, splits, route = shape
     L, M, N, O = plan.L, plan.M, plan.N, plan.O
-    parts = panels * splits
+    parts = panels * splits                                      # 0: no partial products, the panels accumulate
     params = plan.params
     block = _backend.BuildKernelParams.from_buffer_copy(params.kernel)
     block.flags |= route
@@ -302,12 +316,12 @@ def _run_in_panels(plan, shape, stream, device, debug):
     except torch.cuda.OutOfMemoryError:
         return False
     block.c = panel.data_ptr()
-    workspace = _attach_gram_workspace(block, device)
-    if workspace is None:
+    workspace = _attach_gram_workspace(block, device) if route else None
+    if route and workspace is None:
         return False
     if debug:
         print(f"(Kermac Debug) Kernel matrix x coefficients in {panels} panels of {rows} centres, "
-              f"{splits} partial products each")
+              + (f"{splits} partial products each" if splits else "added to the result one after the other"))
     row_major_b = block.b_majorness == _backend.ROW_MAJOR
     contraction = _backend.MatrixCoefficientsParams()
     contraction.m, contraction.o, contraction.l = M, O, L
@@ -326,11 +340,14 @@ def _run_in_panels(plan, shape, stream, device, debug):
         block.b = first_b + 4 * n0 * (block.b_ld if row_major_b else 1)
         block.regularization_offset_y = first_offset + n0
         _backend.build_kernel(block, stream)
-        block.flags |= _backend.FLAG_GRAM_A_KEPT                 # the rows are the same for every panel: split once
+        if route:
+            block.flags |= _backend.FLAG_GRAM_A_KEPT             # the rows are the same for every panel: split once
         contraction.n, contraction.matrix_bs = count, count * ld
         contraction.coef = params.coef + 4 * n0 * params.coef_ld
         if partial is not None:
             contraction.out = partial.data_ptr() + 4 * index * splits * L * M * O
+        else:
+            contraction.accumulate = 1 if index else 0
         _backend.matrix_times_coefficients(contraction, stream)
     if partial is not None:
         _sum_partials(partial, plan.out)

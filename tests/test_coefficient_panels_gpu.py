@@ -240,3 +240,45 @@ def test_auto_mode_takes_panels_where_the_fused_kernel_is_the_slower_one(device,
     with kermac.l2_mode("gram_bf16"):           # the explicit mode follows the library's rule: the fused kernel
         kermac.run_kernel(GAUSSIAN, a, b, coefficients=coef, bandwidth=bandwidth, debug=True)
         assert PANELS not in capsys.readouterr().out
+
+
+@pytest.mark.parametrize("descriptor,names,kw", [
+    (kermac.kernel_descriptor_laplace_l1, ("DIFF", "ABS", "NOOP", "LAPLACE"), {"bandwidth": 7.0}),
+    (kermac.kernel_descriptor_p_norm, ("DIFF", "POW", "POW", "NONE"), {"p": 1.3}),
+    (kermac.kernel_descriptor_laplace_l2, ("DIFF", "SQUARE", "SQRT", "LAPLACE"), {"bandwidth": 5.0}),
+])
+def test_more_than_64_columns_go_in_panels_for_every_descriptor(device, monkeypatch, capsys, descriptor, names, kw):
+    """The fused kernel holds 64 coefficient columns per walk of the kernel matrix; with more, the
+    matrix is built once per panel by kmc_build_kernel (whatever kernel the descriptor launches)
+    and contracted with all columns.  Same tolerance as the fused kernel; a regularised diagonal
+    across panels; partial products, and panels added one after the other when the partial
+    products would take too much memory."""
+    from kermac_amd import kernel_coefficients as module
+    g = torch.Generator().manual_seed(87)
+    L, M, N, K, O = 2, 700, 1800, 24, 70
+    a = make_operand(L, M, K, False, device, g)
+    b = make_operand(L, N, K, True, device, g)
+    coef = torch.randn(L, N, O, generator=g).to(device)
+    extra = dict(kw)
+    if "bandwidth" in kw:
+        extra.update(regularization=0.5, regularization_offset_x=1, regularization_offset_y=4)
+    oracle_kw = dict(kw)
+    if "p" in oracle_kw:
+        oracle_kw = {"p_inner": kw["p"], "p_outer": 1.0 / kw["p"]}
+    if "bandwidth" in kw:
+        oracle_kw.update(regularization=0.5, regularization_offset_x=1, regularization_offset_y=4)
+    truth = oracle.run_kernel_coefficients(*names, a.cpu().contiguous(), b.cpu().contiguous(), coef.cpu(), **oracle_kw)
+    rtol = 1e-4 if "p" in kw else 1e-5
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", str(4 * L * 700 * 512))           # panels of 512 centres
+    for cap, said in ((module._PANEL_MAX_PARTIAL_BYTES, "partial products each"), (1024, "added to the result one after the other")):
+        monkeypatch.setattr(module, "_PANEL_MAX_PARTIAL_BYTES", cap)
+        out = torch.full((L, M, O + 2), 3.0, device=device)
+        got = kermac.run_kernel(descriptor, a, b, out=out[..., :O], coefficients=coef, debug=True, **extra)
+        printed = capsys.readouterr().out
+        assert f"{PANELS} 4 panels of 512 centres" in printed and said in printed, printed
+        assert_close_to_truth(got, truth, rtol=rtol, atol=atol_for(truth, rtol), what=f"{names}, {said}")
+        assert torch.all(out[..., O:] == 3.0), "wrote outside the out view"
+    kermac.run_kernel(descriptor, a, b, coefficients=coef[..., :64], debug=True, **extra)      # 64 columns: one walk, fused
+    assert PANELS not in capsys.readouterr().out
+    kermac.run_kernel(descriptor, a[:, :300], b[:, :300], coefficients=coef[:, :300], debug=True, **extra)     # a small problem: fused
+    assert PANELS not in capsys.readouterr().out

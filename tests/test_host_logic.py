@@ -628,6 +628,13 @@ def test_auto_mode_of_the_coefficient_product_without_a_gpu(monkeypatch):
         assert module._panel_shape(p, _backend.FLAG_L2_GRAM_BF16)[4] == _backend.FLAG_L2_GRAM_BF16
     with kermac.l2_mode("direct"):
         assert plan(4096, 4096, 256, 32).params.kernel.flags & _backend.FLAG_L2_GRAM == 0
+        # more than 64 columns: plain panels (no route flag) in any mode, for any descriptor
+        rows, panels, ld, splits, flags = module._panel_shape(plan(4096, 20000, 256, 100, descriptor=kermac.kernel_descriptor_laplace_l1), 0)
+        assert (rows, panels, ld, flags) == (20000, 1, 4096, 0) and splits >= 1
+    # partial products beyond 512 MiB are not kept: the panels are added to the result one after the other
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", str(1 << 26))
+    assert module._panel_shape(plan(16384, 16384, 256, 1000, L=4, descriptor=kermac.kernel_descriptor_laplace_l1), 0)[3] == 0
+    monkeypatch.delenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES")
     assert plan(4096, 4096, 256, 32, descriptor=kermac.kernel_descriptor_laplace_l1).params.kernel.flags & _backend.FLAG_L2_GRAM == 0
 
 
