@@ -17,7 +17,7 @@ import torch
 
 from . import _backend
 from .common import launch_cuts_enabled, merge_batch_size
-from .module_cache.module_cache import ModuleCache, kernel_coefficients_function_name
+from .module_cache.module_cache import ModuleCache, build_kernel_function_name, kernel_coefficients_function_name
 
 
 class _CoefPlan:
@@ -131,9 +131,8 @@ def run_kernel_coefficients(
         panels = _panel_shape(plan, _backend.FLAG_DOT_PIECES)
         if panels is not None and _run_in_panels(plan, panels, stream, a.device, debug):
             return plan.out
-    if (plan.O > _FUSED_COLUMNS_PER_WALK and float(plan.L) * plan.M * plan.N >= _MANY_COLUMNS_MIN_ELEMENTS
-            and _backend.build_kernel_has_variant(kernel.inner_operator, kernel.inner_power)):
-        # any descriptor: the fused kernel would walk the matrix once per 64 columns
+    if plan.O > _FUSED_COLUMNS_PER_WALK and float(plan.L) * plan.M * plan.N >= _MANY_COLUMNS_MIN_ELEMENTS:
+        # any descriptor, compiled ahead of time or at run time: the fused kernel would walk the matrix once per 64 columns
         panels = _panel_shape(plan, 0)
         if panels is not None and _run_in_panels(plan, panels, stream, a.device, debug):
             return plan.out
@@ -173,7 +172,7 @@ def run_kernel_coefficients(
 # N = 50000, K = 3072, O = 10 56.8 -> 17.8 ms.  The partial products of the panels (and of the
 # ranges a panel is cut into when the rows alone do not fill the chip) are added in a fixed order.
 #
-# The same two steps serve every descriptor when there are more than 64 coefficient columns: the fused
+# The same two steps serve every descriptor (also those compiled at run time) when there are more than 64 coefficient columns: the fused
 # kernel holds at most 64 per walk of the kernel matrix and walks it ceil(O / 64) times, while a panel
 # built once by kmc_build_kernel (whatever kernel this descriptor and l2 mode launch for a stored
 # matrix) is contracted with all columns at 4 bytes of traffic per element.  Laplace kernel on L1
@@ -333,13 +332,23 @@ def _run_in_panels(plan, shape, stream, device, debug):
         contraction.out_ld, contraction.out_bs = O, M * O
         contraction.n_splits, contraction.out_split_stride = splits, L * M * O
     first_b, first_offset = params.kernel.b, params.kernel.regularization_offset_y
+    function = None
+    if not _backend.build_kernel_has_variant(block.inner_operator, block.inner_power):
+        # a descriptor compiled at run time; the panels start at multiples of 256 rows of b, so all of them
+        # take the loader variant of the first
+        load_a, load_b = _backend.build_kernel_load_modes(block)
+        name = build_kernel_function_name(block.inner_operator, block.inner_power, load_a, load_b)
+        function = ModuleCache(debug).get_function(device, name, debug=debug)
     for index in range(panels):
         n0 = index * rows
         count = min(rows, N - n0)
         block.n, block.c_bs = count, count * ld
         block.b = first_b + 4 * n0 * (block.b_ld if row_major_b else 1)
         block.regularization_offset_y = first_offset + n0
-        _backend.build_kernel(block, stream)
+        if function is None:
+            _backend.build_kernel(block, stream)
+        else:
+            _backend.build_kernel_jit(function, block, stream)
         if route:
             block.flags |= _backend.FLAG_GRAM_A_KEPT             # the rows are the same for every panel: split once
         contraction.n, contraction.matrix_bs = count, count * ld

@@ -282,3 +282,22 @@ def test_more_than_64_columns_go_in_panels_for_every_descriptor(device, monkeypa
     assert PANELS not in capsys.readouterr().out
     kermac.run_kernel(descriptor, a[:, :300], b[:, :300], coefficients=coef[:, :300], debug=True, **extra)     # a small problem: fused
     assert PANELS not in capsys.readouterr().out
+
+
+def test_more_than_64_columns_of_a_run_time_compiled_descriptor(device, monkeypatch, capsys):
+    """sum_k sqrt(a b), squared: not built ahead of time; its panels come from the run-time compiled
+    kernel of run_kernel, the contraction is the same."""
+    g = torch.Generator().manual_seed(88)
+    desc = kermac.KernelDescriptor(kermac.InnerOperator.DOT, kermac.PowerType.SQRT, kermac.PowerType.SQUARE, kermac.KernelType.NONE)
+    M, N, K, O = 900, 1300, 20, 66
+    a = torch.rand(M, K, generator=g).to(device)
+    b = torch.rand(K, N, generator=g).to(device).t()
+    coef = torch.randn(N, O, generator=g).to(device)
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", str(4 * 900 * 512))
+    got = kermac.run_kernel(desc, a, b, coefficients=coef, debug=True)
+    assert f"{PANELS} 3 panels of 512 centres" in capsys.readouterr().out
+    truth = oracle.run_kernel_coefficients("DOT", "SQRT", "SQUARE", "NONE", a.cpu(), b.cpu().contiguous(), coef.cpu())
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="run-time compiled descriptor in panels")
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "0")
+    fused = kermac.run_kernel(desc, a, b, coefficients=coef)
+    assert_close_to_truth(fused, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="the same on the fused kernel")
