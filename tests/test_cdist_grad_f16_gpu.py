@@ -94,9 +94,10 @@ def test_signs_at_zero_and_rows_of_different_magnitude(device, f16_route):
     assert error.max().item() < 1e-6, f"error {error.max().item():.2e} of the sum of absolute terms"
 
 
-def test_batches_broadcast_and_views(device, f16_route):
+@pytest.mark.parametrize("O", [6, 20, 37])                      # one tile shape, the other, both
+def test_batches_broadcast_and_views(device, f16_route, O):
     g = torch.Generator().manual_seed(91)
-    L, M, N, O, K = 3, 90, 20, 6, 45
+    L, M, N, K = 3, 90, 20, 45
     a = torch.rand(L, K, M + 3, generator=g).to(device)[:, :, 1:M + 1]       # padded, misaligned rows
     b = torch.randn(N, K + 2, generator=g).to(device)[:, 1:K + 1]            # shared by the batch
     c = torch.randn(L, O, K, generator=g).to(device)
