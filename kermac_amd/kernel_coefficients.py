@@ -172,7 +172,8 @@ def run_kernel_coefficients(
 # N = 50000, K = 3072, O = 10 56.8 -> 17.8 ms.  The partial products of the panels (and of the
 # ranges a panel is cut into when the rows alone do not fill the chip) are added in a fixed order.
 #
-# The same two steps serve every descriptor (also those compiled at run time) when there are more than 64 coefficient columns: the fused
+# The same two steps serve every descriptor (also those compiled at run time) when there are more
+# than 64 coefficient columns: the fused
 # kernel holds at most 64 per walk of the kernel matrix and walks it ceil(O / 64) times, while a panel
 # built once by kmc_build_kernel (whatever kernel this descriptor and l2 mode launch for a stored
 # matrix) is contracted with all columns at 4 bytes of traffic per element.  Laplace kernel on L1
