@@ -1,8 +1,8 @@
 """A seeded sweep of mid-size calls in the default l2 mode, no route forced: sizes from a few
-hundred to twenty thousand rows, contractions from 64 to 3200, 1 to 70 coefficient columns, both
+hundred to twenty thousand rows, contractions from 64 to 3200, 1 to 130 coefficient columns, both
 storage orders, padded rows, operands shared by the batch.  Every call takes whatever the rules
 pick for it (direct kernel, one-step matrix-core kernels, the route through a workspace, the cut
-over k, the fused coefficient kernel in either variant, panels), and the result is checked
+over k, the fused coefficient kernel in either variant, panels of either kind), and the result is checked
 against float64 arithmetic on the device (torch.cdist and matmul in float64; the CPU oracle would
 take minutes at these sizes).  Tolerance as everywhere: rtol 1e-5, for sums with coefficients
 plus an absolute floor proportional to the typical magnitude of the sum.
@@ -36,17 +36,18 @@ def test_mid_size_calls_as_the_rules_route_them(device):
     rng = random.Random(11)
     torch.manual_seed(11)
     done = 0
-    while done < 60:
+    while done < 72:
         L = rng.choice((1, 1, 1, 2, 3))
         M = rng.choice((rng.randint(60, 300), rng.randint(300, 1500), rng.randint(1500, 5000)))
         N = rng.choice((rng.randint(100, 600), rng.randint(600, 3000), rng.randint(3000, 20000)))
         K = rng.choice((rng.randint(64, 200), rng.randint(200, 400), rng.randint(700, 900), rng.randint(1500, 3200)))
-        O = rng.choice((1, 7, 32, 40, 70))
+        O = rng.choice((1, 7, 32, 40, 70, 130))
         if L * M * N * K > 3e10 or L * M * N > 6e7:
             continue
         done += 1
         col_major = rng.random() < 0.4
-        kind = rng.choice(("distances", "gaussian x coefficients", "gaussian x coefficients", "laplace x coefficients", "products"))
+        kind = rng.choice(("distances", "gaussian x coefficients", "gaussian x coefficients", "laplace x coefficients", "products",
+                           "laplace on L1 x coefficients"))
         a = operand(rng, device, L, M, K, col_major, rng.random() < 0.2)
         b = operand(rng, device, L, N, K, col_major if rng.random() < 0.8 else not col_major, rng.random() < 0.2)
         what = f"case {done}: {kind}, L={L} M={M} N={N} K={K} O={O}, a {tuple(a.shape)} {a.stride()}, b {tuple(b.shape)} {b.stride()}"
@@ -66,6 +67,12 @@ def test_mid_size_calls_as_the_rules_route_them(device):
             if kind == "gaussian x coefficients":
                 got = kermac.run_kernel(GAUSSIAN, a, b, coefficients=coef, bandwidth=bandwidth)
                 matrix = torch.exp(-torch.cdist(a64, b64, p=2.0) ** 2 / (2 * bandwidth ** 2))
+            elif kind == "laplace on L1 x coefficients":
+                got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, b, coefficients=coef, bandwidth=4 * bandwidth)
+                # blocks of rows, explicitly: torch.cdist with p = 1 in float64 returns wrong rows on the device at some sizes
+                l1 = torch.stack([torch.cat([(a64[l, i:i + 32, None, :] - b64[l][None]).abs().sum(-1) for i in range(0, M, 32)])
+                                  for l in range(batch)])
+                matrix = torch.exp(-l1 / (4 * bandwidth))
             else:
                 got = kermac.run_kernel(kermac.kernel_descriptor_laplace_l2, a, b, coefficients=coef, bandwidth=bandwidth,
                                         regularization=0.25, regularization_offset_x=3, regularization_offset_y=1)
