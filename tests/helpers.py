@@ -28,3 +28,10 @@ def make_operand(L, rows, K, col_major, device, generator, batch=True, dist="ran
     if col_major:
         t = t.transpose(-1, -2)
     return t
+
+
+def l1_distances_float64(a: torch.Tensor, b: torch.Tensor, block: int = 16) -> torch.Tensor:
+    """sum_k |a[m, k] - b[n, k]| in float64, by blocks of rows of a, on the device of the operands
+    (torch.cdist with p = 1 in float64 has returned wrong rows on the GPU for some sizes)."""
+    a, b = a.double(), b.double()
+    return torch.cat([(a[i:i + block, None, :] - b[None]).abs().sum(-1) for i in range(0, a.size(0), block)])
