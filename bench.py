@@ -245,6 +245,23 @@ def bench_cdist_grad(kermac, device, args, steps=None, warmup=None):
     log(f"  p=2, same operands: {l2_ms:.2f} ms (slab err {l2_err:.2e}); on the fp32 matrix-core kernel {l2_fp32_ms:.2f} ms ({l2_fp32_err:.2e})")
     check_parity("cdist_grad p=2 slab, max abs err / mean |truth|", l2_err, 1e-4)
     check_parity("cdist_grad p=2 (fp32 kernels) slab, max abs err / mean |truth|", l2_fp32_err, 1e-4)
+    # Beside it: 32 outputs, p = 1 (the tile of 16 n x 32 outputs: the sign work is shared by two blocks of outputs).
+    c32 = torch.randn(32, k_ref, device=device)
+    out32 = torch.empty(1, 32, n_ref, m_ref, device=device)
+    truth32 = torch.einsum("ok,km,nmk->onm", c32.double(), a[:, ms].double(), sign)
+    _, o32_ms = time_call(lambda: kermac.cdist_grad(a, b, c32, d, out=out32, p=1.0), side, 1)
+    o32_err = ((out32[0][:, ns, ms].double() - truth32).abs().max() / truth32.abs().mean()).item()
+    os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"] = "0"
+    try:
+        _, o32_fp32_ms = time_call(lambda: kermac.cdist_grad(a, b, c32, d, out=out32, p=1.0), 2, 1)
+    finally:
+        if saved is None:
+            del os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"]
+        else:
+            os.environ["KERMAC_AMD_GRADIENT_WORKSPACE"] = saved
+    del out32
+    log(f"  p=1, 32 outputs: {o32_ms:.2f} ms (slab err {o32_err:.2e}); on the fp32 matrix-core kernel {o32_fp32_ms:.2f} ms")
+    check_parity("cdist_grad p=1, 32 outputs, slab, max abs err / mean |truth|", o32_err, 1e-4)
     # Executed matrix work on the default route: three products of fp16 pieces, 2 * O flops each per (m, n, k),
     # against the dense fp16 peak; the sign work on the vector ALU (2.5 instructions per (m, n, k)) is what bounds it.
     ops = 3.0 * 2.0 * o * m_ref * n_ref * k_ref
@@ -262,7 +279,9 @@ def bench_cdist_grad(kermac, device, args, steps=None, warmup=None):
                                            "route": "e = (d - s) (c a) - (c (b - s)) a with s the row means of b: one product of "
                                                     "(o n) x k by k x m from two fp16 pieces per value, v_mfma_f32_32x32x16_f16",
                                            "mfma_tflops": round(3.0 * 2.0 * o * m_ref * n_ref * k_ref / l2_ms / 1e9, 2),
-                                           "fp32_kernels_ms": round(l2_fp32_ms, 3), "fp32_kernels_parity_max_err_over_mean": l2_fp32_err}},
+                                           "fp32_kernels_ms": round(l2_fp32_ms, 3), "fp32_kernels_parity_max_err_over_mean": l2_fp32_err},
+                      "p1_32_outputs": {"ms": round(o32_ms, 3), "parity_max_err_over_mean": o32_err, "fp32_kernels_ms": round(o32_fp32_ms, 3),
+                                        "route": "tiles of 64 m x 16 n x 32 outputs: the signed pieces meet two blocks of 16 outputs"}},
                      args)
 
 
