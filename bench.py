@@ -354,6 +354,31 @@ def bench_kernel_coef(kermac, device, args, steps=None, warmup=None, with_gaussi
                                         "note": "the default l2 mode 'auto' builds the kernel matrix in panels of 4096 centres "
                                                 "(1 GiB, reused) on the fp16 matrix instruction and contracts each panel; "
                                                 "l2 mode 'gram' is the fused kernel on the fp32 matrix instruction"}
+    if with_gaussian:
+        # Beside it: the Laplace kernel of the headline with 100 coefficient columns.  The fused kernel holds 64 per
+        # walk of the kernel matrix, so the default builds the matrix once per panel and contracts it with all columns.
+        coef100 = torch.randn(L, mz, 100, device=device)
+        out100 = torch.empty(L, nx, 100, device=device)
+        call = lambda: kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, x.transpose(1, 2), z.t(), out=out100,
+                                         bandwidth=10.0, coefficients=coef100)
+        _, many_ms = time_call(call, 3, 1)
+        many_err = ((out100[0, rows].double() - torch.exp(-l1 / 10.0) @ coef100[0].double()).abs().max()
+                    / (torch.exp(-l1 / 10.0) @ coef100[0].double()).abs().mean()).item()
+        saved = os.environ.get("KERMAC_AMD_COEFFICIENT_PANEL_BYTES")
+        os.environ["KERMAC_AMD_COEFFICIENT_PANEL_BYTES"] = "0"
+        try:
+            _, many_fused_ms = time_call(call, 2, 1)
+        finally:
+            if saved is None:
+                del os.environ["KERMAC_AMD_COEFFICIENT_PANEL_BYTES"]
+            else:
+                os.environ["KERMAC_AMD_COEFFICIENT_PANEL_BYTES"] = saved
+        log(f"laplace x 100 coefficient columns: default (panels of the matrix, then contracted) {many_ms:.2f} ms, "
+            f"fused kernel (two walks of the matrix) {many_fused_ms:.2f} ms; slab max abs err / mean |truth| = {many_err:.2e}")
+        check_parity("laplace x 100 coefficient columns (panels) slab, max abs err / mean |truth|", many_err, 1e-4)
+        extra["laplace_100_columns"] = {"default_panels_ms": round(many_ms, 3), "fused_ms": round(many_fused_ms, 3),
+                                        "parity_max_err_over_mean": many_err}
+        del coef100, out100
     ops = float(L) * nx * mz * (3 * k + 2 * o)
     nbytes = 4.0 * (L * k * nx + k * mz + 2 * L * nx * o)
     return side_line("fused Laplace kernel matrix x coefficients ms, L=4 N=M=16384 K=256 O=32",
