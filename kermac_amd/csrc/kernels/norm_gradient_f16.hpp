@@ -19,15 +19,15 @@
 // a2 c2 below 2^-22 |a c|: the error of E from the pieces is below 3 * 2^-22 sum_k |c a|, the size
 // of the rounding of an fp32 accumulation over a few terms, beside the fp32 accumulation itself.
 //
-// Workgroup: 4 waves, 64 m x 32 n x 16 o (for more than 16 outputs 64 m x 16 n x 32 o, below); wave w
-// owns the 8 (4) n  8w .. 8w + 7  and all 64 m as 4 row blocks of 16.  Per 32 k it reads the pieces of C (2 x 16 bytes per lane) and of its A rows
+// Workgroup: 4 waves, 64 m x 32 n x 16 o (for more than 16 outputs 64 m x 16 n x 32 o or 64 m x 8 n x 64 o,
+// below); wave w owns the 8 (4, 2) n  8w .. 8w + 7  and all 64 m as 4 row blocks of 16.  Per 32 k it reads the pieces of C (2 x 16 bytes per lane) and of its A rows
 // (8 x 16 bytes), and per n the 8 values of B that match its 8 k (2 x 16 bytes, the same for the
 // 16 lanes of a row block).  B is copied once into a padded array in the workspace (rows to 32,
 // k to 32 plus what the walk copies ahead), so that everything the walk touches exists and all of
 // it arrives in LDS by global_load_lds_dwordx4, three steps in three buffers, as in
 // gram_f16_wide.hpp (the copies are inline instructions for the reason given there).
 //
-// Measured at M = K = 8192, N = 512, O = 16: 3.86 ms (O = 32 on the second shape: 5.4 ms) for this kernel and 0.33 ms for the row kernels
+// Measured at M = K = 8192, N = 512, O = 16: 3.86 ms (O = 32 on the second shape 5.4 ms, O = 64 on the third 9.2 ms) for this kernel and 0.33 ms for the row kernels
 // against 9.85 ms on the fp32 kernels.  Counters: 2.5 vector instructions per (m, n, k) (the
 // compiler fuses AND and XOR into v_bitop3_b32), the matrix pipeline busy 46 % and the vector
 // pipeline about 44 % of the elapsed cycles, hardly ever together, shader clock 1.75 GHz.  Tried
@@ -50,10 +50,10 @@ constexpr int NGF_THREADS = 256;
 constexpr int NGF_AHEAD = 3;                   // steps copied ahead of the walk
 constexpr int NGF_N_PAD = 32;                  // rows of the padded copy of B come in whole multiples of this
 
-// Two shapes of the workgroup's tile, 64 m in both: 32 n x 16 o (O_BLOCKS = 1) and 16 n x 32 o
-// (O_BLOCKS = 2).  The signed pieces of A are made once per (m, n, k) and meet every block of 16
-// outputs, so with more than 16 outputs the second shape halves the vector work per result, which
-// is what bounds the first (17 to 32 outputs: one pass instead of two passes of 16).
+// Three shapes of the workgroup's tile, 64 m in all: 32 n x 16 o (O_BLOCKS = 1), 16 n x 32 o
+// (O_BLOCKS = 2) and 8 n x 64 o (O_BLOCKS = 4).  The signed pieces of A are made once per (m, n, k)
+// and meet every block of 16 outputs, so with more outputs the wider shapes divide the vector work
+// per result, which is what bounds the first (17 to 32 outputs: one pass instead of two of 16).
 template <int O_BLOCKS>
 struct GradientF16Tile {
     static constexpr int TILE_N = 32 / O_BLOCKS;
@@ -62,7 +62,8 @@ struct GradientF16Tile {
     static constexpr int A_CHUNKS = 8 * NGF_TILE_M;    // per step: 8 runs (slice, piece, half) of 64 rows
     static constexpr int C_CHUNKS = 8 * TILE_O;
     static constexpr int B_CHUNKS = TILE_N * NGF_STEP_K / 4;
-    static constexpr int BUFFER_CHUNKS = A_CHUNKS + C_CHUNKS + B_CHUNKS;      // 14 KB
+    static constexpr int BUFFER_CHUNKS = A_CHUNKS + C_CHUNKS + B_CHUNKS;      // 14 KB (17 KB for 64 outputs)
+    static constexpr int COPIES = O_BLOCKS == 4 ? 5 : 4;                       // per wave and step
 };
 
 struct NormGradientF16Args {
@@ -123,17 +124,20 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
         else return lds2;
     };
 
-    // Copies per step, four per wave.  A: 8 runs of 64 chunks, two per wave.  C: 8 runs of 16 or 32
-    // chunks: with 16, two copies of 4 runs (waves 0 and 2 issue the first, 1 and 3 the second: the
-    // same bytes twice, so that every wave has the same number of copies under way); with 32, one
-    // copy of 2 runs per wave.  B: rows of 128 bytes, 8 per copy: with 32 rows one copy per wave,
-    // with 16 rows waves 2 and 3 repeat the copies of waves 0 and 1.  A run (slice, piece, half) of
-    // a step starts at chunk ((2 step + slice) * 4 + 2 piece + half) * rows_pad of an operand's pieces.
+    // Copies per step, four per wave (five for 64 outputs), the same number in every wave so that
+    // one count of copies under way serves all.  A: 8 runs of 64 chunks, two per wave.  C: 8 runs of
+    // 16, 32 or 64 chunks: with 16, two copies of 4 runs (waves 0 and 2 issue the first, 1 and 3 the
+    // second: the same bytes twice); with 32, one copy of 2 runs per wave; with 64, two copies of one
+    // run per wave.  B: rows of 128 bytes, 8 per copy: with 32 rows one copy per wave, with 16 rows
+    // waves 2 and 3 repeat the copies of waves 0 and 1, with 8 rows every wave issues the one copy.
+    // A run (slice, piece, half) of a step starts at chunk ((2 step + slice) * 4 + 2 piece + half) *
+    // rows_pad of an operand's pieces.
     typedef const __attribute__((address_space(1))) void *global_address;
     typedef __attribute__((address_space(3))) void *lds_address;
-    const gram_chunk *src[4];
-    i64 advance[4];
-    int dst[4];
+    constexpr int COPIES = Tile::COPIES;
+    const gram_chunk *src[COPIES];
+    i64 advance[COPIES];
+    int dst[COPIES];
     {
         const gram_chunk *pieces_a = args.pieces_a + batch * args.pieces_a_bs + m0;
         const gram_chunk *pieces_c = args.pieces_c + batch * args.pieces_c_bs + o0;
@@ -144,22 +148,32 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
             advance[j] = (i64)8 * args.rows_pad_a;
             dst[j] = run * NGF_TILE_M;
         }
-        const int c_copy = O_BLOCKS == 1 ? (wave & 1) : wave;                   // 64 chunks of the step's C each
-        const int c_run = O_BLOCKS == 1 ? 4 * c_copy + q : 2 * c_copy + (lane >> 5);
-        const int c_row = O_BLOCKS == 1 ? r : (lane & 31);
-        src[2] = pieces_c + (i64)c_run * args.rows_pad_c + c_row;
-        advance[2] = (i64)8 * args.rows_pad_c;
-        dst[2] = Tile::A_CHUNKS + 64 * c_copy;
+        if constexpr (O_BLOCKS == 4) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {                                       // 64 chunks of the step's C each: one run
+                const int run = 2 * wave + j;
+                src[2 + j] = pieces_c + (i64)run * args.rows_pad_c + lane;
+                advance[2 + j] = (i64)8 * args.rows_pad_c;
+                dst[2 + j] = Tile::A_CHUNKS + 64 * run;
+            }
+        } else {
+            const int c_copy = O_BLOCKS == 1 ? (wave & 1) : wave;               // 64 chunks of the step's C each
+            const int c_run = O_BLOCKS == 1 ? 4 * c_copy + q : 2 * c_copy + (lane >> 5);
+            const int c_row = O_BLOCKS == 1 ? r : (lane & 31);
+            src[2] = pieces_c + (i64)c_run * args.rows_pad_c + c_row;
+            advance[2] = (i64)8 * args.rows_pad_c;
+            dst[2] = Tile::A_CHUNKS + 64 * c_copy;
+        }
         // 8 rows of B per copy: lane -> row lane / 8, 16 bytes number lane % 8 of the step's 128
-        const int b_copy = O_BLOCKS == 1 ? wave : (wave & 1);
+        const int b_copy = O_BLOCKS == 1 ? wave : O_BLOCKS == 2 ? (wave & 1) : 0;
         const float *b_row = args.b_padded + batch * args.b_padded_bs + (i64)(n0 + 8 * b_copy + (lane >> 3)) * args.k_pad + 4 * (lane & 7);
-        src[3] = reinterpret_cast<const gram_chunk *>(b_row);
-        advance[3] = NGF_STEP_K / 4;
-        dst[3] = Tile::A_CHUNKS + Tile::C_CHUNKS + 64 * b_copy;
+        src[COPIES - 1] = reinterpret_cast<const gram_chunk *>(b_row);
+        advance[COPIES - 1] = NGF_STEP_K / 4;
+        dst[COPIES - 1] = Tile::A_CHUNKS + Tile::C_CHUNKS + 64 * b_copy;
     }
     auto copy_step = [&](auto into) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < COPIES; j++) {
             const unsigned lds_byte = (unsigned)(unsigned long)(lds_address)(buffer(into) + dst[j]);
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                          :
@@ -239,7 +253,7 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
         }
         // the wave's own copies of the next step have arrived (the four of the step after it may
         // still be under way); behind the barrier everybody's have, and this step's buffer is free
-        __builtin_amdgcn_s_waitcnt(0x0F74);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | COPIES);            // vmcnt(COPIES)
         __syncthreads();
         copy_step(which);
     };
@@ -247,7 +261,7 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
     copy_step(GramStep<0>{});
     copy_step(GramStep<1>{});
     copy_step(GramStep<2>{});
-    __builtin_amdgcn_s_waitcnt(0x0F78);                     // vmcnt(8): step 0 has arrived
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * COPIES));      // vmcnt(2 COPIES): step 0 has arrived
     __syncthreads();
     for (int done = 0;;) {
         step(GramStep<0>{});

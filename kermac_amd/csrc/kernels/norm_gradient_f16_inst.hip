@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "../host/host_common.hpp"
 #include "launch.hpp"
@@ -87,7 +88,7 @@ bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)
     layout->b_padded = place(cursor, layout->b_batches * layout->b_padded_bs * 4);
     layout->bytes = cursor;
     // blockIdx.z = batch entry x chunk of outputs, blockIdx.y = tile of at least 16 n
-    const int64_t grid_z = static_cast<int64_t>(p->l) * (p->o / 32 + 1);
+    const int64_t grid_z = static_cast<int64_t>(p->l) * (p->o / 64 + 1);
     if (grid_z > 65535 || layout->n_pad / 16 > 65535) return false;
     return true;
 }
@@ -160,25 +161,25 @@ hipError_t launch_norm_gradient_f16(const kmc_norm_gradient_params *p, bool a_ve
     args.b_padded_bs = layout.b_batches > 1 ? layout.b_padded_bs : 0;
     args.rows_pad_a = layout.a.rows_pad; args.rows_pad_c = layout.c.rows_pad;
     args.k_pad = layout.k_pad; args.steps = layout.steps;
-    // Outputs in chunks of 32 on the 16 n x 32 o tile; what is left, if at most 16, on the 32 n x 16 o tile.
-    const int wide_chunks = p->o > 16 ? p->o / 32 + (p->o % 32 > 16 ? 1 : 0) : 0;
-    const int wide_outputs = wide_chunks * 32 < p->o ? wide_chunks * 32 : (wide_chunks ? p->o : 0);
+    // Outputs in chunks of 64 on the 8 n x 64 o tile while more than 32 are left, then one chunk of 32 on the
+    // 16 n x 32 o tile for 17 to 32 of them, or the 32 n x 16 o tile for up to 16.
+    int wide_chunks = p->o / 64;
+    int left = p->o % 64;
+    if (left > 32) { wide_chunks += 1; left = 0; }
     const unsigned tiles_m = (p->m + kmc::NGF_TILE_M - 1) / kmc::NGF_TILE_M;
+    auto run = [&](auto blocks, int o_begin, int chunks) {
+        using Tile = kmc::GradientF16Tile<decltype(blocks)::value>;
+        args.o_begin = o_begin;
+        args.g.o_chunks = chunks;
+        const dim3 grid(tiles_m, (p->n + Tile::TILE_N - 1) / Tile::TILE_N, static_cast<unsigned>(p->l) * chunks);
+        return launch(kmc::norm_gradient_l1_f16<decltype(blocks)::value>, grid, dim3(kmc::NGF_THREADS), stream, args);
+    };
     if (wide_chunks) {
-        using Tile = kmc::GradientF16Tile<2>;
-        args.o_begin = 0;
-        args.g.o_chunks = wide_chunks;
-        const dim3 grid(tiles_m, (p->n + Tile::TILE_N - 1) / Tile::TILE_N, static_cast<unsigned>(p->l) * wide_chunks);
-        status = launch(kmc::norm_gradient_l1_f16<2>, grid, dim3(kmc::NGF_THREADS), stream, args);
+        status = run(std::integral_constant<int, 4>{}, 0, wide_chunks);
         if (status != hipSuccess) return status;
     }
-    if (wide_outputs < p->o) {
-        using Tile = kmc::GradientF16Tile<1>;
-        args.o_begin = wide_outputs;
-        args.g.o_chunks = 1;
-        const dim3 grid(tiles_m, (p->n + Tile::TILE_N - 1) / Tile::TILE_N, static_cast<unsigned>(p->l));
-        status = launch(kmc::norm_gradient_l1_f16<1>, grid, dim3(kmc::NGF_THREADS), stream, args);
-    }
+    if (left > 16) status = run(std::integral_constant<int, 2>{}, p->o - left, 1);
+    else if (left > 0) status = run(std::integral_constant<int, 1>{}, p->o - left, 1);
     if (status == hipSuccess) *taken = true;
     return status;
 }

@@ -39,9 +39,10 @@ def workspace_bytes(a, b, c, d, p=1.0):
 @pytest.mark.parametrize("M,N,O,K", [(1, 1, 1, 1), (70, 33, 3, 17), (64, 32, 16, 32), (65, 31, 5, 50), (200, 40, 20, 35),
                                      (130, 64, 8, 100), (129, 66, 1, 48), (256, 64, 16, 64), (67, 35, 2, 19), (96, 24, 17, 20),
                                      (80, 20, 33, 33), (64, 16, 90, 16), (300, 70, 16, 1000),
-                                     # 17 and more outputs: tiles of 16 n x 32 o, what is left beyond whole tiles on 32 n x 16 o
+                                     # 17 and more outputs: tiles of 16 n x 32 o and 8 n x 64 o, what is left beyond whole
+                                     # tiles of 64 on the narrower ones
                                      (70, 40, 32, 40), (130, 20, 40, 64), (64, 33, 64, 32), (50, 17, 49, 20), (200, 15, 24, 70),
-                                     (65, 31, 25, 200)])
+                                     (65, 31, 25, 200), (60, 12, 70, 40), (40, 9, 130, 33), (33, 7, 90, 64)])
 def test_gradient_shapes(device, f16_route, M, N, O, K):
     g = torch.Generator().manual_seed(M + 2 * N + 3 * O + 5 * K)
     a = (torch.rand(K, M, generator=g) - 0.3).to(device)        # weights of both signs
