@@ -178,7 +178,7 @@ def run_kernel_coefficients(
 # built once by kmc_build_kernel (whatever kernel this descriptor and l2 mode launch for a stored
 # matrix) is contracted with all columns at 4 bytes of traffic per element.  Laplace kernel on L1
 # distances, L = 4, M = N = 16384, K = 256: O = 65 .. 128 22.1 -> 11.8 .. 12.0 ms, O = 256 44.0 -> 14.6 ms,
-# O = 1000 176 -> 30.7 ms; p = 1.3 norm, M = 1000, N = 20000, K = 784, O = 300: 15.1 -> 3.2 ms.
+# O = 1000 176 -> 18.7 ms (the panels contracted from fp16 pieces, below); p = 1.3 norm, M = 1000, N = 20000, K = 784, O = 300: 15.1 -> 3.2 ms.
 _PANEL_BYTES = 1 << 30
 _FUSED_COLUMNS_PER_WALK = 64
 _MANY_COLUMNS_MIN_ELEMENTS = 1e6        # below, the three launches cost what the second walk does (500 x 500, O = 100: 54 against 41 us)
@@ -312,7 +312,8 @@ def _run_in_panels(plan, shape, stream, device, debug):
     block.n, block.c_ld, block.c_bs = rows, ld, rows * ld
     try:
         panel = torch.empty(L * rows * ld, dtype=torch.float32, device=device)
-        partial = torch.empty((parts, L, M, O), dtype=torch.float32, device=device) if parts > 1 else None
+        product = _contraction_by_pieces(plan, rows, ld, panel, device)
+        partial = torch.empty((parts, L, M, O), dtype=torch.float32, device=device) if parts > 1 and product is None else None
     except torch.cuda.OutOfMemoryError:
         return False
     block.c = panel.data_ptr()
@@ -321,7 +322,8 @@ def _run_in_panels(plan, shape, stream, device, debug):
         return False
     if debug:
         print(f"(Kermac Debug) Kernel matrix x coefficients in {panels} panels of {rows} centres, "
-              + (f"{splits} partial products each" if splits else "added to the result one after the other"))
+              + ("contracted from fp16 pieces" if product is not None else
+                 f"{splits} partial products each" if splits else "added to the result one after the other"))
     row_major_b = block.b_majorness == _backend.ROW_MAJOR
     contraction = _backend.MatrixCoefficientsParams()
     contraction.m, contraction.o, contraction.l = M, O, L
@@ -352,6 +354,20 @@ def _run_in_panels(plan, shape, stream, device, debug):
             _backend.build_kernel_jit(function, block, stream)
         if route:
             block.flags |= _backend.FLAG_GRAM_A_KEPT             # the rows are the same for every panel: split once
+        if product is not None:
+            # out[m, o] (+)= sum_n panel[n, m] coef[n, o] as a product of fp16 pieces (below)
+            pieces, sums, _ = product
+            pieces.k, pieces.b_bs = count, count * ld
+            pieces.a = params.coef + 4 * n0 * params.coef_ld
+            if index == 0:
+                pieces.c, pieces.c_ld, pieces.c_bs = params.out, params.out_ld, params.out_bs
+            else:
+                pieces.c, pieces.c_ld, pieces.c_bs = sums.data_ptr(), O, M * O
+            _backend.build_kernel(pieces, stream)
+            if index:
+                target = plan.out if plan.out.dim() == 3 else plan.out.unsqueeze(0)
+                target.add_(sums)
+            continue
         contraction.n, contraction.matrix_bs = count, count * ld
         contraction.coef = params.coef + 4 * n0 * params.coef_ld
         if partial is not None:
@@ -361,8 +377,61 @@ def _run_in_panels(plan, shape, stream, device, debug):
         _backend.matrix_times_coefficients(contraction, stream)
     if partial is not None:
         _sum_partials(partial, plan.out)
-    plan.keepalive += [panel, partial, workspace]
+    plan.keepalive += [panel, partial, workspace, product]
     return True
+
+
+# Hundreds of coefficient columns: kmc_matrix_times_coefficients multiplies on the fp32 matrix instruction and is
+# bound by it from about 128 columns on (O = 1000 above: 20 of 31 ms).  The contraction of a panel is itself a
+# sum of products, out[m, o] = sum_n panel[n, m] coef[n, o], with both operands stored the way kmc_build_kernel reads
+# them (m and o contiguous), so from _PIECES_MIN_COLUMNS columns on it runs on kmc_build_kernel's route for sums of
+# products (KMC_FLAG_DOT_PIECES: two fp16 pieces per value, scale per row m and o, error below 3 * 2^-22 sum_n |k c|)
+# into the result for the first panel and into a buffer that is added to the result for the others.  Gaussian
+# kernel, fp32 contraction -> pieces: L = 4, M = N = 16384, K = 256 at O = 256 9.6 -> 8.1 ms, O = 512 15.6 -> 9.4,
+# O = 1000 25.5 -> 12.0; M = 10000, N = 100000, K = 784, O = 1000 28.5 -> 17.2 ms.  The split of a panel costs what
+# its fp32 contraction with 64 columns does, and the product runs in tiles of 256 x 256 over (o, m): not below 256
+# columns (O = 128: 6.7 -> 7.8 ms) nor below 128 tiles over the batch (M = 10000, O = 256, 40 tiles: 12.3 -> 16.1 ms;
+# M = 2000, O = 1000, 32 tiles: 1.2 -> 2.0 ms).  KERMAC_AMD_COEFFICIENT_PIECES_MIN_COLUMNS replaces both conditions
+# by a number of columns (tests send small shapes this way with 1).
+_PIECES_MIN_COLUMNS = 256
+_PIECES_MIN_TILES = 128
+
+
+def _contraction_by_pieces_pays(L, M, O):
+    forced = os.environ.get("KERMAC_AMD_COEFFICIENT_PIECES_MIN_COLUMNS")
+    if forced is not None:
+        return O >= int(forced)
+    return O >= _PIECES_MIN_COLUMNS and -(-O // 256) * -(-M // 256) * L >= _PIECES_MIN_TILES
+
+
+def _contraction_by_pieces(plan, rows, ld, panel, device):
+    """(parameter block, buffer for the sums of a panel, workspace) of the contraction as a product of fp16
+    pieces; None when kmc_matrix_times_coefficients contracts the panels."""
+    from .build_a_kernel import _attach_gram_workspace
+
+    L, M, N, O = plan.L, plan.M, plan.N, plan.O
+    if not _contraction_by_pieces_pays(L, M, O):
+        return None
+    params = plan.params
+    block = _backend.BuildKernelParams()
+    block.inner_operator, block.inner_power, block.outer_power, block.kernel_type = _backend.OP_DOT, _backend.POW_NOOP, 0, 0
+    block.a_majorness = block.b_majorness = _backend.COL_MAJOR
+    block.flags = _backend.FLAG_DOT_PIECES | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
+    # the product the library sees: rows o of the coefficients against rows m of the panel, contraction over n;
+    # its result C(o, m) at c[o + m c_ld] is out[m, o]
+    block.m, block.n, block.k, block.l = O, M, min(rows, N), L
+    block.a, block.a_ld, block.a_bs = params.coef, params.coef_ld, params.coef_bs
+    block.b, block.b_ld, block.b_bs = panel.data_ptr(), ld, min(rows, N) * ld
+    block.c, block.c_ld, block.c_bs = params.out, params.out_ld, params.out_bs
+    block.epsilon = 0.0
+    workspace = _attach_gram_workspace(block, device)
+    if workspace is None:
+        return None
+    try:
+        sums = torch.empty((L, M, O), dtype=torch.float32, device=device) if N > rows else None
+    except torch.cuda.OutOfMemoryError:
+        return None
+    return block, sums, workspace
 
 
 def _sum_partials(partial, out):

@@ -301,3 +301,31 @@ def test_more_than_64_columns_of_a_run_time_compiled_descriptor(device, monkeypa
     monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", "0")
     fused = kermac.run_kernel(desc, a, b, coefficients=coef)
     assert_close_to_truth(fused, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what="the same on the fused kernel")
+
+
+@pytest.mark.parametrize("M,N,K,O,L", [(300, 1100, 24, 70, 2), (130, 700, 40, 5, 1), (257, 520, 17, 33, 3)])
+def test_contraction_from_fp16_pieces(device, monkeypatch, capsys, M, N, K, O, L):
+    """Hundreds of columns on many rows contract their panels as a product of fp16 pieces
+    (kmc_build_kernel's route for sums of products) instead of kmc_matrix_times_coefficients;
+    KERMAC_AMD_COEFFICIENT_PIECES_MIN_COLUMNS=1 sends these small shapes that way.  Several panels
+    (the first is stored, the others are added), padded and misaligned coefficients, a padded result."""
+    from kermac_amd import kernel_coefficients as module
+    g = torch.Generator().manual_seed(M + N + K + O)
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PIECES_MIN_COLUMNS", "1")
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PANEL_BYTES", str(4 * L * 512 * (-(-M // 4) * 4)))       # panels of 512 centres
+    monkeypatch.setattr(module, "_FUSED_COLUMNS_PER_WALK", 0)                # any number of columns in plain panels
+    monkeypatch.setattr(module, "_MANY_COLUMNS_MIN_ELEMENTS", 0.0)
+    a = make_operand(L, M, K, False, device, g)
+    b = make_operand(L, N, K, True, device, g)
+    coef = torch.randn(L, N, O + 3, generator=g).to(device)[..., 1:O + 1]    # rows neither aligned nor a multiple of 4 long
+    out = torch.full((L, M, O + 1), 9.0, device=device)
+    for descriptor, names, kw in ((kermac.kernel_descriptor_laplace_l1, ("DIFF", "ABS", "NOOP", "LAPLACE"), {"bandwidth": 9.0}),
+                                  (GAUSSIAN, ("DIFF", "SQUARE", "NOOP", "GAUSSIAN"), {"bandwidth": 5.0})):
+        got = kermac.run_kernel(descriptor, a, b, out=out[..., :O], coefficients=coef, debug=True, **kw)
+        printed = capsys.readouterr().out
+        assert f"{PANELS} {-(-N // 512)} panels of 512 centres, contracted from fp16 pieces" in printed, printed
+        truth = oracle.run_kernel_coefficients(*names, a.cpu().contiguous(), b.cpu().contiguous(), coef.cpu().contiguous(), **kw)
+        assert_close_to_truth(got, truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"{names} contracted from pieces")
+        assert torch.all(out[..., O] == 9.0), "wrote outside the out view"
+        assert torch.equal(got, kermac.run_kernel(descriptor, a, b, coefficients=coef, **kw)), "two runs differ"
+

@@ -638,6 +638,18 @@ def test_auto_mode_of_the_coefficient_product_without_a_gpu(monkeypatch):
     assert plan(4096, 4096, 256, 32, descriptor=kermac.kernel_descriptor_laplace_l1).params.kernel.flags & _backend.FLAG_L2_GRAM == 0
 
 
+def test_which_products_contract_their_panels_from_fp16_pieces(monkeypatch):
+    """At least 256 coefficient columns and 128 tiles of 256 x 256 over (columns, rows, batch); the
+    environment variable replaces both conditions by a number of columns."""
+    from kermac_amd.kernel_coefficients import _contraction_by_pieces_pays as pays
+    monkeypatch.delenv("KERMAC_AMD_COEFFICIENT_PIECES_MIN_COLUMNS", raising=False)
+    assert not pays(4, 16384, 128) and pays(4, 16384, 256)
+    assert not pays(1, 10000, 256) and pays(1, 10000, 1000)             # 40 and 160 tiles
+    assert not pays(1, 2000, 1000)                                      # 32 tiles
+    monkeypatch.setenv("KERMAC_AMD_COEFFICIENT_PIECES_MIN_COLUMNS", "5")
+    assert pays(1, 10, 5) and not pays(4, 16384, 4)
+
+
 def test_matrix_times_coefficients_checks_its_arguments_before_any_device_call():
     """kmc_matrix_times_coefficients: extents, strides and the l * n_splits limit are checked
     first, and an empty product returns without touching a device."""
