@@ -329,3 +329,20 @@ def test_contraction_from_fp16_pieces(device, monkeypatch, capsys, M, N, K, O, L
         assert torch.all(out[..., O] == 9.0), "wrote outside the out view"
         assert torch.equal(got, kermac.run_kernel(descriptor, a, b, coefficients=coef, **kw)), "two runs differ"
 
+
+
+def test_headline_shape_with_256_columns(device, capsys):
+    """The fused benchmark shape with 256 coefficient columns, by the rules alone: panels on the
+    fp16 matrix instruction, each contracted as a product of fp16 pieces; float64 slabs."""
+    torch.manual_seed(6)
+    L, K, NX, MZ, O = 4, 256, 16384, 16384, 256
+    x = torch.rand(L, K, NX, device=device) * 2 - 1
+    z = torch.rand(K, MZ, device=device) * 2 - 1
+    coef = torch.randn(L, MZ, O, device=device)
+    out = torch.empty(L, NX, O, device=device)
+    kermac.run_kernel(GAUSSIAN, x.transpose(1, 2), z.t(), out=out, bandwidth=9.0, coefficients=coef, debug=True)
+    assert f"{PANELS} 4 panels of 4096 centres, contracted from fp16 pieces" in capsys.readouterr().out
+    for l, rows in ((0, slice(0, 96)), (3, slice(16300, 16384))):
+        d2 = torch.cdist(x[l, :, rows].t().double(), z.t().double(), p=2.0) ** 2
+        truth = torch.exp(-d2 / (2 * 9.0 ** 2)) @ coef[l].double()
+        assert_close_to_truth(out[l, rows], truth, rtol=1e-5, atol=atol_for(truth, 1e-5), what=f"256 columns, slab of batch {l}")
