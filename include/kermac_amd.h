@@ -197,6 +197,8 @@ typedef struct kmc_build_kernel_params {
  * a panel against itself the tiles on and below the diagonal count, and the panel is split once;
  * squared differences of operands that both have k contiguous take the route from 48 tiles, k = 256 and
  * tiles * k = 36864 on, whatever the shape of a batch entry, unless m or n is at most 128;
+ * sums of products take it from k = 128, 64 tiles and tiles * k = 65536 on with at most 20 % padding, and from
+ * k = 256 on from 32 tiles (64 for l = 1) and tiles * k = 24576 on whatever the padding;
  * KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE sets the size rules aside).  About 1.1 times the bytes of the
  * operands.  No counterpart in the reference. */
 int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes);

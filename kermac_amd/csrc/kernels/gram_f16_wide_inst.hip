@@ -47,7 +47,11 @@ struct WideLayout {
 // Sums of products have no one-step matrix-core kernel to fall back to: the alternative is the direct
 // kernel, which the route beats much earlier (direct / route time: 64 tiles 1.04 .. 1.42 at K = 1024,
 // 0.82 .. 1.04 at K = 512; 256 tiles 1.25 at K = 256, 0.86 at K = 128; 1024 tiles 1.17 .. 1.35 at K = 128,
-// 0.91 .. 1.02 at K = 64; 64 batch entries of 2 x 2 tiles 1.5, 118 x 2 tiles 1.9).
+// 0.91 .. 1.02 at K = 64; 64 batch entries of 2 x 2 tiles 1.5, 118 x 2 tiles 1.9).  From K = 256 on it is
+// taken from 32 tiles and tiles * k = 24576 on whatever the padding (8 entries of 512 x 512 x 784 1.3 .. 1.4, at
+// K = 3072 1.7 .. 1.9; 4 of 1000 x 1000 x 784 1.7; 144 tiles at K = 256 1.2 .. 1.3; 300 x 30000, 41 % of the tiles
+// padding, 1.1 .. 1.2 at K = 256 and 1.7 .. 1.9 beyond; at K = 256 with 64 tiles 0.8 .. 0.9), but a single problem
+// only from 64 tiles on: the direct path cuts such a call over k (1500 x 1500, 36 tiles: 0.77 .. 0.84).
 //
 // Operands with k contiguous (row-major, as torch allocates them): the one-step kernels stage such operands
 // more slowly, the route splits them once and walks pieces whose layout is its own, so it pays much earlier
@@ -56,12 +60,14 @@ struct WideLayout {
 // 2 x 118 tiles 1.07 at K = 256, 1.3 at K = 784; 36 tiles 0.9 / 1.2; 32 tiles as 8 entries of 2 x 2 0.75 / 0.8;
 // K = 128 never above 1).  Not for a dimension that half a tile holds, where the 128 x 128 tiles of the
 // one-step kernels waste half as much (100 x 50000: 0.87 at K = 784, 4 entries 0.73; 128 x 20000 0.8).
-bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t tiles, int k, bool products, bool k_contiguous)
+bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t tiles, int k, bool products, bool k_contiguous,
+               bool batched)
 {
     const char *text = std::getenv("KERMAC_AMD_WIDE_MIN_TILES");
     const int forced = text ? std::atoi(text) : 0;
     if (forced > 0) return tiles >= forced && k >= 1;
     if (k_contiguous && !products && k >= 256 && tiles >= 48 && tiles * k >= 36864 && m > kmc::GW_TILE / 2 && n > kmc::GW_TILE / 2) return true;
+    if (products && k >= 256 && tiles * k >= 24576 && tiles >= (batched ? 32 : 64)) return true;
     if (products)
         return k >= 128 && tiles >= 64 && tiles * k >= 65536 && 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
     // (from 768 tiles on the route is as fast as the one-step kernel also for the shortest contractions
@@ -123,7 +129,7 @@ bool wide_layout(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
                                          : static_cast<int64_t>(layout->tiles_m) * layout->tiles_n;
     const bool k_contiguous = p->a_majorness == KMC_ROW_MAJOR && p->b_majorness == KMC_ROW_MAJOR;
     const bool asked_for = (p->flags & KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE) && args.k >= 1;
-    if (!asked_for && !wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k, products, k_contiguous)) return false;
+    if (!asked_for && !wide_pays(args.m, args.n, layout->tiles_m, layout->tiles_n, tiles * args.l, args.k, products, k_contiguous, args.l > 1)) return false;
     // an operand that is the same for every batch entry is split once, unless the centre differs
     // (products have no centre: the caller's parameter block carries none into `args`)
     const bool one_centre = products || !args.centre || args.centre_bs == 0;

@@ -361,6 +361,11 @@ def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
     assert chosen(2000, 2000, 784, rows_contiguous=True) == core              # the split one-step kernel there
     assert chosen(8192, 4096, 512, dot=True) == _backend.FLAG_DOT_PIECES
     assert chosen(300, 300, 512, dot=True) == 0
+    # from K = 256 on: 32 tiles over a batch, 64 of a single problem (which the direct path would cut over k), any padding
+    assert chosen(512, 512, 784, l=8, dot=True) == _backend.FLAG_DOT_PIECES
+    assert chosen(1500, 1500, 784, dot=True) == 0 and chosen(2000, 2000, 784, dot=True) == _backend.FLAG_DOT_PIECES
+    assert chosen(300, 30000, 784, dot=True) == _backend.FLAG_DOT_PIECES
+    assert chosen(1000, 1000, 256, l=4, dot=True) == 0                          # tiles * k below 24576
     monkeypatch.setenv("KERMAC_AMD_L2_WORKSPACE", "0")
     assert chosen(8192, 4096, 512, dot=True) == 0 and chosen(10000, 10000, 96) == 0 and chosen(10000, 10000, 256) == core
 
