@@ -301,7 +301,8 @@ typedef struct kmc_norm_gradient_params {
 
 /* Bytes of workspace that kmc_norm_kernel_gradient would use for these parameters, 0 when it would
  * not use one.  KMC_NORM_L1: at least 3 outputs, n >= 24 and m * n * k * l terms of at least
- * 6.4e9 / min(o, 16) (4e8 at 16 outputs); about 1.1 times the bytes of a, b and c.  KMC_NORM_L2:
+ * 6.4e9 / o (4e8 at 16 outputs), with more than 16 outputs of at least 1.5e7; about 1.1 times the
+ * bytes of a, b and c.  KMC_NORM_L2:
  * when a model of both times favours the route by 15 % (tiles of 256 x 256 over m and o * n, in
  * both directions, and a contraction of about 512 or more); about 4 (m + 2 o n) k bytes.
  * KMC_NORM_P: never.  No counterpart in the reference. */

@@ -66,7 +66,11 @@ bool f16_pays(const kmc_norm_gradient_params *p)
     const double forced = text ? std::atof(text) : 0.0;
     const double terms = static_cast<double>(p->m) * p->n * p->k * p->l;
     if (forced > 0.0) return terms >= forced;
-    return p->o >= 3 && p->n >= 24 && terms * (p->o < 16 ? p->o : 16) >= 6.4e9;
+    // more than 16 outputs: the wider tiles of the route share the sign work between blocks of outputs, while the
+    // fp32 kernels go to their 32-column tiles (O = 32: 98 against 75 us at 1.7e7 terms, 187 against 128 at 2.7e8;
+    // O = 128: 101 against 70 and 588 against 206)
+    if (p->o > 16) return p->n >= 24 && terms >= 1.5e7;
+    return p->o >= 3 && p->n >= 24 && terms * p->o >= 6.4e9;
 }
 
 bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)

@@ -578,6 +578,8 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert gradient(8192, 512, 1, 8192, norm_type=1) > 0                             # one output: the fp32 kernel is slow there
     assert gradient(8192, 512, 2, 8192) == 0                                         # two outputs: the vector kernel
     assert gradient(1024, 64, 16, 1024) == 0                                         # 6.7e7 terms
+    assert gradient(1024, 64, 17, 1024) > 0 and gradient(512, 64, 64, 512) > 0       # more than 16 outputs: from 1.5e7 terms on
+    assert gradient(256, 64, 64, 512) == 0                                           # 8.4e6 terms
     assert gradient(8192, 16, 16, 8192) == 0                                         # half of every tile of 32 columns unused
     assert gradient(2048, 128, 4, 2048) == 0 and gradient(2048, 128, 16, 2048) > 0   # 5.4e8 terms: enough for 16 outputs, not for 4
     monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
