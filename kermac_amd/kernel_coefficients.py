@@ -194,17 +194,15 @@ def _panel_splits(M, O, L, rows):
 
 
 def _products_in_panels(plan):
-    """Sums of products (linear and polynomial kernels) have the same route: as run_kernel decides
-    for a stored matrix, large ones in the l2 modes "auto" and "gram_bf16"."""
-    from .build_a_kernel import _L2_AUTO_MIN_TERMS, _l2_current
+    """Sums of products (linear and polynomial kernels) have the same route, in the l2 modes "auto" and
+    "gram_bf16" (_panel_shape decides which problems take it)."""
+    from .build_a_kernel import _l2_current
 
     kernel = plan.params.kernel
     if kernel.inner_operator != _backend.OP_DOT or kernel.inner_power != _backend.POW_NOOP:
         return False
     l2 = _l2_current()
-    if l2["mode"] not in ("auto", "gram_bf16") or plan.K < l2["min_k"]:
-        return False
-    return l2["mode"] != "auto" or float(plan.L) * plan.M * plan.N * plan.K >= _L2_AUTO_MIN_TERMS
+    return l2["mode"] in ("auto", "gram_bf16") and plan.K >= l2["min_k"]
 
 
 # The matrix-core variant of the fused kernel holds 32 coefficient columns per workgroup where the
@@ -263,6 +261,34 @@ def _auto_panels_of_any_size(plan):
     return plan.K >= _AUTO_PANEL_LONG_K or (plan.K >= _AUTO_PANEL_MID_K and tiles >= _AUTO_PANEL_MID_TILES)
 
 
+# Sums of products: the fused kernel walks them more slowly than squared differences (it has no matrix-core
+# variant), so panels pay earlier (fused kernel / panels): any number of tiles from K = 784 on (500 x 500: 1.4 at
+# K = 784, 2.1 at K = 3072), and with more than 32 coefficient columns any contraction from 1e7 elements on
+# (4096 x 4096 x 64 1.2, 4 x 4096 x 4096 x 64 1.55, 1000 x 20000 x 128 1.6; 2000 x 2000 x 64 0.54), both with 60 % of
+# the tiles' area used;
+# few rows against many centres stay fused with up to 32 columns even where the library would take the route
+# (100 x 50000 x 256: 0.74, x 784: 0.86).
+_AUTO_PRODUCT_PANEL_ANY_TILES_K = 784
+_AUTO_PRODUCT_PANEL_MIN_ELEMENTS = 1e7
+
+
+def _auto_product_panels(plan, library_takes_them):
+    """l2 mode "auto", sums of products: None (fused kernel), False (panels as the library's rule has them) or
+    True (panels of any size)."""
+    tiles_m, tiles_n = -(-plan.M // 256), -(-plan.N // 256)
+    used = plan.M * plan.N / (65536.0 * tiles_m * tiles_n)
+    many_columns = plan.O > _AUTO_FUSED_MAX_COLUMNS
+    if used < _AUTO_PANEL_MIN_USED and not many_columns:
+        return None
+    if library_takes_them:
+        return False
+    if used < _AUTO_PANEL_MIN_USED:
+        return None
+    if plan.K >= _AUTO_PRODUCT_PANEL_ANY_TILES_K:
+        return True
+    return True if many_columns and float(plan.L) * plan.M * plan.N >= _AUTO_PRODUCT_PANEL_MIN_ELEMENTS else None
+
+
 def _panel_shape(plan, route):
     """(rows, panels, ld, splits, flags) of the product panel by panel (above); None when this problem
     stays with the fused kernel.  `route`: the flag of kmc_build_kernel's route through a workspace
@@ -275,7 +301,9 @@ def _panel_shape(plan, route):
         return None
     # l2 mode "gram" asks for the fp32 matrix instruction; the panels of a route are built from fp16 pieces
     mode = _l2_current()["mode"]
-    if route and (mode not in ("auto", "gram_bf16") or (mode == "auto" and plan.K < _AUTO_PANEL_MIN_K)):
+    if route and mode not in ("auto", "gram_bf16"):
+        return None
+    if route == _backend.FLAG_L2_GRAM_BF16 and mode == "auto" and plan.K < _AUTO_PANEL_MIN_K:
         return None
     ld = -(-M // 4) * 4                                          # rows of the panel start on 16 bytes
     rows = min(N, max(256, budget // (4 * L * ld) // 256 * 256))
@@ -285,14 +313,21 @@ def _panel_shape(plan, route):
     block = _backend.BuildKernelParams.from_buffer_copy(plan.params.kernel)
     block.flags |= route
     block.n, block.c, block.c_ld, block.c_bs = rows, 256, ld, rows * ld      # c: any address, for the query
-    if route and _backend.gram_workspace_bytes(block) == 0:
-        # panels of this shape would not take the fast route by themselves
-        if mode != "auto" or route != _backend.FLAG_L2_GRAM_BF16 or not _auto_panels_of_any_size(plan):
+    if route:
+        taken = _backend.gram_workspace_bytes(block) > 0       # by the library's rule, made for stored matrices
+        if mode != "auto":
+            any_size = None if not taken else False
+        elif route == _backend.FLAG_DOT_PIECES:
+            any_size = _auto_product_panels(plan, taken)
+        else:
+            any_size = False if taken else (True if _auto_panels_of_any_size(plan) else None)
+        if any_size is None:
             return None
-        route |= _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
-        block.flags |= route
-        if _backend.gram_workspace_bytes(block) == 0:
-            return None
+        if any_size:
+            route |= _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
+            block.flags |= route
+            if _backend.gram_workspace_bytes(block) == 0:
+                return None
     splits = _panel_splits(M, O, L, rows)
     if panels * splits > 1 and 4 * panels * splits * L * M * O > _PANEL_MAX_PARTIAL_BYTES:
         splits = 0              # too many partial products to keep: every panel is added to the result as it comes

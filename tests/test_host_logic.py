@@ -599,7 +599,8 @@ def test_auto_mode_of_the_coefficient_product_without_a_gpu(monkeypatch):
     def plan(M, N, K, O, L=1, k_contiguous=True, descriptor=kermac.kernel_descriptor_laplace_l2):
         a = torch.empty(L, M, K) if k_contiguous else torch.empty(L, K, M).transpose(1, 2)
         b = torch.empty(L, N, K) if k_contiguous else torch.empty(L, K, N).transpose(1, 2)
-        return module._plan_run_kernel_coefficients(descriptor, a, b, torch.empty(L, N, O), None, None, None, None, 2.0,
+        bandwidth = None if descriptor._kernel_type is kermac.KernelType.NONE else 2.0
+        return module._plan_run_kernel_coefficients(descriptor, a, b, torch.empty(L, N, O), None, None, None, None, bandwidth,
                                                     None, None, 0, 0, require_device=False)
 
     def chosen(*shape, **kw):
@@ -633,8 +634,25 @@ def test_auto_mode_of_the_coefficient_product_without_a_gpu(monkeypatch):
         assert not p.l2_auto and module._panel_shape(p, _backend.FLAG_L2_GRAM_BF16) is None
         p = plan(8192, 8192, 256, 32, k_contiguous=False)
         assert module._panel_shape(p, _backend.FLAG_L2_GRAM_BF16)[4] == _backend.FLAG_L2_GRAM_BF16
+    # sums of products have rules of their own (their fused kernel has no matrix-core variant)
+    products = kermac.KernelDescriptor(kermac.InnerOperator.DOT, kermac.PowerType.NOOP, kermac.PowerType.NOOP, kermac.KernelType.NONE)
+
+    def product_panels(*shape, **kw):
+        p = plan(*shape, descriptor=products, **kw)
+        if not module._products_in_panels(p):
+            return None
+        panels = module._panel_shape(p, _backend.FLAG_DOT_PIECES)
+        return None if panels is None else bool(panels[4] & any_size)
+
+    assert product_panels(8192, 8192, 512, 8) is False                                 # the library's rule takes them
+    assert product_panels(500, 500, 784, 8) is True and product_panels(500, 500, 256, 8) is None
+    assert product_panels(4096, 4096, 64, 40) is True and product_panels(4096, 4096, 64, 32) is None
+    assert product_panels(2000, 2000, 64, 40) is None                                  # 4e6 elements
+    assert product_panels(100, 50000, 784, 8) is None and product_panels(100, 50000, 784, 40) is False
+    assert product_panels(4096, 4096, 32, 40) is None                                  # K below 64
     with kermac.l2_mode("direct"):
         assert plan(4096, 4096, 256, 32).params.kernel.flags & _backend.FLAG_L2_GRAM == 0
+        assert product_panels(8192, 8192, 512, 8) is None
         # more than 64 columns: plain panels (no route flag) in any mode, for any descriptor
         rows, panels, ld, splits, flags = module._panel_shape(plan(4096, 20000, 256, 100, descriptor=kermac.kernel_descriptor_laplace_l1), 0)
         assert (rows, panels, ld, flags) == (20000, 1, 4096, 0) and splits >= 1
