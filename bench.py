@@ -56,6 +56,28 @@ def measured_traffic():
         return None, None
 
 
+# What the vector ALU issues on registers alone (bench_issue_rates.hip): read from the summary of that program's
+# run under profiles/, "key = value" lines at its end; nothing is pasted here.
+ISSUE_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "valu_issue_rates_gfx950.txt")
+
+
+def issue_rates():
+    """{key: float} of the "key = value" lines of the issue-rate summary; {} when the file is missing."""
+    rates = {}
+    try:
+        with open(ISSUE_PROFILE) as handle:
+            for text in handle:
+                key, sep, value = text.partition("=")
+                if sep:
+                    try:
+                        rates[key.strip()] = float(value)
+                    except ValueError:
+                        pass
+    except OSError:
+        pass
+    return rates
+
+
 def log(*args):
     print(*args, file=sys.stderr, flush=True)
 
@@ -387,6 +409,19 @@ def bench_kernel_coef(kermac, device, args, steps=None, warmup=None, with_gaussi
                      wall_ms, kernel_ms, ops, nbytes, "valu_fp32", 157.3, extra, args)
 
 
+def measured_issue_ceiling(p):
+    """What the kernel's own instruction mix reaches on registers alone, for launches as long as the benchmark's
+    (profiles/valu_issue_rates_gfx950.txt): the time the problem would take at that rate, and the clock it ran at."""
+    rates = issue_rates()
+    case = {1.0: "p1_rows", 2.0: "p2_rows"}.get(p, "pow_rows")
+    per_term = 2 if p in (1.0, 2.0) else 5
+    if case + "_lane_ops_per_s" not in rates:
+        return None
+    return {"source": "profiles/" + os.path.basename(ISSUE_PROFILE), "case": case,
+            "lane_ops_per_s": rates[case + "_lane_ops_per_s"], "clock_mhz": rates.get(case + "_clock_mhz"),
+            "floor_ms": round(M * N * K * per_term / rates[case + "_lane_ops_per_s"] * 1e3, 2)}
+
+
 def finish(line):
     """Print the one JSON line; a parity failure is part of it and makes the exit status 1."""
     line["parity_failed"] = PARITY_FAILURES
@@ -397,9 +432,24 @@ def finish(line):
 
 
 def p_entry(k_ms, err, rtol, **more):
+    """A cdist timing on the vector ALU: the counted 3 fp32 operations per (m, n, k) against the fp32 vector peak."""
     return {"ms": round(k_ms, 3), "tflops_3op": round(OPS_PER_CALL / k_ms / 1e9, 2),
             "pct_fp32_valu_peak": round(OPS_PER_CALL / k_ms / 1e9 / PEAK_FP32_VALU_TFLOPS * 100, 2),
             "parity_max_rel_err": err, "rtol": rtol, **more}
+
+
+PEAK_MFMA_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}     # dense matrix peaks of the MI355X
+
+
+def mfma_entry(k_ms, err, rtol, products, operand_type, **more):
+    """A timing whose multiply-adds run on the matrix cores: the executed matrix work (2 M N K per piece product)
+    against the dense peak of the matrix instruction's operand type."""
+    executed = products * 2.0 * M * N * K / k_ms / 1e9
+    peak = PEAK_MFMA_TFLOPS[operand_type]
+    return {"ms": round(k_ms, 3), "parity_max_rel_err": err, "rtol": rtol,
+            "roofline": {"bound": "mfma", "operands": operand_type, "piece_products": products,
+                         "achieved": round(executed, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(executed / peak, 4)},
+            **more}
 
 
 def main():
@@ -469,23 +519,30 @@ def main():
             log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
             check_parity(f"cdist p={label} slab max rel err", e, rtol)
             per_p[label] = p_entry(k_ms, e, rtol)
+        if kermac.get_l2_mode() in ("auto", "gram_bf16"):
+            # this problem takes the route through the workspace: three products of fp16 pieces
+            per_p["2.0"] = mfma_entry(per_p["2.0"]["ms"], per_p["2.0"]["parity_max_rel_err"], 1e-5, 3, "f16")
         per_p["2.0"]["l2_mode"] = kermac.get_l2_mode()
         per_p["2.0"]["note"] = ("default mode 'auto': |a-c|^2 + |b-c|^2 - 2 (a-c).(b-c), c = sample mean, with the cross term on "
                                 "the fp16 matrix instruction (both operands split once into two fp16 pieces per value, scaled per "
                                 "row, in a workspace; 256 x 256 tiles; three piece products), ill-conditioned 128 x 128 parts "
                                 "recomputed by the direct kernel; the vector-ALU kernel is per_p['2.0_direct']")
-        # Fractional p costs five instructions per (m, n, k), two of them transcendentals that issue at a
-        # quarter of the rate.  Rates measured with kermac_amd/_lib/valu_issue_rates (examples/valu_issue_rates.hip):
-        # v_exp_f32 / v_log_f32 19.0e12 lane-operations/s, v_add_f32 65.4e12 -> 2 / 19.0e12 + 3 / 65.4e12 s per term
-        # is the sum of the parts; the kernel's own chain (sub, log2, mul, exp2, add) on registers alone runs at
-        # 27.86e12 lane-operations/s, i.e. 5 / 27.86e12 s per term: mixing the two kinds costs a fifth on top.
-        floor_ms = M * N * K * (2 / 19.0e12 + 3 / 65.4e12) * 1e3
-        chain_ms = M * N * K * 5 / 27.86e12 * 1e3
-        for label in ("1.3", "1.3_skip_epilogue"):
-            per_p[label]["issue_floor_ms"] = round(floor_ms, 1)
-            per_p[label]["frac_of_issue_ceiling"] = round(floor_ms / per_p[label]["ms"], 4)
-            per_p[label]["isolated_chain_ms"] = round(chain_ms, 1)
-            per_p[label]["frac_of_isolated_chain"] = round(chain_ms / per_p[label]["ms"], 4)
+        # Fractional p costs five instructions per (m, n, k), two of them transcendentals that issue at a quarter
+        # of the rate.  issue_floor_ms adds the parts (2 transcendentals + 3 plain instructions per term at the
+        # rates each kind reaches alone); isolated_chain_ms is the kernel's own chain (sub, log2, mul, exp2, add)
+        # on registers alone: mixing the two kinds costs a fifth on top of the sum of the parts.
+        rates = issue_rates()
+        needed = ("v_exp_f32_lane_ops_per_s", "v_log_f32_lane_ops_per_s", "v_add_f32_lane_ops_per_s", "pow_rows_lane_ops_per_s")
+        if all(key in rates for key in needed):
+            floor_ms = M * N * K * (1 / rates["v_exp_f32_lane_ops_per_s"] + 1 / rates["v_log_f32_lane_ops_per_s"]
+                                    + 3 / rates["v_add_f32_lane_ops_per_s"]) * 1e3
+            chain_ms = M * N * K * 5 / rates["pow_rows_lane_ops_per_s"] * 1e3
+            for label in ("1.3", "1.3_skip_epilogue"):
+                per_p[label]["issue_floor_ms"] = round(floor_ms, 1)
+                per_p[label]["frac_of_issue_ceiling"] = round(floor_ms / per_p[label]["ms"], 4)
+                per_p[label]["isolated_chain_ms"] = round(chain_ms, 1)
+                per_p[label]["frac_of_isolated_chain"] = round(chain_ms / per_p[label]["ms"], 4)
+                per_p[label]["issue_rates_source"] = "profiles/" + os.path.basename(ISSUE_PROFILE)
 
         # The two matrix-core paths for p = 2 by name (|a|^2 + |b|^2 - 2 a.b on fp32 MFMA, ill-conditioned tiles
         # recomputed directly); same 1e-5 tolerance.  The default 'auto' picks the second for this problem.
@@ -508,7 +565,7 @@ def main():
                     os.environ["KERMAC_AMD_L2_WORKSPACE"] = saved
             log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
             check_parity(f"cdist p=2.0 ({label}) slab max rel err", e, 1e-5)
-            per_p[label] = p_entry(k_ms, e, 1e-5, mfma_tflops=round(products * 2.0 * M * N * K / k_ms / 1e9, 2), l2_mode=mode)
+            per_p[label] = mfma_entry(k_ms, e, 1e-5, products, {1: "f32", 3: "f16", 6: "bf16"}[products], l2_mode=mode)
 
         # x against x (the kernel matrix of a training set): the library computes the tiles on and
         # below the diagonal only and stores each twice; bit-identical to the full computation.
@@ -519,6 +576,24 @@ def main():
         check_parity("cdist p=1.0 (a against itself) slab max rel err", e, 1e-5)
         per_p["1.0_a_against_itself"] = {"ms": round(k_ms, 3), "parity_max_rel_err": e, "rtol": 1e-5,
                                          "note": "symmetric result: half the tiles computed, each stored twice"}
+        # The opt-in fixed-point route for p = 1 (kermac.l1_mode("fixed")): both operands rounded once to a common
+        # 22-bit grid, one v_sad_u32 per term, tiles whose error bound is not met recomputed by the fp32 kernel.
+        log("timing p = 1.0, l1 mode 'fixed'")
+        with kermac.l1_mode("fixed"):
+            _, k_ms = time_cdist(kermac, a, b, out, 1.0, False, side_steps, 1)
+            e = parity_slab(out, a, b, 1.0, False)
+        log(f"  {k_ms:.2f} ms kernel, slab max rel err {e:.2e}")
+        check_parity("cdist p=1.0 (l1 mode 'fixed') slab max rel err", e, 1e-5)
+        per_p["1.0_fixed_point"] = p_entry(k_ms, e, 1e-5, l1_mode="fixed",
+                                           note="opt-in: sums of |qb - qa| on 32-bit integers (one v_sad_u32 per term where fp32 "
+                                                "issues two instructions), operands rounded once to a common power-of-two grid "
+                                                "in a workspace, error bound K grid steps per element, elements whose bound "
+                                                "exceeds 8e-6 recomputed tile-wise by the fp32 kernel; all launches included")
+        rate = issue_rates().get("v_sad_u32_lane_ops_per_s")
+        if rate:
+            per_p["1.0_fixed_point"]["issue_floor_ms"] = round(M * N * K / rate * 1e3, 2)
+            per_p["1.0_fixed_point"]["frac_of_issue_ceiling"] = round(M * N * K / rate * 1e3 / k_ms, 4)
+
         log("timing p = 2.0, a against itself")
         _, k_ms = time_cdist(kermac, a, a, out, 2.0, False, side_steps, 1)
         e = parity_slab(out, a, a, 2.0, False, slabs=OFF_DIAGONAL_SLABS)
@@ -546,7 +621,7 @@ def main():
         check_parity("sum of products, max abs err / sum_k |a b|", dot_err, 1e-6)
         check_parity("sum of products (direct kernel), max abs err / sum_k |a b|", dot_direct_err, 1e-6)
         per_p["sum_of_products"] = {"ms": round(dot_ms, 3), "parity_max_err_over_sum_of_absolute_terms": dot_err,
-                                    "mfma_tflops": round(3 * 2.0 * M * N * K / dot_ms / 1e9, 2),
+                                    "roofline": mfma_entry(dot_ms, dot_err, 1e-6, 3, "f16")["roofline"],
                                     "direct_kernel_ms": round(dot_direct_ms, 3),
                                     "direct_kernel_parity_max_err_over_sum_of_absolute_terms": dot_direct_err,
                                     "note": "run_kernel with inner operator DOT: two fp16 pieces per value on the 256 x 256 walk; "
@@ -599,6 +674,7 @@ def main():
             "counting": "3 fp32 ops per (m,n,k); the kernel issues 2 VALU instructions per (m,n,k), so its "
                         "instruction-issue ceiling is 1.5 x 78.6 = 117.9 TFLOP/s in this unit at 2.4 GHz",
             "frac_of_issue_ceiling": round(achieved / 117.9, 4),
+            "measured_issue_rate": measured_issue_ceiling(headline_p),
             "clock": {"nominal_mhz_in_peak": 2400,
                       "shader_mhz_under_this_kernel": (traffic_source or {}).get("shader_clock_mhz"),
                       "how": "GRBM_GUI_ACTIVE / kernel duration in the profile named by traffic_source; "

@@ -119,7 +119,25 @@ enum kmc_flags {
      * one-step kernels are faster.  For callers whose alternative is not those kernels: the
      * product of a kernel matrix with coefficients taken panel by panel competes with the fused
      * kernel of kmc_kernel_times_coefficients, which walks the matrix several times more slowly. */
-    KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE = 256
+    KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE = 256,
+    /* kmc_build_kernel, inner_operator DIFF with inner_power ABS (sums of absolute differences: the
+     * L1 norm, Laplace-L1), with gram_workspace: large problems are summed on 32-bit fixed point.
+     * Both operands are rounded once to a common grid (one power-of-two step per batch entry, from
+     * the largest magnitude in both panels; 22 bits for k > 256, 24 for k <= 256, 26 for k <= 64) and
+     * the walk adds |qb - qa| with one integer instruction (v_sad_u32) where fp32 takes two; integer
+     * sums are exact.  An element is off by at most k grid steps; one whose sum is below
+     * k / tolerance steps is not trusted (tolerance = gram_trust when 0 < gram_trust < 1, else 8e-6),
+     * its 128 x 128 tile is stamped and the direct kernel recomputes the stamped tiles right behind,
+     * as for KMC_FLAG_L2_GRAM.  Data with a NaN or an infinity, and data where a sample of 1024
+     * pairs has more than one in 64 below the threshold (outliers that stretch the grid, sets of
+     * near-duplicates), go to the direct kernel whole.  Trusted elements carry a relative error
+     * below the tolerance; on spread-out data far less than the fp32 kernel's own rounding.
+     * kmc_gram_workspace_bytes says which problems take the route (2048 tiles of 128 x 128 over the
+     * batch and k >= 128; KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE: any) and how much memory it wants
+     * (4 bytes per element of the padded operands).  Without a workspace, or for a problem the
+     * query reports 0 for, the direct kernel runs.  Not with k_total.
+     * The reference has no such path (include/build_a_kernel.cuh:339-370 is fp32 only). */
+    KMC_FLAG_L1_FIXED = 512
 };
 
 /*
@@ -177,7 +195,7 @@ typedef struct kmc_build_kernel_params {
      * as it is; kmc_sample_mean writes all of this).  NULL: nothing is subtracted. */
     const float *gram_centre;
     int64_t gram_centre_bs;
-    /* With KMC_FLAG_L2_GRAM_BF16 or KMC_FLAG_DOT_PIECES (ignored otherwise): device memory the call may use, 256-byte
+    /* With KMC_FLAG_L2_GRAM_BF16, KMC_FLAG_DOT_PIECES or KMC_FLAG_L1_FIXED (ignored otherwise): device memory the call may use, 256-byte
      * aligned, of at least the size kmc_gram_workspace_bytes reports for these parameters.  With
      * it, large problems take a faster route in three steps (statistics per row, both operands
      * split once into two fp16 pieces per value in the order the matrix instruction reads them,

@@ -11,7 +11,8 @@ from .module_cache.module_cache import ModuleCache
 from .build_a_kernel import (InnerOperator, KernelDescriptor, KernelType, PowerType, Symmetry,
                              kernel_descriptor_l1_norm, kernel_descriptor_l2_norm, kernel_descriptor_laplace_l1,
                              kernel_descriptor_laplace_l2, kernel_descriptor_mma, kernel_descriptor_p_norm,
-                             pre_compile_descriptors, run_kernel, set_l2_mode, get_l2_mode, l2_mode, DEFAULT_L2_MODE)
+                             pre_compile_descriptors, run_kernel, set_l2_mode, get_l2_mode, l2_mode, DEFAULT_L2_MODE,
+                             set_l1_mode, get_l1_mode, l1_mode, DEFAULT_L1_MODE)
 from .cdist import cdist
 from .cdist_grad import cdist_grad
 
@@ -24,4 +25,5 @@ __all__ = [
     "pre_compile_descriptors", "ModuleCache", "CudaTimer", "PyTorchStreamWrapper", "TensorStats",
     "tensor_stats", "Majorness", "Alignment", "FillMode", "ceil_div", "merge_batch_size",
     "set_l2_mode", "get_l2_mode", "l2_mode", "DEFAULT_L2_MODE",
+    "set_l1_mode", "get_l1_mode", "l1_mode", "DEFAULT_L1_MODE",
 ]

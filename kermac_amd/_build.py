@@ -55,7 +55,7 @@ EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_i
                         "kernels/gram_coefficients_inst.hip", "kernels/gram_bf16_kernel_inst.hip",
                         "kernels/finish_partials.hip", "kernels/cut_static_scratch.hip", "kernels/sample_mean.hip",
                         "kernels/gram_f16_wide_inst.hip", "kernels/norm_gradient_f16_inst.hip",
-                        "kernels/matrix_times_coefficients.hip"]
+                        "kernels/matrix_times_coefficients.hip", "kernels/l1_fixed_inst.hip"]
 
 
 def _hipcc() -> str:
@@ -141,24 +141,17 @@ def build(force: bool = True, verbose: bool = False, workers: int | None = None,
 
 
 def build_c_example(verbose: bool = False) -> Path:
-    """Build the two stand-alone HIP programs of examples/ next to the library:
-    c_abi_cdist (uses nothing but the C ABI; linked against the library with an rpath relative
-    to the binary) and valu_issue_rates (the inner-loop instruction mixes of the kernel headers
-    on registers only: the issue ceilings the benchmark reports against)."""
+    """Build the stand-alone program of examples/ next to the library: c_abi_cdist uses nothing but
+    the C ABI and is linked against the library with an rpath relative to the binary."""
     examples = PACKAGE_DIR.parent / "examples"
     target = LIB_DIR / "c_abi_cdist"
-    commands = [
-        [_hipcc(), f"--offload-arch={ARCH}", "-O2", "-std=c++17", f"-I{PACKAGE_DIR.parent / 'include'}",
-         str(examples / "c_abi_cdist.cpp"), f"-L{LIB_DIR}", "-lkermac_amd", "-Wl,-rpath,$ORIGIN", "-o", str(target)],
-        [_hipcc(), *[flag for flag in HIPCC_FLAGS if flag != "-fPIC"], str(examples / "valu_issue_rates.hip"),
-         "-o", str(LIB_DIR / "valu_issue_rates")],
-    ]
-    for cmd in commands:
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        proc = subprocess.run(cmd, capture_output=True, text=True)
-        if proc.returncode != 0:
-            raise RuntimeError(f"building {cmd[-1]} failed:\n{proc.stdout}\n{proc.stderr}")
+    cmd = [_hipcc(), f"--offload-arch={ARCH}", "-O2", "-std=c++17", f"-I{PACKAGE_DIR.parent / 'include'}",
+           str(examples / "c_abi_cdist.cpp"), f"-L{LIB_DIR}", "-lkermac_amd", "-Wl,-rpath,$ORIGIN", "-o", str(target)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building {cmd[-1]} failed:\n{proc.stdout}\n{proc.stderr}")
     return target
 
 

@@ -267,6 +267,65 @@ def _gram_trust(K: int, setting) -> float:
     return max(0.25, (K ** 0.5) * 2.0 ** -24 / 8e-6)
 
 
+# How DIFF + ABS descriptors (L1 norm, Laplace-L1) are evaluated.
+#   "direct": subtract, add |x| on the vector ALU in fp32 (the reference's arithmetic).  The default.
+#   "fixed":  large stored matrices on 32-bit fixed point: both operands rounded once to a common
+#             power-of-two grid (in a workspace allocated per call, as large as the operands), the
+#             sums of |qb - qa| on one integer instruction per term, exactly; an element whose distance
+#             is so small against the grid step that the rounding of the operands could show
+#             (relative error bound above `tolerance`, 8e-6 unless given) has its 128 x 128 tile
+#             recomputed by the direct kernel.  About 0.85 of the direct kernel's time at
+#             M = N = 30000, K = 1024, and closer to the exact sums on spread-out data.
+_L1_MODES = ("direct", "fixed")
+DEFAULT_L1_MODE = os.environ.get("KERMAC_AMD_L1_MODE", "direct")
+_l1_process = {"mode": DEFAULT_L1_MODE, "tolerance": None}
+if _l1_process["mode"] not in _L1_MODES:
+    raise ValueError(f"KERMAC_AMD_L1_MODE must be one of {_L1_MODES}, got {_l1_process['mode']!r}")
+_l1_thread = threading.local()
+
+
+def _l1_setting(mode, tolerance):
+    if mode not in _L1_MODES:
+        raise ValueError(f"l1 mode must be 'direct' or 'fixed', got {mode!r}")
+    if tolerance is not None and not 0.0 < tolerance < 1.0:
+        raise ValueError("tolerance must lie between 0 and 1")
+    return {"mode": mode, "tolerance": tolerance}
+
+
+def _l1_current():
+    stack = getattr(_l1_thread, "stack", None)
+    return stack[-1] if stack else _l1_process
+
+
+def set_l1_mode(mode: str, tolerance: Optional[float] = None) -> None:
+    """Choose, for the whole process, how sums of absolute differences (``cdist(p=1)``, the L1-norm and
+    Laplace-L1 descriptors) are evaluated: ``"direct"`` (default; fp32 on the vector ALU, the
+    reference's arithmetic) or ``"fixed"`` (large stored matrices on 32-bit fixed point with one
+    integer instruction per term; elements whose relative error bound exceeds ``tolerance``, 8e-6
+    by default, are recomputed by the direct kernel tile by tile).  A thread inside an
+    ``l1_mode(...)`` block keeps the mode of its block."""
+    _l1_process.update(_l1_setting(mode, tolerance))
+
+
+@contextlib.contextmanager
+def l1_mode(mode: str, tolerance: Optional[float] = None):
+    """``with kermac.l1_mode("fixed"): ...`` for the calls the current host thread makes inside the
+    block; arguments as for ``set_l1_mode``; blocks nest."""
+    setting = _l1_setting(mode, tolerance)
+    stack = getattr(_l1_thread, "stack", None)
+    if stack is None:
+        stack = _l1_thread.stack = []
+    stack.append(setting)
+    try:
+        yield
+    finally:
+        stack.pop()
+
+
+def get_l1_mode() -> str:
+    return _l1_current()["mode"]
+
+
 class _LaunchPlan:
     """Everything needed to launch: the C parameter block, the tensor that will
     be returned, and references that keep device memory alive until launch."""
@@ -431,6 +490,16 @@ def _plan_run_kernel(
         # fp16 pieces per value, when the library has a use for the workspace that run_kernel offers it
         l2_auto = l2["mode"] == "auto"
         params.flags |= _backend.FLAG_DOT_PIECES
+    l1 = _l1_current()
+    if (l1["mode"] == "fixed" and d._inner_operator is InnerOperator.DIFF and d._inner_power is PowerType.ABS
+            and stats_c is not None):
+        # sums of absolute differences: large stored matrices on fixed point, when the library has a
+        # use for the workspace that run_kernel offers it
+        params.flags |= _backend.FLAG_L1_FIXED
+        if os.environ.get("KERMAC_AMD_L1_FIXED_ANY_SIZE", "0") not in ("", "0"):
+            params.flags |= _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE      # tests send small shapes down the route
+        if l1["tolerance"] is not None:
+            params.gram_trust = float(l1["tolerance"])
     params.m, params.n, params.k, params.l = M, N, K, L
     params.a, params.a_ld, params.a_bs = a.data_ptr(), stats_a.leading_dimension_stride, stats_a.batch_stride
     params.b, params.b_ld, params.b_bs = b.data_ptr(), stats_b.leading_dimension_stride, stats_b.batch_stride
@@ -546,6 +615,13 @@ def run_kernel(
         if workspace is None:
             params.flags &= ~_backend.FLAG_DOT_PIECES
         plan.keepalive.append(workspace)
+    if params.flags & _backend.FLAG_L1_FIXED:
+        # the fixed-point route exists only through a workspace: without one (a problem too small
+        # for the library to want one, no memory) the call is an ordinary one of the direct kernel
+        workspace = _attach_gram_workspace(params, a.device, switch="KERMAC_AMD_L1_WORKSPACE")
+        if workspace is None:
+            params.flags &= ~_backend.FLAG_L1_FIXED
+        plan.keepalive.append(workspace)
     cut = _cut_over_contraction(params)
     if params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
         plan.keepalive.append(_attach_gram_centre(params, stream, a.device))
@@ -637,12 +713,12 @@ def _workspace_route_applies(params, flags):
         params.flags = kept
 
 
-def _attach_gram_workspace(params, device):
+def _attach_gram_workspace(params, device, switch="KERMAC_AMD_L2_WORKSPACE"):
     """Large squared-difference problems in the split-bf16 mode go through a workspace (include/
     kermac_amd.h, gram_workspace: both operands split once into fp16 pieces, then 256 x 256 tiles);
     the library says how much it wants for this call, 0 when it would not use one.
     KERMAC_AMD_L2_WORKSPACE=0 keeps every call on the one-step kernel."""
-    if os.environ.get("KERMAC_AMD_L2_WORKSPACE", "1") in ("", "0"):
+    if os.environ.get(switch, "1") in ("", "0"):
         return None
     needed = _backend.gram_workspace_bytes(params)
     if needed == 0:
@@ -709,7 +785,8 @@ def _choose_cut(tiles, K, mirrored, plane_bytes):
 
 def _cut_over_contraction(params):
     """(ranges of k, k per range), or None when the launch goes out as it is."""
-    if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16 | _backend.FLAG_DOT_PIECES):
+    if params.l != 1 or params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16 | _backend.FLAG_DOT_PIECES
+                                        | _backend.FLAG_L1_FIXED):
         return None
     tiles = -(-params.m // 128) * -(-params.n // 128)
     if tiles == 0 or params.k < _CUT_MIN_K or not launch_cuts_enabled():

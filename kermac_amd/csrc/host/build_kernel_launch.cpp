@@ -144,6 +144,8 @@ hipError_t launch_gram_l2(int load_a, int load_b, const kmc::BuildKernelArgs &ar
 hipError_t launch_gram_bf16_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
 int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
 hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
+int64_t l1_fixed_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
+hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
 hipError_t launch_finish_partials(const kmc::BuildKernelArgs &kernel, const float *partials, int64_t partial_ld,
                                   int64_t partial_bs, int64_t partial_slice, int slices, int vec, hipStream_t stream);
 }
@@ -186,6 +188,7 @@ int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *byt
     int status = prepare(&asked, true, &args, &load_a, &load_b);
     if (status != KMC_OK) return status;
     *bytes = gram_f16_wide_bytes(&asked, args);
+    if (*bytes == 0) *bytes = l1_fixed_bytes(&asked, args);
     return KMC_OK;
 }
 
@@ -238,6 +241,15 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
             if (g != hipSuccess) return fail_hip(g, "gram_l2_kernel launch");
         }
         args.repair_only = 1;
+    }
+    if (params->flags & KMC_FLAG_L1_FIXED) {
+        if (params->inner_operator != KMC_OP_DIFF || params->inner_power != KMC_POW_ABS)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L1_FIXED needs inner_operator DIFF and inner_power ABS");
+        // Fixed-point pass over every tile, then the direct kernel over the tiles it marked.
+        bool fixed = false;
+        hipError_t g = launch_l1_fixed(params, args, static_cast<hipStream_t>(stream), &fixed);
+        if (g != hipSuccess) return fail_hip(g, "l1_fixed launches");
+        if (fixed) args.repair_only = 1;
     }
     hipError_t e = launch(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail_hip(e, "build_kernel launch");

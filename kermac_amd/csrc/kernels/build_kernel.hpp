@@ -488,57 +488,16 @@ __device__ __forceinline__ bool tile_of_workgroup(const BuildKernelArgs &args, i
 // marked tiles.
 constexpr unsigned BK_REPAIR_MARKER = 0x7fc5a5a5u;
 
-template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs args)
+// Stores of one finished 128 x 128 register tile (layout of finish_tile): 16 pieces of 4 consecutive m
+// per lane, and for a symmetric result the same values again at C(n, m).  `lds_a` / `lds_b` are the
+// staging arrays of the K walk, idle by now (the walk ends with a barrier).  `distrusted` (uniform over
+// the workgroup; kernels whose tiles the direct kernel may have to recompute) stamps BK_REPAIR_MARKER
+// into the tile's first element and leaves the mirrored copy to the repair launch.
+__device__ __forceinline__ void store_tile(
+    const float (&acc)[8][8], const BuildKernelArgs &args, int batch, int tile_m, int tile_n, int m0, int n0,
+    int m_valid, int n_valid, int tx, int ty, int tid, float *lds_a, float *lds_b, bool distrusted)
 {
-    // Two slices per operand plus one pad row (see the fragment prefetch).
-    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE + BK_LDS_PITCH];
-    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE + BK_LDS_PITCH];
-
-    const int tid = threadIdx.x;
-    const int batch = blockIdx.y;
-    int tile_m, tile_n;
-    if (!tile_of_workgroup(args, tile_m, tile_n)) return;
-    const int m0 = tile_m * BK_TILE_M;
-    const int n0 = tile_n * BK_TILE_N;
-    const int m_valid = args.m - m0;   // rows of A that exist from m0 on (may exceed 128)
-    const int n_valid = args.n - n0;
-    const int tx = tid & 15;
-    const int ty = tid >> 4;
-
-    if (args.repair_only) {
-        const float first = args.c[batch * args.c_bs + (i64)n0 * args.c_ld + m0];
-        if (__float_as_uint(first) != BK_REPAIR_MARKER) return;   // uniform over the workgroup
-    }
-
-    float p_inner = 0.0f;
-    if (INNER_POW == POW_POW) {
-        p_inner = args.p_inner ? args.p_inner[batch * args.p_inner_bs] : args.p_inner_value;
-    }
-
-    TileLoader<LOAD_A> load_a;
-    TileLoader<LOAD_B> load_b;
-    load_a.init(args.a + batch * args.a_bs, args.a_ld, m0, tid);
-    load_b.init(args.b + batch * args.b_bs, args.b_ld, n0, tid);
-
-    float acc[8][8];
-#pragma unroll
-    for (int j = 0; j < 8; j++)
-#pragma unroll
-        for (int i = 0; i < 8; i++) acc[j][i] = 0.0f;
-
-    const int k_here = args.k_total > 0 ? min(args.k, args.k_total - batch * args.k) : args.k;
-    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && k_here % BK_TILE_K == 0) {
-        accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, true>(
-            acc, load_a, load_b, lds_a, lds_b, k_here, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
-    } else {
-        accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, false>(
-            acc, load_a, load_b, lds_a, lds_b, k_here, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
-    }
-
-    finish_tile(acc, args, batch, m0, n0, tx, ty);
-
-    // Store: each lane writes 16 pieces of 4 consecutive m.
+    // Each lane writes 16 pieces of 4 consecutive m.
     float *c_tile = args.c + batch * args.c_bs;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
@@ -548,19 +507,21 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
         for (int h = 0; h < 2; h++) {
             const int m_local = tx * 4 + h * 64;
             float *dst = c_tile + (i64)(n0 + n_local) * args.c_ld + m0 + m_local;
+            float first = acc[j][4 * h];
+            if (distrusted && j == 0 && h == 0 && tid == 0) first = __uint_as_float(BK_REPAIR_MARKER);
             if (args.c_vec && m_local + 3 < m_valid) {
-                *reinterpret_cast<float4 *>(dst) =
-                    make_float4(acc[j][4 * h], acc[j][4 * h + 1], acc[j][4 * h + 2], acc[j][4 * h + 3]);
+                *reinterpret_cast<float4 *>(dst) = make_float4(first, acc[j][4 * h + 1], acc[j][4 * h + 2], acc[j][4 * h + 3]);
             } else {
+                if (m_local < m_valid) dst[0] = first;
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 1; i < 4; i++)
                     if (m_local + i < m_valid) dst[i] = acc[j][4 * h + i];
             }
         }
     }
 
     // Symmetric result: the same values also belong at C(n, m).
-    if (args.symmetric && tile_m != tile_n) {
+    if (args.symmetric && tile_m != tile_n && !distrusted) {
         if (args.c_vec && m_valid >= BK_TILE_M && n_valid >= BK_TILE_N) {
             // Through LDS (idle after the K walk, which ends with a barrier), a quarter of 32 rows m
             // at a time and the two staging arrays in turn, so that every store instruction of a
@@ -616,6 +577,59 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
             }
         }
     }
+}
+
+template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
+__global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs args)
+{
+    // Two slices per operand plus one pad row (see the fragment prefetch).
+    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+
+    const int tid = threadIdx.x;
+    const int batch = blockIdx.y;
+    int tile_m, tile_n;
+    if (!tile_of_workgroup(args, tile_m, tile_n)) return;
+    const int m0 = tile_m * BK_TILE_M;
+    const int n0 = tile_n * BK_TILE_N;
+    const int m_valid = args.m - m0;   // rows of A that exist from m0 on (may exceed 128)
+    const int n_valid = args.n - n0;
+    const int tx = tid & 15;
+    const int ty = tid >> 4;
+
+    if (args.repair_only) {
+        const float first = args.c[batch * args.c_bs + (i64)n0 * args.c_ld + m0];
+        if (__float_as_uint(first) != BK_REPAIR_MARKER) return;   // uniform over the workgroup
+    }
+
+    float p_inner = 0.0f;
+    if (INNER_POW == POW_POW) {
+        p_inner = args.p_inner ? args.p_inner[batch * args.p_inner_bs] : args.p_inner_value;
+    }
+
+    TileLoader<LOAD_A> load_a;
+    TileLoader<LOAD_B> load_b;
+    load_a.init(args.a + batch * args.a_bs, args.a_ld, m0, tid);
+    load_b.init(args.b + batch * args.b_bs, args.b_ld, n0, tid);
+
+    float acc[8][8];
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[j][i] = 0.0f;
+
+    const int k_here = args.k_total > 0 ? min(args.k, args.k_total - batch * args.k) : args.k;
+    if (m_valid >= BK_TILE_M && n_valid >= BK_TILE_N && k_here % BK_TILE_K == 0) {
+        accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, true>(
+            acc, load_a, load_b, lds_a, lds_b, k_here, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
+    } else {
+        accumulate_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B, false>(
+            acc, load_a, load_b, lds_a, lds_b, k_here, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
+    }
+
+    finish_tile(acc, args, batch, m0, n0, tx, ty);
+
+    store_tile(acc, args, batch, tile_m, tile_n, m0, n0, m_valid, n_valid, tx, ty, tid, lds_a, lds_b, false);
 }
 
 }  // namespace kmc
