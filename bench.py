@@ -527,6 +527,32 @@ def main():
                                 "the fp16 matrix instruction (both operands split once into two fp16 pieces per value, scaled per "
                                 "row, in a workspace; 256 x 256 tiles; three piece products), ill-conditioned 128 x 128 parts "
                                 "recomputed by the direct kernel; the vector-ALU kernel is per_p['2.0_direct']")
+        # The default mode on data that defeats the matrix-core route: 64 tight clusters far apart (centres N(0, 10^2),
+        # noise 1e-3, seed 11), so one pair in 64 is a pair of near-duplicates and every 128 x 128 part holds some.  The
+        # route samples pairs before its product kernel and, finding them, leaves everything to the direct kernel.
+        log("timing p = 2.0 on clustered data, default mode and direct")
+        gen = torch.Generator(device=device).manual_seed(11)
+        centres_a = 10.0 * torch.randn(K, 64, device=device, generator=gen)
+        centres_b = 10.0 * torch.randn(K, 64, device=device, generator=gen)
+        ca_store = centres_a[:, torch.randint(0, 64, (M,), device=device, generator=gen)] + 1e-3 * torch.randn(K, M, device=device, generator=gen)
+        cb_store = centres_a[:, torch.randint(0, 64, (N,), device=device, generator=gen)] + 1e-3 * torch.randn(K, N, device=device, generator=gen)
+        del centres_b
+        ca, cb = ca_store.t(), cb_store.t()
+        _, clustered_ms = time_cdist(kermac, ca, cb, out, 2.0, False, side_steps, 1)
+        clustered_err = parity_slab(out, ca, cb, 2.0, False)
+        with kermac.l2_mode("direct"):
+            _, clustered_direct_ms = time_cdist(kermac, ca, cb, out, 2.0, False, side_steps, 1)
+            clustered_direct_err = parity_slab(out, ca, cb, 2.0, False)
+        log(f"  default {clustered_ms:.2f} ms (slab max rel err {clustered_err:.2e}), direct {clustered_direct_ms:.2f} ms ({clustered_direct_err:.2e})")
+        check_parity("cdist p=2.0 clustered data (default mode) slab max rel err", clustered_err, 1e-5)
+        check_parity("cdist p=2.0 clustered data (direct) slab max rel err", clustered_direct_err, 1e-5)
+        per_p["2.0_clustered"] = {"ms": round(clustered_ms, 3), "direct_ms": round(clustered_direct_ms, 3),
+                                  "default_over_direct": round(clustered_ms / clustered_direct_ms, 4),
+                                  "parity_max_rel_err": clustered_err, "direct_parity_max_rel_err": clustered_direct_err, "rtol": 1e-5,
+                                  "data": "both operands drawn from the same 64 centres N(0, 10^2) per k, plus N(0, 1e-6) noise, seed 11",
+                                  "l2_mode": kermac.get_l2_mode()}
+        del ca_store, cb_store, ca, cb
+
         # Fractional p costs five instructions per (m, n, k), two of them transcendentals that issue at a quarter
         # of the rate.  issue_floor_ms adds the parts (2 transcendentals + 3 plain instructions per term at the
         # rates each kind reaches alone); isolated_chain_ms is the kernel's own chain (sub, log2, mul, exp2, add)

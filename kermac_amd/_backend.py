@@ -43,6 +43,7 @@ FLAG_GRAM_A_KEPT = 64
 FLAG_DOT_PIECES = 128
 FLAG_GRAM_WORKSPACE_ANY_SIZE = 256
 FLAG_L1_FIXED = 512
+FLAG_NO_PROBE = 1024
 
 _float_p = c_void_p  # device pointers are passed as integers
 

@@ -95,7 +95,17 @@ struct GramWideArgs {
     const float *gradient_g; i64 gradient_g_ld, gradient_g_bs;
     const float *gradient_shift; i64 gradient_shift_bs;
     int gradient_n;
+    // GW_EPILOGUE_DISTANCE only, or null: two counters that gram_probe_pairs fills before the product
+    // kernel starts -- pairs sampled, and those of them below the trust threshold.  When 4 or more
+    // sampled pairs in 16384 are below it, (nearly) every 128 x 128 part holds such a pair and would be
+    // recomputed by the repair launch anyway: the product kernel then only stamps its parts.
+    unsigned *probe;
+    int probe_pairs;
 };
+
+constexpr int GW_PROBE_PAIRS = 16384;
+constexpr int GW_PROBE_SLICES = 32;         // of each sampled pair, this many 16-deep slices spread over K
+constexpr unsigned GW_PROBE_BAIL = 4;       // per GW_PROBE_PAIRS
 
 constexpr int GW_MAX_RANGES = 9;      // ranges of K per row: ceil(slices / 8) up to 71 slices, 8 beyond
 
@@ -225,6 +235,57 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsA
     }
 }
 
+template <int UNUSED = 0>
+__global__ void gram_probe_clear(unsigned *probe)
+{
+    if (threadIdx.x < 2) probe[threadIdx.x] = 0u;
+}
+
+// Would the product kernel's results be trusted?  One wave per sampled pair (m, n): squared distance and
+// norms over up to GW_PROBE_SLICES slices spread over K, from the first fp16 piece of every value (2^-11
+// of the row's largest magnitude: ample for a threshold that is a quarter of the norms or more).  The
+// criterion is that of the product kernel on these k alone; near-duplicate points fail it on any
+// subset of k.  blockIdx.y = batch entry; both counters are per launch.
+template <int UNUSED = 0>
+__global__ __launch_bounds__(256) void gram_probe_pairs(const GramWideArgs args)
+{
+    const int batch = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair >= args.probe_pairs) return;
+    unsigned h = (unsigned)pair * 2654435761u + 0x9e3779b9u * (unsigned)(batch + 1);
+    h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 13;
+    const int m = (int)(h % (unsigned)args.kernel.m);
+    h = h * 0x7feb352du + 0x1234567u; h ^= h >> 16;
+    const int n = (int)(h % (unsigned)args.kernel.n);
+    // lane = 2 * (sampled slice) + half
+    const int sampled = min(args.slices, GW_PROBE_SLICES);
+    const int s = lane >> 1, half = lane & 1;
+    float d2 = 0.0f, norms = 0.0f;
+    if (s < sampled) {
+        const int slice = (int)((long long)s * args.slices / sampled);
+        const gram_chunk ca = args.pieces_a[batch * args.pieces_a_bs + ((i64)slice * GW_SEGMENTS + half) * args.rows_pad_a + m];
+        const gram_chunk cb = args.pieces_b[batch * args.pieces_b_bs + ((i64)slice * GW_SEGMENTS + half) * args.rows_pad_b + n];
+        const float ua = args.unscale_a[batch * args.unscale_a_bs + m], ub = args.unscale_b[batch * args.unscale_b_bs + n];
+        const gram_half8 ha = __builtin_bit_cast(gram_half8, ca), hb = __builtin_bit_cast(gram_half8, cb);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float a = (float)ha[e] * ua, b = (float)hb[e] * ub;
+            d2 += (b - a) * (b - a);
+            norms += a * a + b * b;
+        }
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        d2 += __shfl_xor(d2, offset);
+        norms += __shfl_xor(norms, offset);
+    }
+    if (lane == 0) {
+        atomicAdd(&args.probe[0], 1u);
+        if (!(d2 >= args.kernel.gram_trust * norms)) atomicAdd(&args.probe[1], 1u);
+    }
+}
+
 // Workgroup -> tile, as tile_of_workgroup of build_kernel.hpp with bands of GW_BAND_N tiles: a
 // CU holds one workgroup, so the 32 of an XCD cover 4 n tiles x 8 m tiles of a band at a time.
 // SYMMETRIC (a panel against itself): the ids count through the tiles on and below the diagonal,
@@ -299,6 +360,21 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
     const int n0 = tile_n * GW_TILE;
     const int m_valid = args.kernel.m - m0;
     const int n_valid = args.kernel.n - n0;
+
+    if constexpr (EPILOGUE == GW_EPILOGUE_DISTANCE) {
+        // The sample of pairs says that the repair launch would redo (nearly) every part: stamp them all
+        // and leave.  Parts above the diagonal of a symmetric result belong to nobody.
+        if (args.probe && args.probe[1] * (unsigned)GW_PROBE_PAIRS >= GW_PROBE_BAIL * args.probe[0] && args.probe[1] > 0u) {
+            if (tid < 4) {
+                const int part_m = tid & 1, part_n = tid >> 1;
+                const bool above = SYMMETRIC && tile_m == tile_n && part_m < part_n;
+                if (!above && part_m * 128 < m_valid && part_n * 128 < n_valid)
+                    args.kernel.c[batch * args.kernel.c_bs + (i64)(n0 + part_n * 128) * args.kernel.c_ld + m0 + part_m * 128] =
+                        __uint_as_float(BK_REPAIR_MARKER);
+            }
+            return;
+        }
+    }
 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -28,6 +28,7 @@ struct WideLayout {
     int slices, slices_per_range, ranges;
     int tiles_m, tiles_n, tiles_n_padded;
     OperandRegions a, b;
+    int64_t probe;          // byte offset of the two counters of gram_probe_pairs
     int64_t bytes;
 };
 
@@ -112,6 +113,7 @@ bool place_wide(int m, int n, int k, int l, bool a_once, bool b_once, bool symme
     place_operand(layout->a, m, a_once, l, *layout, cursor);
     if (symmetric) layout->b = layout->a;      // one panel, split once
     else place_operand(layout->b, n, b_once, l, *layout, cursor);
+    layout->probe = place(cursor, 256);
     layout->bytes = cursor;
     return true;
 }
@@ -215,6 +217,19 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     wide.slices = layout.slices; wide.ranges = layout.ranges;
     wide.wide_tiles_m = layout.tiles_m; wide.wide_tiles_n = layout.tiles_n; wide.wide_tiles_n_padded = layout.tiles_n_padded;
     const bool products = p->inner_operator == KMC_OP_DOT;
+    // Squared differences of problems whose walk is long against a launch: a sample of pairs first, so
+    // that data the trust rule would reject wholesale (sets of near-duplicates) costs the direct
+    // kernel's time and little more, instead of both.  KMC_FLAG_NO_PROBE leaves it out.
+    if (!products && !(p->flags & KMC_FLAG_NO_PROBE) &&
+        static_cast<int64_t>(layout.tiles_m) * layout.tiles_n * args.l * layout.slices >= 65536) {      // 0.5 ms and more: the sample is 10 us
+        wide.probe = reinterpret_cast<unsigned *>(workspace + layout.probe);
+        wide.probe_pairs = kmc::GW_PROBE_PAIRS / args.l > 1024 ? kmc::GW_PROBE_PAIRS / args.l : 1024;
+        void *clear_args[] = {&wide.probe};
+        status = hipLaunchKernel(reinterpret_cast<const void *>(kmc::gram_probe_clear<0>), dim3(1), dim3(64), clear_args, 0, stream);
+        if (status != hipSuccess) return status;
+        status = launch(kmc::gram_probe_pairs<0>, dim3((wide.probe_pairs + 3) / 4, args.l), dim3(256), stream, wide);
+        if (status != hipSuccess) return status;
+    }
     if (args.symmetric) {
         const dim3 grid(static_cast<unsigned>(layout.tiles_m) * (layout.tiles_m + 1) / 2, args.l, 1);
         status = products ? launch(kmc::gram_f16_wide<true, kmc::GW_EPILOGUE_DOT>, grid, dim3(kmc::GW_THREADS), stream, wide)

@@ -270,3 +270,39 @@ def test_a_batch_of_panels_against_themselves_with_near_twins(device, wide):
     assert torch.equal(d_self, d_self.t())
     assert not torch.isnan(d_self).any()
     assert_close_to_truth(d_self, oracle.cdist(y.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30, what="near duplicates")
+
+
+def clustered(rows, middle, device, seed):
+    """Every row one of the points `middle` plus noise of 1e-3: two rows of one cluster are near-duplicates."""
+    g = torch.Generator().manual_seed(seed)
+    which = torch.randint(0, middle.size(0), (rows,), generator=g)
+    return (middle[which] + 1e-3 * torch.randn(rows, middle.size(1), generator=g)).to(device)
+
+
+def test_sets_of_near_duplicates_go_to_the_direct_kernel_whole(device):
+    """The default mode on data that the trust rule rejects nearly everywhere (64 tight clusters: one pair in 64 is a
+    pair of near-duplicates, so every 128 x 128 part holds some): the sample of pairs sees it, the matrix-core kernel only
+    stamps its parts, and the result is the direct kernel's, bit for bit, at its tolerance -- for the direct kernel's
+    time, not for both."""
+    M, N, K = 8192, 8192, 1024          # 1024 tiles of 256 x 256, 64 slices: the route applies and the sample is taken
+    middle = 10.0 * torch.randn(64, K, generator=torch.Generator().manual_seed(4))
+    a, b = clustered(M, middle, device, 5), clustered(N, middle, device, 6)
+    out = torch.empty(N, M, device=device).t()
+    assert kermac.get_l2_mode() == "auto"
+    with kermac.l2_mode("gram_bf16"):
+        assert workspace_bytes(a.t().contiguous().t(), b.t().contiguous().t()) > 0
+    at, bt = a.t().contiguous().t(), b.t().contiguous().t()       # rows contiguous: the benchmark's storage
+    got = kermac.cdist(at, bt, out=out, p=2.0)
+    with kermac.l2_mode("direct"):
+        plain = kermac.cdist(at, bt, p=2.0)[0]
+    assert torch.equal(got, plain)
+    truth = torch.cdist(a[:512].double(), b[:768].double(), p=2.0)
+    assert_close_to_truth(got[:512, :768], truth, rtol=1e-5, atol=1e-30, what="clustered data")
+    # and spread-out data of the same shape still takes the matrix cores (different bits than the direct kernel)
+    g = torch.Generator().manual_seed(7)
+    a2, b2 = torch.randn(K, M, generator=g).to(device).t(), torch.randn(K, N, generator=g).to(device).t()
+    got2 = kermac.cdist(a2, b2, p=2.0)
+    with kermac.l2_mode("direct"):
+        plain2 = kermac.cdist(a2, b2, p=2.0)
+    assert not torch.equal(got2, plain2)
+    assert_close_to_truth(got2[0][:512, :768], torch.cdist(a2[:512].double(), b2[:768].double(), p=2.0), rtol=1e-5, what="spread-out data")
