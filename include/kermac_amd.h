@@ -101,8 +101,11 @@ enum kmc_flags {
      * workspace still holds the split of `a` that the previous kmc_build_kernel call through this
      * workspace made, for the same a, a_ld, a_bs, a_majorness, m, k, l and gram_centre and with
      * `a` unchanged since; it is not made again.  For callers that build the matrix panel by panel
-     * of `b` (the split of `a` is a quarter of the cost of a panel of 2048 rows of b).  Anything
-     * else in those fields of the previous call gives a wrong result, not an error. */
+     * of `b` (the split of `a` is a quarter of the cost of a panel of 2048 rows of b).  The library
+     * keeps, per workspace address, what the last split of `a` there was made from, and makes the
+     * split again when these fields differ, when the previous call through the workspace took another
+     * route, or when it has not seen the workspace before; that the contents of `a` and of the
+     * workspace itself are unchanged is the caller's word. */
     KMC_FLAG_GRAM_A_KEPT = 64,
     /* kmc_build_kernel, inner_operator DOT with inner_power NOOP (sum_k a b: linear and polynomial
      * kernels), with gram_workspace: large problems are multiplied on the fp16 matrix instruction
@@ -279,7 +282,9 @@ int kmc_sample_mean(const float *x, int32_t majorness, int32_t rows, int32_t k, 
  * ceil(k / depth) * n * (m rounded up to 4) floats do not fit is rejected with
  * KMC_ERR_INVALID_ARGUMENT before anything is launched.  No hipMalloc, hipFree or other
  * allocating call is made.  All calls on one GPU share the array: calls on one stream are
- * ordered, calls that overlap on one GPU (two streams, two host threads) race.
+ * ordered, calls that overlap on one GPU (two streams, two host threads) race.  The first call on
+ * a device looks up the array's address there (once, under a lock): make one eager call per device
+ * before capturing calls into a HIP graph.  The stream must belong to the current device.
  */
 #define KMC_STATIC_SCRATCH_BYTES (64u << 20)
 int kmc_build_kernel_cut_static(const kmc_build_kernel_params *params, int32_t ranges, void *stream);
@@ -366,8 +371,8 @@ typedef struct kmc_kernel_coefficients_params {
     int64_t out_range_stride;
 } kmc_kernel_coefficients_params;
 
-/* Coefficient columns are processed in chunks of 32 per workgroup; o > 32 works
- * (the kernel values are then recomputed per chunk).  Returns
+/* Coefficient columns are processed in chunks of up to 64 per workgroup (one chunk of 32 for o <= 32);
+ * o > 64 works (the kernel values are then recomputed per chunk).  Returns
  * KMC_ERR_UNSUPPORTED_VARIANT when the (inner_operator, inner_power) pair is not
  * among the ahead-of-time compiled ones. */
 int kmc_kernel_times_coefficients(const kmc_kernel_coefficients_params *params, void *stream);

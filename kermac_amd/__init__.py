@@ -14,6 +14,7 @@ from .build_a_kernel import (InnerOperator, KernelDescriptor, KernelType, PowerT
                              pre_compile_descriptors, run_kernel, set_l2_mode, get_l2_mode, l2_mode, DEFAULT_L2_MODE,
                              set_l1_mode, get_l1_mode, l1_mode, DEFAULT_L1_MODE)
 from .cdist import cdist
+from ._scratch import scratch, set_max_scratch_bytes, get_max_scratch_bytes
 from .cdist_grad import cdist_grad
 
 __version__ = "0.1.0"
@@ -26,4 +27,5 @@ __all__ = [
     "tensor_stats", "Majorness", "Alignment", "FillMode", "ceil_div", "merge_batch_size",
     "set_l2_mode", "get_l2_mode", "l2_mode", "DEFAULT_L2_MODE",
     "set_l1_mode", "get_l1_mode", "l1_mode", "DEFAULT_L1_MODE",
+    "scratch", "set_max_scratch_bytes", "get_max_scratch_bytes",
 ]

@@ -25,6 +25,7 @@ import numpy as np
 import torch
 
 from . import _backend
+from . import _scratch
 from .common import (Alignment, Majorness, PyTorchStreamWrapper, TensorStats, ceil_div, launch_cuts_enabled,
                      merge_batch_size, tensor_stats)
 from .module_cache.module_cache import ModuleCache, build_kernel_function_name
@@ -225,17 +226,29 @@ def _l2_current():
 
 
 def set_l2_mode(mode: str, trust: Optional[float] = None, min_k: Optional[int] = None) -> None:
-    """Choose, for the whole process, how squared-difference descriptors are evaluated:
-    ``"direct"`` (default), ``"gram"`` (fp32 matrix cores + automatic repair of
-    ill-conditioned tiles) or ``"gram_bf16"`` (the same on the bf16 matrix instruction,
-    three bf16 pieces per operand).  A thread inside an ``l2_mode(...)`` block keeps the
-    mode of its block.
+    """Choose, for the whole process, how squared-difference descriptors (L2 norm, Laplace-L2, Gaussian) are
+    evaluated.  A thread inside an ``l2_mode(...)`` block keeps the mode of its block.
 
-    ``trust`` (gram modes) is the fraction of ``|a|^2 + |b|^2`` below which a squared
-    distance is recomputed directly.  The default keeps the relative error of the
-    squared distance below about 8e-6: ``max(0.25, sqrt(K) * 2**-24 / 8e-6)``.
-    ``min_k`` (gram modes, default 64): contractions shorter than this use the direct
-    kernel, which is the faster one there.
+    ``"auto"`` (the default; ``KERMAC_AMD_L2_MODE`` sets what the process starts with): by shape -- large
+        problems through a workspace on the fp16 matrix instruction (two fp16 pieces per value, three piece
+        products), mid-size ones on the one-step matrix-core kernels, short contractions (K < ``min_k``) and
+        small ones on the direct kernel; every matrix-core route checks its result against
+        ``trust * (|a|^2 + |b|^2)`` and has the direct kernel recompute what fails.  The arithmetic differs from
+        the reference's fp32 subtract-square-accumulate; the stated tolerance (1e-5 relative to the float64
+        truth) is the same.
+    ``"direct"``: the reference's arithmetic everywhere (fp32 on the vector ALU).
+    ``"gram"``: ``|a|^2 + |b|^2 - 2 a.b`` with the cross term on the fp32 matrix instruction.
+    ``"gram_bf16"``: the cross term from 16-bit pieces (the workspace route where the library takes it, else
+        three bf16 pieces split inside the kernel).
+
+    ``trust`` (matrix-core routes) is the fraction of ``|a|^2 + |b|^2`` below which a squared distance is recomputed
+    directly.  The default, ``max(0.25, sqrt(K) * 2**-24 / 8e-6)``, keeps the relative error of a trusted squared
+    distance below about 8e-6 on the one-step kernels.  The workspace route stops the rule at 0.5 (it would pass 1
+    near K = 18000 and send everything to the direct kernel, whose own fp32 sum over so many terms is no better): for
+    K above about 4500 the error of a trusted squared distance there is bounded by ``sqrt(K) * 2**-24 / 0.5``, 1.1e-5 at
+    K = 8192 (5e-6 on the distance itself), and both kernels' measured errors stay below 1e-5 of the distance up to
+    K = 200000.
+    ``min_k`` (default 64): contractions shorter than this use the direct kernel, which is the faster one there.
     """
     _l2_process.update(_l2_setting(mode, trust, min_k))
 
@@ -535,6 +548,7 @@ def _current_stream_for(device: torch.device) -> int:
     return PyTorchStreamWrapper(torch.cuda.current_stream()).handle
 
 
+@_scratch.operator
 def run_kernel(
     kernel_descriptor: KernelDescriptor,
     a: torch.Tensor,
@@ -571,7 +585,7 @@ def run_kernel(
     are used whenever pointer, leading dimension and batch stride allow them.
 
     ``coefficients`` (an addition to the reference's signature): a ``[L?, N, O]``
-    tensor with ``O <= 64`` contiguous columns.  When given, the kernel matrix is
+    tensor with the ``O`` columns contiguous (any number of them).  When given, the kernel matrix is
     contracted with it on the fly and ``out`` is ``[L?, M, O]``:
     ``out[l, m, o] = sum_n kernelmatrix[l, m, n] * coefficients[l, n, o]``; the
     M x N matrix is never written to memory.
@@ -644,7 +658,9 @@ def _attach_gram_centre(params, stream, device):
     # library leaves it out when the centre is negligible against the spread) and the variances
     width = 2 * (-(-params.k // _backend.CENTRE_PAD) * _backend.CENTRE_PAD) + _backend.CENTRE_PAD
     batches = params.l if params.a_bs != 0 else 1
-    centre = torch.empty((batches, width), dtype=torch.float32, device=device)
+    centre = _scratch.allocate_floats((batches, width), device)
+    if centre is None:
+        return None
     _backend.sample_mean(params.a, params.a_majorness, params.m, params.k, params.a_ld, params.a_bs, batches,
                          centre.data_ptr(), width, stream)
     params.gram_centre, params.gram_centre_bs = centre.data_ptr(), (width if batches > 1 else 0)
@@ -723,10 +739,9 @@ def _attach_gram_workspace(params, device, switch="KERMAC_AMD_L2_WORKSPACE"):
     needed = _backend.gram_workspace_bytes(params)
     if needed == 0:
         return None
-    try:
-        workspace = torch.empty(needed, dtype=torch.uint8, device=device)
-    except torch.cuda.OutOfMemoryError:
-        return None             # no room for it: the one-step kernel needs none
+    workspace = _scratch.allocate(needed, device)
+    if workspace is None:
+        return None             # no room for it, or the caller's limit: the one-step kernel needs none
     params.gram_workspace, params.gram_workspace_bytes = workspace.data_ptr(), needed
     return workspace
 
@@ -805,7 +820,10 @@ def _run_cut_over_contraction(cut, params, launch, stream, device):
     slices, depth = cut
     ld = -(-params.m // 4) * 4
     plane = ld * params.n
-    partial = torch.empty(slices * plane, dtype=torch.float32, device=device)
+    partial = _scratch.allocate_floats((slices * plane,), device)
+    if partial is None:
+        launch(params)          # no memory for the partial sums: the launch goes out as it is
+        return
 
     def k_stride(majorness, leading):
         return leading if majorness == _backend.COL_MAJOR else 1

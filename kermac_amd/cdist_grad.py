@@ -12,6 +12,7 @@ import numpy as np
 import torch
 
 from . import _backend
+from . import _scratch
 from .build_a_kernel import _current_stream_for
 from .common import launch_cuts_enabled, merge_batch_size, tensor_stats
 
@@ -133,6 +134,7 @@ def _plan_cdist_grad(a, b, c, d, out, p, require_device=True) -> _GradPlan:
     return plan
 
 
+@_scratch.operator
 def cdist_grad(
     a: torch.Tensor,           # [K,M]   m contiguous   kernel_matrix
     b: torch.Tensor,           # [N,K]   k contiguous   x
@@ -149,7 +151,7 @@ def cdist_grad(
 
     ``sign`` is ``copysign(1, x)`` (so ``sign(0) = 1``); for ``p = 2`` the weight is
     simply the difference.  Every tensor may carry a leading batch dimension of 1
-    or L.  Returns ``out`` (allocated as zeros ``[L, O, N, M]`` when None).
+    or L.  Returns ``out`` (allocated ``[L, O, N, M]`` when None; every element is written).
 
     Raises:
         TypeError: non-tensor inputs or a dtype other than fp32.
@@ -157,8 +159,7 @@ def cdist_grad(
     """
     plan = _plan_cdist_grad(a, b, c, d, out, p)
     split = _split_over_contraction(plan) if _may_split else None
-    if split is not None:
-        _run_split_over_contraction(split, plan, a, b, c, d, p, debug)
+    if split is not None and _run_split_over_contraction(split, plan, a, b, c, d, p, debug):
         return plan.out
     stream = _current_stream_for(a.device)
     if debug:
@@ -181,10 +182,9 @@ def _attach_workspace(params, device):
     needed = _backend.norm_gradient_workspace_bytes(params)
     if needed == 0:
         return None
-    try:
-        workspace = torch.empty(needed, dtype=torch.uint8, device=device)
-    except torch.cuda.OutOfMemoryError:
-        return None             # no room for it: the fp32 kernels need none
+    workspace = _scratch.allocate(needed, device)
+    if workspace is None:
+        return None             # no room for it, or the caller's limit: the fp32 kernels need none
     params.workspace, params.workspace_bytes = workspace.data_ptr(), needed
     return workspace
 
@@ -228,7 +228,13 @@ def _run_split_over_contraction(split, plan, a, b, c, d, p, debug):
     slices, depth, leftover = split
     a2, b2, c2, d2 = (t[0] if t.dim() == 3 else t for t in (a, b, c, d))
     M, N, O = plan.M, plan.N, plan.O
-    partial = torch.empty((slices + (1 if leftover else 0), O, N, M), dtype=torch.float32, device=a.device)
+    partial = _scratch.allocate_floats((slices + (1 if leftover else 0), O, N, M), a.device)
+    target = plan.out[0] if plan.out.dim() == 4 else plan.out
+    # the order in which torch adds the slices depends on the layout of the result: a strided `out` gets the
+    # bits of a contiguous one, through a buffer of its own
+    staged = None if target.is_contiguous() or partial is None else _scratch.allocate_floats((O, N, M), a.device)
+    if partial is None or (staged is None and not target.is_contiguous()):
+        return False            # no memory for the partial results: the call goes out as it is
     a_slices = a2.as_strided((slices, depth, M), (depth * a2.stride(0), a2.stride(0), a2.stride(1)), a2.storage_offset())
     b_slices = b2.as_strided((slices, N, depth), (depth * b2.stride(1), b2.stride(0), b2.stride(1)), b2.storage_offset())
     c_slices = c2.as_strided((slices, O, depth), (depth * c2.stride(1), c2.stride(0), c2.stride(1)), c2.storage_offset())
@@ -236,10 +242,9 @@ def _run_split_over_contraction(split, plan, a, b, c, d, p, debug):
     if leftover:
         done = slices * depth
         cdist_grad(a2[done:], b2[:, done:], c2[:, done:], d2, out=partial[slices:], p=p, debug=debug, _may_split=False)
-    target = plan.out[0] if plan.out.dim() == 4 else plan.out
-    if target.is_contiguous():
+    if staged is None:
         torch.sum(partial, dim=0, out=target)
     else:
-        # the order in which torch adds the slices depends on the layout of the result: a strided
-        # `out` gets the bits of a contiguous one
-        target.copy_(torch.sum(partial, dim=0))
+        torch.sum(partial, dim=0, out=staged)
+        target.copy_(staged)
+    return True

@@ -10,6 +10,8 @@
 // once per device with that device current, and uses only that pointer afterwards.  All
 // calls on one GPU share the array, so two calls that overlap on one GPU (different
 // streams, different host threads) race on it; calls on one stream are ordered.
+// The first call on a device looks the address up (a lock, hipGetSymbolAddress, possibly the
+// load of the code object): make one eager call per device before capturing calls into a graph.
 #include <hip/hip_runtime.h>
 
 #include <mutex>
@@ -55,14 +57,30 @@ extern "C" int kmc_build_kernel_cut_static(const kmc_build_kernel_params *params
     if (!params) return fail(KMC_ERR_INVALID_ARGUMENT, "null parameter block");
     if (params->l != 1) return fail(KMC_ERR_INVALID_ARGUMENT, "kmc_build_kernel_cut_static takes one problem (l = 1), got l = %d", params->l);
     if (params->k_total != 0) return fail(KMC_ERR_INVALID_ARGUMENT, "k_total must be 0: the ranges are made here");
-    if (params->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16))
-        return fail(KMC_ERR_INVALID_ARGUMENT, "the matrix-core flags cannot be combined with a cut over k");
+    if (params->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16 | KMC_FLAG_DOT_PIECES | KMC_FLAG_L1_FIXED))
+        return fail(KMC_ERR_INVALID_ARGUMENT, "the matrix-core and fixed-point flags cannot be combined with a cut over k");
     if (ranges < 1) return fail(KMC_ERR_INVALID_ARGUMENT, "ranges = %d, need at least 1", ranges);
     if (params->m < 0 || params->n < 0 || params->k < 0)
         return fail(KMC_ERR_INVALID_ARGUMENT, "negative extent (m=%d n=%d k=%d)", params->m, params->n, params->k);
     if (!kmc_build_kernel_has_variant(params->inner_operator, params->inner_power))
         return fail(KMC_ERR_UNSUPPORTED_VARIANT, "inner_operator=%d inner_power=%d is not compiled ahead of time",
                     params->inner_operator, params->inner_power);
+
+    // What the finishing call would reject is rejected here, before the ranges are launched.
+    if (params->m > 0 && params->n > 0 && !params->c) return fail(KMC_ERR_INVALID_ARGUMENT, "c: null pointer");
+    if (params->n > 1 && params->c_ld < params->m)
+        return fail(KMC_ERR_INVALID_ARGUMENT, "c: leading dimension %lld is smaller than m=%d",
+                    static_cast<long long>(params->c_ld), params->m);
+    if (params->c_ld < 0 || params->c_bs < 0) return fail(KMC_ERR_INVALID_ARGUMENT, "c: negative stride");
+    // The array belongs to the current device, and so must the stream.
+    if (stream) {
+        int current = 0, of_stream = 0;
+        hipError_t e = hipGetDevice(&current);
+        if (e == hipSuccess) e = hipStreamGetDevice(static_cast<hipStream_t>(stream), &of_stream);
+        if (e != hipSuccess) return kmc_host::fail_hip(e, "hipStreamGetDevice");
+        if (current != of_stream)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "the stream belongs to device %d, the current device is %d", of_stream, current);
+    }
 
     // Ranges of whole 16-term slices; the last one takes what is left of k.
     const int64_t k = params->k;

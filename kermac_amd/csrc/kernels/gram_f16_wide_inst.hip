@@ -5,6 +5,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
 
 #include "../host/host_common.hpp"
 #include "launch.hpp"
@@ -157,7 +160,50 @@ kmc::GramRowsArgs rows_args(const float *x, int64_t ld, int64_t bs, int rows, in
     return rows_of;
 }
 
+// What the split of `a` in a workspace was made from, kept on the host per workspace address: a call with
+// KMC_FLAG_GRAM_A_KEPT skips the split only when this record says that the previous split through this
+// workspace was of the same operand, shape, centre and layout; anything else (another operand, a call
+// that did not take this route in between and left no record, a workspace seen for the first time)
+// makes the split again.  What the host cannot see is whether the memory itself was overwritten since.
+struct SplitRecord {
+    const float *a; int64_t ld, bs; int majorness, m, k, l, slices, rows_pad;
+    const float *centre; int64_t centre_bs;
+};
+
+std::mutex split_records_mutex;
+std::unordered_map<const void *, SplitRecord> split_records;
+
+SplitRecord record_of(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, const WideLayout &layout)
+{
+    SplitRecord record;
+    std::memset(&record, 0, sizeof record);          // padding too: the records are compared as bytes
+    record.a = p->a; record.ld = p->a_ld; record.bs = p->a_bs; record.majorness = p->a_majorness;
+    record.m = p->m; record.k = p->k; record.l = layout.a.batches; record.slices = layout.slices; record.rows_pad = layout.a.rows_pad;
+    record.centre = args.centre; record.centre_bs = args.centre_bs;
+    return record;
+}
+
+// true: the split of `a` in this workspace is the one this call needs; either way the record is this call's afterwards
+bool split_of_a_is_kept(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, const WideLayout &layout)
+{
+    const SplitRecord wanted = record_of(p, args, layout);
+    std::lock_guard<std::mutex> lock(split_records_mutex);
+    auto found = split_records.find(p->gram_workspace);
+    const bool kept = (p->flags & KMC_FLAG_GRAM_A_KEPT) && found != split_records.end() &&
+                      std::memcmp(&found->second, &wanted, sizeof wanted) == 0;
+    if (split_records.size() > 4096) split_records.clear();      // addresses of freed workspaces pile up otherwise
+    split_records[p->gram_workspace] = wanted;
+    return kept;
+}
+
 }  // namespace
+
+// A route other than this one is about to write into `workspace`: whatever split it held is gone.
+void forget_split_in(const void *workspace)
+{
+    std::lock_guard<std::mutex> lock(split_records_mutex);
+    split_records.erase(workspace);
+}
 
 // Statistics and split of one operand (also used by the gradient's fp16 route).
 hipError_t launch_gram_rows(const kmc::GramRowsArgs &rows_of, int batches, hipStream_t stream)
@@ -189,7 +235,7 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     const kmc::GramRowsArgs rows_a = rows_args(args.a, args.a_ld, args.a_bs, args.m, p->a_majorness, scalar_only, args, layout, layout.a, workspace);
     const kmc::GramRowsArgs rows_b = rows_args(args.b, args.b_ld, args.b_bs, args.n, p->b_majorness, scalar_only, args, layout, layout.b, workspace);
     // the region of a lies first in the workspace and its size does not depend on b
-    hipError_t status = (p->flags & KMC_FLAG_GRAM_A_KEPT) ? hipSuccess : launch_gram_rows(rows_a, layout.a.batches, stream);
+    hipError_t status = split_of_a_is_kept(p, args, layout) ? hipSuccess : launch_gram_rows(rows_a, layout.a.batches, stream);
     if (status != hipSuccess) return status;
     if (!args.symmetric) {
         status = launch_gram_rows(rows_b, layout.b.batches, stream);

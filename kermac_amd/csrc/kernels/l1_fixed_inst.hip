@@ -87,6 +87,8 @@ int64_t l1_fixed_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelA
     return fixed_layout(p, args, &layout) ? layout.bytes : 0;
 }
 
+void forget_split_in(const void *workspace);      // gram_f16_wide_inst.hip
+
 // *taken = the walk was launched: the caller follows it with the direct kernel in repair mode.
 hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken)
 {
@@ -96,6 +98,7 @@ hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKer
     if (!fixed_layout(p, args, &layout) || p->gram_workspace_bytes < layout.bytes) return hipSuccess;
     if (args.l > 65535 || layout.k_padded / 64 + 1 > 65535) return hipSuccess;
     char *workspace = static_cast<char *>(p->gram_workspace);
+    forget_split_in(workspace);
 
     kmc::L1FixedArgs fixed;
     fixed.kernel = args;

@@ -91,9 +91,10 @@ bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)
     layout->b_padded_bs = static_cast<int64_t>(layout->n_pad) * layout->k_pad;
     layout->b_padded = place(cursor, layout->b_batches * layout->b_padded_bs * 4);
     layout->bytes = cursor;
-    // blockIdx.z = batch entry x chunk of outputs, blockIdx.y = tile of at least 16 n
+    // blockIdx.z = batch entry x chunk of outputs; blockIdx.y = one padded row n for gradient_pad_b (the
+    // largest grid.y of the route; the contraction's tiles of 8, 16 or 32 n need fewer)
     const int64_t grid_z = static_cast<int64_t>(p->l) * (p->o / 64 + 1);
-    if (grid_z > 65535 || layout->n_pad / 16 > 65535) return false;
+    if (grid_z > 65535 || layout->n_pad > 65535) return false;
     return true;
 }
 

@@ -16,6 +16,7 @@ from typing import Optional
 import torch
 
 from . import _backend
+from . import _scratch
 from .common import launch_cuts_enabled, merge_batch_size
 from .module_cache.module_cache import ModuleCache, build_kernel_function_name, kernel_coefficients_function_name
 
@@ -96,6 +97,7 @@ def _plan_run_kernel_coefficients(
     return plan
 
 
+@_scratch.operator
 def run_kernel_coefficients(
     kernel_descriptor, a, b, coefficients, out: Optional[torch.Tensor] = None, p=None, inner_p=None, outer_p=None,
     bandwidth=None, epsilon=None, regularization=None, regularization_offset_x: int = 0,
@@ -140,8 +142,9 @@ def run_kernel_coefficients(
     partial = None
     if ranges > 1:
         # every range of centres writes its own partial product; they are added below in range order
-        partial = torch.empty((ranges, plan.L, plan.M, plan.O), dtype=torch.float32, device=a.device)
-        params.out, params.out_ld, params.out_bs = partial.data_ptr(), plan.O, plan.M * plan.O
+        partial = _partial_products(ranges, plan, a.device)       # refused: the centres stay one range
+    if partial is not None:
+        params.out, params.out_ld, params.out_bs = partial[0].data_ptr(), plan.O, plan.M * plan.O
         params.n_ranges, params.out_range_stride = ranges, plan.L * plan.M * plan.O
     if aot:
         if debug:
@@ -158,6 +161,21 @@ def run_kernel_coefficients(
     if partial is not None:
         _sum_partials(partial, plan.out)
     return plan.out
+
+
+def _partial_products(parts, plan, device):
+    """(buffer [parts, L, M, O], staging buffer or None) for partial products that are added into `plan.out`; None
+    when the memory for them is refused (the caller then does without partial products)."""
+    partial = _scratch.allocate_floats((parts, plan.L, plan.M, plan.O), device)
+    if partial is None:
+        return None
+    target = plan.out if plan.out.dim() == 3 else plan.out.unsqueeze(0)
+    if target.is_contiguous():
+        return partial, None
+    # the order in which torch adds the ranges depends on the layout of the result: a strided `out` gets the
+    # bits of a contiguous one, through a buffer of its own
+    staged = _scratch.allocate_floats((plan.L, plan.M, plan.O), device)
+    return None if staged is None else (partial, staged)
 
 
 # Squared differences and sums of products on the matrix cores: the route of kmc_build_kernel through a workspace
@@ -345,12 +363,15 @@ def _run_in_panels(plan, shape, stream, device, debug):
     block = _backend.BuildKernelParams.from_buffer_copy(params.kernel)
     block.flags |= route
     block.n, block.c_ld, block.c_bs = rows, ld, rows * ld
-    try:
-        panel = torch.empty(L * rows * ld, dtype=torch.float32, device=device)
-        product = _contraction_by_pieces(plan, rows, ld, panel, device)
-        partial = torch.empty((parts, L, M, O), dtype=torch.float32, device=device) if parts > 1 and product is None else None
-    except torch.cuda.OutOfMemoryError:
+    panel = _scratch.allocate_floats((L * rows * ld,), device)
+    if panel is None:
         return False
+    product = _contraction_by_pieces(plan, rows, ld, panel, device)
+    partial = None
+    if parts > 1 and product is None:
+        partial = _partial_products(parts, plan, device)
+        if partial is None:
+            return False
     block.c = panel.data_ptr()
     workspace = _attach_gram_workspace(block, device) if route else None
     if route and workspace is None:
@@ -406,7 +427,7 @@ def _run_in_panels(plan, shape, stream, device, debug):
         contraction.n, contraction.matrix_bs = count, count * ld
         contraction.coef = params.coef + 4 * n0 * params.coef_ld
         if partial is not None:
-            contraction.out = partial.data_ptr() + 4 * index * splits * L * M * O
+            contraction.out = partial[0].data_ptr() + 4 * index * splits * L * M * O
         else:
             contraction.accumulate = 1 if index else 0
         _backend.matrix_times_coefficients(contraction, stream)
@@ -462,21 +483,20 @@ def _contraction_by_pieces(plan, rows, ld, panel, device):
     workspace = _attach_gram_workspace(block, device)
     if workspace is None:
         return None
-    try:
-        sums = torch.empty((L, M, O), dtype=torch.float32, device=device) if N > rows else None
-    except torch.cuda.OutOfMemoryError:
+    sums = _scratch.allocate_floats((L, M, O), device) if N > rows else None
+    if N > rows and sums is None:
         return None
     return block, sums, workspace
 
 
-def _sum_partials(partial, out):
+def _sum_partials(buffers, out):
+    partial, staged = buffers
     target = out if out.dim() == 3 else out.unsqueeze(0)
-    if target.is_contiguous():
+    if staged is None:
         torch.sum(partial, dim=0, out=target)
     else:
-        # the order in which torch adds the ranges depends on the layout of the result: a strided
-        # `out` gets the bits of a contiguous one
-        target.copy_(torch.sum(partial, dim=0))
+        torch.sum(partial, dim=0, out=staged)
+        target.copy_(staged)
 
 
 # A workgroup of the fused kernel owns 128 rows of ``a`` (one batch entry, one chunk of up to 64

@@ -330,3 +330,28 @@ def test_cdist_full_size_properties(device, p):
     self_out = kermac.cdist(a_store.t()[:5000], a_store.t()[:5000], p=p)[0]
     assert torch.all(torch.diagonal(self_out) == 0)
     assert torch.equal(self_out, self_out.t())
+
+
+def test_cdist_full_size_direct_kernel_for_squared_differences(device):
+    """M = N = 30000, K = 1024, p = 2 on the kernel with the reference's arithmetic (subtract, square, accumulate:
+    include/build_a_kernel.cuh:339-370), which the default mode no longer runs at this size: float64 slabs at 1e-5, also
+    without the square root."""
+    M = N = 30000
+    K = 1024
+    torch.manual_seed(1)
+    a_store = torch.randn(K, M, device=device)
+    b_store = torch.randn(K, N, device=device)
+    out_store = torch.empty(N, M, device=device)
+    slabs = ((slice(0, 300), slice(0, 2000)), (slice(29900, 30000), slice(29800, 30000)), (slice(14000, 14200), slice(7000, 7600)))
+    with kermac.l2_mode("direct"):
+        out = kermac.cdist(a_store.t(), b_store.t(), out=out_store.t(), p=2.0)
+        for ms, ns in slabs:
+            truth = torch.cdist(a_store.t()[ms].double(), b_store.t()[ns].double(), p=2.0)
+            assert_close_to_truth(out[ms, ns], truth, rtol=1e-5, what="direct kernel, slab p=2")
+        default = torch.empty(2000, 300, device=device)
+    kermac.cdist(a_store.t()[:300], b_store.t()[:2000], out=default.t(), p=2.0)
+    with kermac.l2_mode("direct"):
+        raw = kermac.cdist(a_store.t(), b_store.t(), out=out_store.t(), p=2.0, skip_epilogue=True)
+        for ms, ns in slabs:
+            truth = torch.cdist(a_store.t()[ms].double(), b_store.t()[ns].double(), p=2.0) ** 2
+            assert_close_to_truth(raw[ms, ns], truth, rtol=1e-5, what="direct kernel, slab p=2, skip_epilogue")

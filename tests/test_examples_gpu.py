@@ -61,3 +61,15 @@ def test_build_a_kernel_and_broadcast_examples(device, tmp_path, monkeypatch):
     assert len(errors) == 9 and max(errors) < 1e-4, errors
     text = run_example("build_a_kernel.py", "-m", "130", "-n", "70", "-k", "8", "-s", "-a")
     assert "difference to torch" not in text
+
+
+def test_broadcast_kernel_example(device):
+    """The reference's examples/broadcast_kernel.py: per-batch bandwidths with a regularised diagonal moved by the offsets
+    3 and 1 (its result for out=None has 1 + regularization at [n + 2, n] and nowhere else), then per-batch p and
+    regularization."""
+    text = run_example("broadcast_kernel.py", "-n", "700", "-k", "6")
+    assert "(2, 700, 700)" in text and "(4, 700, 700)" in text
+    found = re.search(r"elements \[n \+ 2, n\] that hold 1 \+ regularization = 11: (\d+) of (\d+); elsewhere: (\d+)", text)
+    assert found, text
+    assert found.group(1) == found.group(2) == str(2 * 698) and found.group(3) == "0"
+    assert numbers_after(text, "largest deviation of the diagonals from 1 + regularization:")[0] < 1e-6

@@ -436,7 +436,7 @@ def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
         for field, _ in binding._fields_:
             lines.append(f'  printf("{c_name} {field} %zu\\n", offsetof(struct {c_name}, {field}));')
     for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16", "GRAM_A_KEPT",
-                 "DOT_PIECES", "GRAM_WORKSPACE_ANY_SIZE"):
+                 "DOT_PIECES", "GRAM_WORKSPACE_ANY_SIZE", "L1_FIXED", "NO_PROBE"):
         lines.append(f'  printf("flag {flag} %d\\n", (int)KMC_FLAG_{flag});')
     lines += ['  printf("err WRONG_DEVICE %d\\n", (int)KMC_ERR_WRONG_DEVICE);', "  return 0;", "}"]
     source = tmp_path / "probe.c"
@@ -453,7 +453,7 @@ def test_header_is_plain_c_and_agrees_with_the_binding(tmp_path):
         for field, _ in binding._fields_:
             assert reported[(c_name, field)] == getattr(binding, field).offset, f"{c_name}.{field}"
     for flag in ("FORCE_SCALAR_ACCESS", "NEGATE_DIFF", "L2_GRAM", "GENERIC_POWER", "NO_SYMMETRY", "L2_GRAM_BF16", "GRAM_A_KEPT",
-                 "DOT_PIECES", "GRAM_WORKSPACE_ANY_SIZE"):
+                 "DOT_PIECES", "GRAM_WORKSPACE_ANY_SIZE", "L1_FIXED", "NO_PROBE"):
         assert reported[("flag", flag)] == getattr(_backend, f"FLAG_{flag}")
     assert reported[("err", "WRONG_DEVICE")] == _backend.ERR_WRONG_DEVICE
 
@@ -582,6 +582,28 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert gradient(256, 64, 64, 512) == 0                                           # 8.4e6 terms
     assert gradient(8192, 16, 16, 8192) == 0                                         # half of every tile of 32 columns unused
     assert gradient(2048, 128, 4, 2048) == 0 and gradient(2048, 128, 16, 2048) > 0   # 5.4e8 terms: enough for 16 outputs, not for 4
+    # a row n is a workgroup row of the route's padding kernel: beyond 65535 of them the fp32 kernels run
+    assert gradient(1000, 65000, 16, 100) > 0 and gradient(1000, 70000, 16, 100) == 0
+
+    def absolute_differences(m, n, k, l=1, flags=_backend.FLAG_L1_FIXED, same=False):
+        params = _backend.BuildKernelParams()
+        params.inner_operator, params.inner_power, params.outer_power = 0, 1, 0      # DIFF, ABS, NOOP
+        params.m, params.n, params.k, params.l = m, n, k, l
+        params.a, params.a_ld, params.a_bs = fake, m, m * k
+        params.b, params.b_ld, params.b_bs = (fake if same else fake + 4 * m * k * l), n, n * k
+        params.c_ld, params.c_bs = m, m * n
+        params.flags = flags
+        return _backend.gram_workspace_bytes(params)
+
+    # the fixed-point route of sums of absolute differences: 2048 tiles of 128 x 128 over the batch, k >= 128
+    padded = (6016 + 6016) * 512 * 4
+    assert padded <= absolute_differences(6000, 6000, 512) <= padded + 1024         # 47 x 47 tiles, 4 bytes per padded element
+    assert absolute_differences(6000, 6000, 512, flags=0) == 0
+    assert absolute_differences(5000, 5000, 512) == 0 and absolute_differences(5000, 5000, 512, l=2) > 0
+    assert absolute_differences(6000, 6000, 100) == 0
+    assert 0 < absolute_differences(9000, 9000, 512, same=True) < 0.6 * absolute_differences(9000, 9000, 512)
+    assert absolute_differences(300, 200, 5, flags=_backend.FLAG_L1_FIXED | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE) > 0
+    assert squared_differences(6000, 6000, 512, flags=_backend.FLAG_L1_FIXED) == 0  # squared differences: not this route
     monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
     assert gradient(3, 2, 1, 5) > 0
 
@@ -799,3 +821,43 @@ def test_cut_decision_for_a_tall_narrow_result():
     assert plan.swapped and (plan.params.m, plan.params.n) == (100, 100000)
     cut = module._cut_over_contraction(plan.params)
     assert cut is not None and cut[0] * cut[1] >= 4096 and cut[1] % 16 == 0
+
+
+def test_scratch_memory_is_handed_out_within_the_limit_or_from_the_callers_buffer():
+    """kermac_amd/_scratch.py on host memory: the limit counts per outermost operator call, a supplied buffer is
+    handed out from its start at 256-byte aligned addresses by every call, what does not fit is refused."""
+    import torch
+    from kermac_amd import _scratch
+    cpu = torch.device("cpu")
+    assert _scratch.get_max_scratch_bytes() is None
+    with _scratch.operator_call():
+        assert _scratch.allocate(1000, cpu).numel() == 1000
+    _scratch.set_max_scratch_bytes(4096)
+    try:
+        with _scratch.operator_call():
+            assert _scratch.allocate(3000, cpu) is not None
+            with _scratch.operator_call():                       # an operator called by an operator shares the budget
+                assert _scratch.allocate(2000, cpu) is None
+                assert _scratch.allocate_floats((16, 16), cpu).shape == (16, 16)
+            assert _scratch.allocate(100, cpu) is None
+        with _scratch.operator_call():                           # the next call starts afresh
+            assert _scratch.allocate(4096, cpu) is not None
+        _scratch.set_max_scratch_bytes(0)
+        with _scratch.operator_call():
+            assert _scratch.allocate(1, cpu) is None
+    finally:
+        _scratch.set_max_scratch_bytes(None)
+    buffer = torch.empty(5000, dtype=torch.uint8)
+    with _scratch.scratch(buffer):
+        for _ in range(2):
+            with _scratch.operator_call():
+                first = _scratch.allocate(1000, cpu)
+                second = _scratch.allocate(2000, cpu)
+                assert first.data_ptr() % 256 == 0 and second.data_ptr() % 256 == 0
+                assert buffer.data_ptr() <= first.data_ptr() and second.data_ptr() + 2000 <= buffer.data_ptr() + 5000
+                assert second.data_ptr() >= first.data_ptr() + 1000
+                assert _scratch.allocate(3000, cpu) is None
+        with _scratch.operator_call():
+            assert _scratch.allocate(100, torch.device("meta")) is None     # another device than the buffer's
+    with _scratch.operator_call():
+        assert _scratch.allocate(6000, cpu) is not None          # outside the block: torch's allocator again

@@ -306,3 +306,48 @@ def test_sets_of_near_duplicates_go_to_the_direct_kernel_whole(device):
         plain2 = kermac.cdist(a2, b2, p=2.0)
     assert not torch.equal(got2, plain2)
     assert_close_to_truth(got2[0][:512, :768], torch.cdist(a2[:512].double(), b2[:768].double(), p=2.0), rtol=1e-5, what="spread-out data")
+
+
+def test_the_kept_split_is_made_again_when_it_is_not_the_one_needed(device, wide):
+    """KMC_FLAG_GRAM_A_KEPT on a workspace that holds no split of this `a` (never used, used for another `a`, used by
+    another route in between): the library notices from its record of the workspace and makes the split; the result is
+    that of a call without the flag, bit for bit."""
+    g = torch.Generator().manual_seed(41)
+    a1 = torch.randn(600, 96, generator=g).to(device)
+    a2 = torch.randn(600, 96, generator=g).to(device)
+    b = torch.randn(500, 96, generator=g).to(device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+
+    def plan_for(a):
+        plan = module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, a, b, None, None, None, None, None, None, None, 0, 0, False)
+        plan.keepalive.append(module._attach_gram_centre(plan.params, stream, device))
+        return plan
+
+    plan1, plan2 = plan_for(a1), plan_for(a2)
+    needed = _backend.gram_workspace_bytes(plan1.params)
+    assert needed > 0 and needed == _backend.gram_workspace_bytes(plan2.params)
+    workspace = torch.zeros(needed, dtype=torch.uint8, device=device)
+    for plan in (plan1, plan2):
+        plan.params.gram_workspace, plan.params.gram_workspace_bytes = workspace.data_ptr(), needed
+    expected1 = kermac.cdist(a1, b, p=2.0).clone()
+    expected2 = kermac.cdist(a2, b, p=2.0).clone()
+    # the workspace has never held a split: the flag is set all the same
+    plan1.params.flags |= _backend.FLAG_GRAM_A_KEPT
+    _backend.build_kernel(plan1.params, stream)
+    assert torch.equal(plan1.out, expected1)
+    # now it holds the split of a1: kept for a1 (same bits), made again for a2
+    plan1.out.fill_(-1.0)
+    _backend.build_kernel(plan1.params, stream)
+    assert torch.equal(plan1.out, expected1)
+    plan2.params.flags |= _backend.FLAG_GRAM_A_KEPT
+    _backend.build_kernel(plan2.params, stream)
+    assert torch.equal(plan2.out, expected2)
+    # another route writes into the workspace in between (the fixed-point route of absolute differences)
+    l1 = module._plan_run_kernel(kermac.kernel_descriptor_l1_norm, a2, b, None, None, None, None, None, None, None, 0, 0, False)
+    l1.params.flags |= _backend.FLAG_L1_FIXED | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
+    assert 0 < _backend.gram_workspace_bytes(l1.params) <= needed
+    l1.params.gram_workspace, l1.params.gram_workspace_bytes = workspace.data_ptr(), needed
+    _backend.build_kernel(l1.params, stream)
+    plan2.out.fill_(-1.0)
+    _backend.build_kernel(plan2.params, stream)
+    assert torch.equal(plan2.out, expected2)

@@ -120,3 +120,41 @@ def test_static_scratch_rejects_what_does_not_fit_and_what_it_does_not_do(device
     with pytest.raises(_backend.BackendError, match="not compiled ahead of time"):
         _backend.build_kernel_cut_static(jit_only, 2, stream)
     assert _backend.STATIC_SCRATCH_BYTES == 64 << 20
+    no_result = block(a, a, out, True, 1, 0)
+    no_result.c = 0
+    with pytest.raises(_backend.BackendError, match="c: null pointer"):          # before anything is launched
+        _backend.build_kernel_cut_static(no_result, 2, stream)
+    fixed = block(a, a, out, True, 1, 0)
+    fixed.flags = _backend.FLAG_L1_FIXED
+    with pytest.raises(_backend.BackendError, match="fixed-point"):
+        _backend.build_kernel_cut_static(fixed, 2, stream)
+
+
+def test_static_scratch_replays_from_a_hip_graph(device):
+    """After one eager call (which looks up the array's address on this device) the entry point is captured into a
+    HIP graph; every replay, with eager work on the shared array and synchronisation in between, gives the bits of the
+    two-call form."""
+    g = torch.Generator().manual_seed(77)
+    M, N, K, ranges = 260, 190, 3000, 6
+    a, b = operands(M, N, K, True, device, g)
+    expected = torch.empty(N, M, device=device)
+    got = torch.empty(N, M, device=device)
+    other = torch.empty(90, 100, device=device)
+    a2, b2 = operands(100, 90, 800, True, device, g)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    two_call_form(block(a, b, expected, True, 1, 0, kernel_type=1, bandwidth=float(K)), ranges, device, stream)
+    params = block(a, b, got, True, 1, 0, kernel_type=1, bandwidth=float(K))
+    _backend.build_kernel_cut_static(params, ranges, stream)                     # eager: the address is looked up here
+    torch.cuda.synchronize()
+    assert torch.equal(got, expected)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _backend.build_kernel_cut_static(params, ranges, torch.cuda.current_stream(device).cuda_stream)
+    for replay in range(3):
+        got.fill_(float("nan"))
+        # eager work in between that overwrites the shared array with another problem's partial sums
+        _backend.build_kernel_cut_static(block(a2, b2, other, True, 2, 3), 4, torch.cuda.current_stream(device).cuda_stream)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, expected), f"replay {replay} differs from the two-call form"
