@@ -219,17 +219,14 @@ typedef struct kmc_build_kernel_params {
 } kmc_build_kernel_params;
 
 /* Bytes of gram_workspace that kmc_build_kernel would use for these parameters, 0 when it would
- * not use one (neither KMC_FLAG_L2_GRAM_BF16 with squared differences nor KMC_FLAG_DOT_PIECES with
- * products, or a problem too small to gain: fewer than 128 tiles of
- * 256 x 256 over the batch, k < 64, tiles * k below 147456 with fewer than 768 tiles, fewer tiles within a batch entry than
- * tiles_m * tiles_n >= 2.5 * (tiles_m + tiles_n), or more than 20 % of the tiles' area padding; of
- * a panel against itself the tiles on and below the diagonal count, and the panel is split once;
- * squared differences of operands that both have k contiguous take the route from 48 tiles, k = 256 and
- * tiles * k = 36864 on, whatever the shape of a batch entry, unless m or n is at most 128;
- * sums of products take it from k = 128, 64 tiles and tiles * k = 65536 on with at most 20 % padding, and from
- * k = 256 on from 32 tiles (64 for l = 1) and tiles * k = 24576 on whatever the padding;
- * KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE sets the size rules aside).  About 1.1 times the bytes of the
- * operands.  No counterpart in the reference. */
+ * not use one: none of KMC_FLAG_L2_GRAM_BF16 with squared differences, KMC_FLAG_DOT_PIECES with
+ * products and KMC_FLAG_L1_FIXED with absolute differences, or a problem too small to gain by the
+ * library's rule for that route.  The rules weigh the tiles over the batch (of a panel against
+ * itself: those on and below the diagonal; the panel is split once), the contraction length, tiles
+ * in both directions of every batch entry, the share of padding, and whether k is the contiguous
+ * index of both operands; their thresholds are the table that kmc_dispatch_rules() prints, the
+ * only place where those numbers are kept.  KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE sets the size rules
+ * aside.  About 1.1 times the bytes of the operands.  No counterpart in the reference. */
 int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *bytes);
 
 /* Stands in for launch(stream, config, cute_build_kernel<...>, *args)
@@ -331,8 +328,8 @@ typedef struct kmc_norm_gradient_params {
 } kmc_norm_gradient_params;
 
 /* Bytes of workspace that kmc_norm_kernel_gradient would use for these parameters, 0 when it would
- * not use one.  KMC_NORM_L1: at least 3 outputs, n >= 24 and m * n * k * l terms of at least
- * 6.4e9 / o (4e8 at 16 outputs), with more than 16 outputs of at least 1.5e7; about 1.1 times the
+ * not use one.  KMC_NORM_L1: enough outputs, columns n and terms m * n * k * l (the GRADIENT_F16 lines
+ * of kmc_dispatch_rules(); 4e8 terms at 16 outputs), and n within one grid dimension; about 1.1 times the
  * bytes of a, b and c.  KMC_NORM_L2:
  * when a model of both times favours the route by 15 % (tiles of 256 x 256 over m and o * n, in
  * both directions, and a contraction of about 512 or more); about 4 (m + 2 o n) k bytes.
@@ -441,6 +438,11 @@ int kmc_build_kernel_load_modes(const kmc_build_kernel_params *params, int32_t *
 
 /* ---- misc ---- */
 int kmc_abi_version(void);
+/* The thresholds of the library's rules for its routes through a workspace (which
+ * kmc_gram_workspace_bytes and kmc_norm_gradient_workspace_bytes apply) as text, one
+ * "NAME = integer" per line, into buf (4096 bytes are enough).  A tile is 256 x 256 for the
+ * matrix-core routes and 128 x 128 for the fixed-point one.  No counterpart in the reference. */
+int kmc_dispatch_rules(char *buf, size_t buf_len);
 /* Message of the last failing call on this thread ("" if none). */
 const char *kmc_last_error(void);
 /* gcnArchName of `device` (e.g. "gfx950:sramecc+:xnack-") into buf. */

@@ -113,6 +113,7 @@ SIGNATURES = {
     "kmc_abi_version": (ctypes.c_int, []),
     "kmc_last_error": (c_char_p, []),
     "kmc_device_arch": (ctypes.c_int, [ctypes.c_int, c_char_p, c_size_t]),
+    "kmc_dispatch_rules": (ctypes.c_int, [c_char_p, c_size_t]),
     "kmc_build_kernel_has_variant": (ctypes.c_int, [c_int32, c_int32]),
     "kmc_build_kernel": (ctypes.c_int, [POINTER(BuildKernelParams), c_void_p]),
     "kmc_build_kernel_jit": (ctypes.c_int, [c_void_p, POINTER(BuildKernelParams), c_void_p]),
@@ -267,6 +268,17 @@ def matrix_times_coefficients(params: MatrixCoefficientsParams, stream: int) -> 
 
 def kernel_times_coefficients_has_variant(inner_operator: int, inner_power: int) -> bool:
     return bool(library().kmc_kernel_times_coefficients_has_variant(inner_operator, inner_power))
+
+
+def dispatch_rules() -> dict:
+    """The library's table of thresholds for its routes through a workspace: {name: integer}."""
+    buf = ctypes.create_string_buffer(4096)
+    check(library().kmc_dispatch_rules(buf, 4096))
+    rules = {}
+    for text in buf.value.decode().splitlines():
+        name, _, value = text.partition("=")
+        rules[name.strip()] = int(value)
+    return rules
 
 
 def device_arch(device: int) -> str:

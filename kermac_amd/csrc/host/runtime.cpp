@@ -1,5 +1,6 @@
 // Error reporting, device checks, and the hiprtc / hipModule wrappers of the C ABI.
 #include "host_common.hpp"
+#include "dispatch_rules.hpp"
 
 #include <hip/hiprtc.h>
 
@@ -66,6 +67,24 @@ using namespace kmc_host;
 extern "C" {
 
 int kmc_abi_version(void) { return KMC_ABI_VERSION; }
+
+int kmc_dispatch_rules(char *buf, size_t buf_len)
+{
+    static const struct { const char *name; long long value; } rules[] = {
+#define KMC_LIST_RULE(name, value) {#name, value},
+        KMC_DISPATCH_RULES(KMC_LIST_RULE)
+#undef KMC_LIST_RULE
+    };
+    if (!buf || buf_len == 0) return fail(KMC_ERR_INVALID_ARGUMENT, "kmc_dispatch_rules: no buffer");
+    size_t used = 0;
+    for (const auto &rule : rules) {
+        const int wrote = std::snprintf(buf + used, buf_len - used, "%s = %lld\n", rule.name, rule.value);
+        if (wrote < 0 || static_cast<size_t>(wrote) >= buf_len - used)
+            return fail(KMC_ERR_INVALID_ARGUMENT, "kmc_dispatch_rules: the buffer of %zu bytes is too small", buf_len);
+        used += static_cast<size_t>(wrote);
+    }
+    return KMC_OK;
+}
 
 const char *kmc_last_error(void) { return g_last_error.c_str(); }
 

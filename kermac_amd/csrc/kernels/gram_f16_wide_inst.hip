@@ -10,6 +10,7 @@
 #include <unordered_map>
 
 #include "../host/host_common.hpp"
+#include "../host/dispatch_rules.hpp"
 #include "launch.hpp"
 #include "gram_f16_wide.hpp"
 #include "norm_gradient_l2_wide.hpp"
@@ -19,6 +20,8 @@ namespace kmc_host {
 namespace {
 
 constexpr int64_t REGION_ALIGN = 256;
+static_assert(kmc::GW_PROBE_PAIRS == kmc_rules::PROBE_PAIRS && kmc::GW_PROBE_BAIL == kmc_rules::PROBE_BAIL_PER_16384,
+              "the device constants of the sample of pairs are those of the table of rules");
 
 struct OperandRegions {
     int rows_pad, batches;
@@ -70,15 +73,20 @@ bool wide_pays(int64_t m, int64_t n, int64_t tiles_m, int64_t tiles_n, int64_t t
     const char *text = std::getenv("KERMAC_AMD_WIDE_MIN_TILES");
     const int forced = text ? std::atoi(text) : 0;
     if (forced > 0) return tiles >= forced && k >= 1;
-    if (k_contiguous && !products && k >= 256 && tiles >= 48 && tiles * k >= 36864 && m > kmc::GW_TILE / 2 && n > kmc::GW_TILE / 2) return true;
-    if (products && k >= 256 && tiles * k >= 24576 && tiles >= (batched ? 32 : 64)) return true;
-    if (products)
-        return k >= 128 && tiles >= 64 && tiles * k >= 65536 && 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
+    namespace r = kmc_rules;
+    if (k_contiguous && !products && k >= r::WIDE_K_CONTIGUOUS_MIN_K && tiles >= r::WIDE_K_CONTIGUOUS_MIN_TILES &&
+        tiles * k >= r::WIDE_K_CONTIGUOUS_MIN_TILES_TIMES_K && m >= r::WIDE_K_CONTIGUOUS_MIN_ROWS && n >= r::WIDE_K_CONTIGUOUS_MIN_ROWS)
+        return true;
+    const bool little_padding = 100 * m * n >= (100 - r::WIDE_MAX_PADDING_PERCENT) * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
+    if (products && k >= r::DOT_LONG_K && tiles * k >= r::DOT_LONG_MIN_TILES_TIMES_K &&
+        tiles >= (batched ? r::DOT_LONG_MIN_TILES_BATCHED : r::DOT_LONG_MIN_TILES_SINGLE))
+        return true;
+    if (products) return k >= r::DOT_MIN_K && tiles >= r::DOT_MIN_TILES && tiles * k >= r::DOT_MIN_TILES_TIMES_K && little_padding;
     // (from 768 tiles on the route is as fast as the one-step kernel also for the shortest contractions
     // it takes, 8192 x 8192 x 64 180 us against 187, and ahead of the direct kernel, 236)
-    if (k < 64 || tiles < 128 || (tiles * k < 147456 && tiles < 768)) return false;
-    if (2 * tiles_m * tiles_n < 5 * (tiles_m + tiles_n)) return false;
-    return 5 * m * n >= 4 * (tiles_m * kmc::GW_TILE) * (tiles_n * kmc::GW_TILE);
+    if (k < r::WIDE_MIN_K || tiles < r::WIDE_MIN_TILES || (tiles * k < r::WIDE_MIN_TILES_TIMES_K && tiles < r::WIDE_TILES_FOR_ANY_K)) return false;
+    if (2 * tiles_m * tiles_n < r::WIDE_MIN_TILES_PER_SIDE_X2 * (tiles_m + tiles_n)) return false;
+    return little_padding;
 }
 
 int64_t place(int64_t &cursor, int64_t bytes)
@@ -267,7 +275,7 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     // that data the trust rule would reject wholesale (sets of near-duplicates) costs the direct
     // kernel's time and little more, instead of both.  KMC_FLAG_NO_PROBE leaves it out.
     if (!products && !(p->flags & KMC_FLAG_NO_PROBE) &&
-        static_cast<int64_t>(layout.tiles_m) * layout.tiles_n * args.l * layout.slices >= 65536) {      // 0.5 ms and more: the sample is 10 us
+        static_cast<int64_t>(layout.tiles_m) * layout.tiles_n * args.l * layout.slices >= kmc_rules::PROBE_MIN_TILES_TIMES_SLICES) {      // 0.5 ms and more: the sample is 10 us
         wide.probe = reinterpret_cast<unsigned *>(workspace + layout.probe);
         wide.probe_pairs = kmc::GW_PROBE_PAIRS / args.l > 1024 ? kmc::GW_PROBE_PAIRS / args.l : 1024;
         void *clear_args[] = {&wide.probe};
@@ -325,7 +333,7 @@ bool gradient_l2_pays(const kmc_norm_gradient_params *p, int64_t tiles_m, int64_
     const double padded = static_cast<double>(tiles_m) * tiles_n * kmc::GW_TILE * kmc::GW_TILE * p->k * p->l;
     const double walk_us = padded * 6.3e-9 > 0.056 * p->k ? padded * 6.3e-9 : 0.056 * p->k;
     const double route_us = 200.0 + 1.5e-6 * (static_cast<double>(o) * p->n + p->m) * p->k * p->l + walk_us;
-    return 1.15 * route_us < fp32_us;
+    return (100 + kmc_rules::GRADIENT_L2_ADVANTAGE_PERCENT) * route_us < 100 * fp32_us;
 }
 
 bool gradient_l2_layout(const kmc_norm_gradient_params *p, GradientL2Layout *layout)

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include "../host/host_common.hpp"
+#include "../host/dispatch_rules.hpp"
 #include "launch.hpp"
 #include "l1_fixed.hpp"
 
@@ -18,7 +19,7 @@ constexpr int SAMPLE_PAIRS = 1024;
 // a problem whose walk is long against both.  (KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE sets the rule aside.)
 bool fixed_pays(int64_t tiles, int k)
 {
-    return tiles >= 2048 && k >= 128;
+    return tiles >= kmc_rules::L1_FIXED_MIN_TILES && k >= kmc_rules::L1_FIXED_MIN_K;
 }
 
 struct FixedLayout {

@@ -8,6 +8,7 @@
 #include <type_traits>
 
 #include "../host/host_common.hpp"
+#include "../host/dispatch_rules.hpp"
 #include "launch.hpp"
 #include "norm_gradient_f16.hpp"
 
@@ -69,8 +70,10 @@ bool f16_pays(const kmc_norm_gradient_params *p)
     // more than 16 outputs: the wider tiles of the route share the sign work between blocks of outputs, while the
     // fp32 kernels go to their 32-column tiles (O = 32: 98 against 75 us at 1.7e7 terms, 187 against 128 at 2.7e8;
     // O = 128: 101 against 70 and 588 against 206)
-    if (p->o > 16) return p->n >= 24 && terms >= 1.5e7;
-    return p->o >= 3 && p->n >= 24 && terms * p->o >= 6.4e9;
+    namespace r = kmc_rules;
+    if (p->o > 16) return p->n >= r::GRADIENT_F16_MIN_N && terms >= static_cast<double>(r::GRADIENT_F16_MANY_OUTPUTS_MIN_TERMS);
+    return p->o >= r::GRADIENT_F16_MIN_OUTPUTS && p->n >= r::GRADIENT_F16_MIN_N &&
+           terms * p->o >= static_cast<double>(r::GRADIENT_F16_MIN_TERMS_TIMES_OUTPUTS);
 }
 
 bool gradient_layout(const kmc_norm_gradient_params *p, GradientLayout *layout)

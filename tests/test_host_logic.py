@@ -861,3 +861,39 @@ def test_scratch_memory_is_handed_out_within_the_limit_or_from_the_callers_buffe
             assert _scratch.allocate(100, torch.device("meta")) is None     # another device than the buffer's
     with _scratch.operator_call():
         assert _scratch.allocate(6000, cpu) is not None          # outside the block: torch's allocator again
+
+
+def test_the_dispatch_table_of_the_design_is_the_generated_one():
+    """One source of truth for "which kernel runs when": the thresholds live in csrc/host/dispatch_rules.hpp (read by the
+    library's rules, printed by kmc_dispatch_rules) and in the Python layer's module constants; kermac_amd.dispatch renders the
+    table from them, and the copy in DESIGN.md must be that rendering.  The rules themselves must flip at the printed numbers."""
+    from kermac_amd import dispatch
+    known = dispatch.rules()
+    table = dispatch.table_markdown()
+    design = (ROOT / "DESIGN.md").read_text()
+    assert table in design, "DESIGN.md: regenerate the dispatch table with `python -m kermac_amd.dispatch`"
+    header = (ROOT / "include" / "kermac_amd.h").read_text()
+    assert "kmc_dispatch_rules" in header and "147456" not in header and "36864" not in header      # pointed to, not restated
+    fake = 4096
+
+    def wants_workspace(m, n, k, inner_power, flags, l=1):
+        params = _backend.BuildKernelParams()
+        params.inner_operator, params.inner_power = 0, inner_power
+        params.m, params.n, params.k, params.l = m, n, k, l
+        params.a, params.a_ld, params.a_bs = fake, m, m * k
+        params.b, params.b_ld, params.b_bs = fake + 4 * m * k * l, n, n * k
+        params.c_ld, params.c_bs = m, m * n
+        params.flags = flags
+        return _backend.gram_workspace_bytes(params) > 0
+
+    wide = _backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16
+    side = 256 * 12                                                     # 144 tiles of 256 x 256
+    assert known["WIDE_MIN_TILES"] <= 144 < known["WIDE_TILES_FOR_ANY_K"]
+    k_needed = -(-known["WIDE_MIN_TILES_TIMES_K"] // 144)
+    assert wants_workspace(side, side, k_needed, 2, wide) and not wants_workspace(side, side, k_needed - 1, 2, wide)
+    assert not wants_workspace(8192, 8192, known["WIDE_MIN_K"] - 1, 2, wide) and wants_workspace(8192, 8192, known["WIDE_MIN_K"], 2, wide)
+    rows = 128 * 46                                                     # 46 x 46 = 2116 tiles of 128 x 128
+    assert known["L1_FIXED_MIN_TILES"] <= 2116
+    assert wants_workspace(rows, rows, known["L1_FIXED_MIN_K"], 1, _backend.FLAG_L1_FIXED)
+    assert not wants_workspace(rows, rows, known["L1_FIXED_MIN_K"] - 1, 1, _backend.FLAG_L1_FIXED)
+    assert not wants_workspace(128 * 45, 128 * 45, 512, 1, _backend.FLAG_L1_FIXED) and 45 * 45 < known["L1_FIXED_MIN_TILES"]
