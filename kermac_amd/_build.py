@@ -156,5 +156,18 @@ def build_c_example(verbose: bool = False) -> Path:
 
 
 if __name__ == "__main__":
-    path = build(force="--incremental" not in sys.argv, verbose="-v" in sys.argv)
+    # python -m kermac_amd._build [--incremental] [-v] [--define NAME[=VALUE]]... [--output PATH]
+    # --define / --output build a variant of the library elsewhere (the measurement switches of the kernel headers,
+    # e.g. --define NGF_ABLATE_NO_SIGN --output /tmp/no_sign/libkermac_amd.so; KERMAC_AMD_LIBRARY=PATH then loads it)
+    arguments = sys.argv[1:]
+    defines, output = [], None
+    while "--define" in arguments:
+        at = arguments.index("--define")
+        defines.append("-D" + arguments[at + 1])
+        del arguments[at:at + 2]
+    if "--output" in arguments:
+        at = arguments.index("--output")
+        output = Path(arguments[at + 1])
+        del arguments[at:at + 2]
+    path = build(force="--incremental" not in arguments, verbose="-v" in arguments, extra_flags=defines, lib_path=output)
     print(path)

@@ -35,6 +35,16 @@
 // the same), a software pipeline that makes the pieces of the next (n, row block) between the three
 // matrix instructions of this one, pinned with scheduling groups (co-issue rises to 47 % of the
 // matrix cycles, but the kernel takes more cycles: 4.1 .. 4.3 ms), D parked in LDS to free registers.
+// Two compile-time switches leave a part of the walk out, for the measurement of what bounds it (the results are
+// then wrong): -DNGF_ABLATE_NO_SIGN multiplies the pieces of A as they are, -DNGF_ABLATE_NO_MFMA makes the signed
+// pieces and issues no matrix instruction.  Measured with them at M = K = 8192, N = 512, O = 16: matrix instructions and
+// copies alone 2.01 ms (3.46e6 cycles at 1.72 GHz, the matrix pipeline busy 91 % of them), sign work and copies alone
+// 2.04 ms (4.17e6 cycles at 2.05 GHz), both 3.72 ms (6.83e6 cycles at 1.84 GHz): the two parts take nine tenths of
+// the sum of their cycles, whichever wave they come from -- a source-level pipeline that puts the vector work of pair
+// i + 1 between the three dependent matrix instructions of pair i (one matrix instruction, seven vector instructions,
+// three times; 255 registers) took 4.28 ms against 4.12 ms on the same box.  This 16-bit matrix instruction and the
+// vector ALU do not run side by side here; the kernel is at the sum of two floors, each already at its minimum of
+// instructions (2.5 vector instructions per (m, n, k) without packed fp32; three piece products).
 #pragma once
 
 #include "gram_f16_wide.hpp"
@@ -233,6 +243,7 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
             for (int mb = 0; mb < 4; mb++) {
                 gram_chunk t1 = __builtin_bit_cast(gram_chunk, fa[mb][0]);
                 gram_chunk t2 = __builtin_bit_cast(gram_chunk, fa[mb][1]);
+#ifndef NGF_ABLATE_NO_SIGN
 #pragma unroll
                 for (int pair = 0; pair < 4; pair++) {
                     const unsigned low = __float_as_uint(dval[nb][mb] - bk[2 * pair]);
@@ -243,14 +254,19 @@ __global__ __launch_bounds__(NGF_THREADS, 2) void norm_gradient_l1_f16(const Nor
                     t2[pair] ^= flip;
                 }
                 const gram_half8 h1 = __builtin_bit_cast(gram_half8, t1), h2 = __builtin_bit_cast(gram_half8, t2);
+#ifdef NGF_ABLATE_NO_MFMA
+                asm volatile("" : : "v"(h1), "v"(h2));      // the signed pieces are made and dropped
+#else
 #pragma unroll
                 for (int ob = 0; ob < O_BLOCKS; ob++) acc[nb][mb][ob] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h2, fc[ob][0], acc[nb][mb][ob], 0, 0, 0);
 #pragma unroll
                 for (int ob = 0; ob < O_BLOCKS; ob++) acc[nb][mb][ob] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[ob][1], acc[nb][mb][ob], 0, 0, 0);
 #pragma unroll
                 for (int ob = 0; ob < O_BLOCKS; ob++) acc[nb][mb][ob] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h1, fc[ob][0], acc[nb][mb][ob], 0, 0, 0);
+#endif
             }
         }
+#endif
         // the wave's own copies of the next step have arrived (the four of the step after it may
         // still be under way); behind the barrier everybody's have, and this step's buffer is free
         __builtin_amdgcn_s_waitcnt(0x0F70 | COPIES);            // vmcnt(COPIES)
