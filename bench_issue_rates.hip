@@ -372,6 +372,91 @@ __global__ __launch_bounds__(kmc::BK_THREADS, 2) void walk_wide_tile_counted(con
     if (tid == 0 && blockIdx.x == gridDim.x / 2) { clocks[0] = wall1 - wall0; clocks[1] = tick1 - tick0; }
 }
 
+
+// The walk with the panels copied from memory straight into LDS (global_load_lds_dwordx4: a wave writes two
+// k-rows of 128 floats, 1 KB, per instruction; no registers, no ds_write; LDS pitch 128 instead of 132) on its own,
+// at 4, 3 and 2 waves per SIMD: what the product kernel's interior tiles run (accumulate_tile_direct).  The variants
+// further up ("same walk", "no global loads" ...) are the walk through staging registers that other layouts take.
+template <int WAVES>
+__global__ __launch_bounds__(kmc::BK_THREADS) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void walk_direct_to_lds(const kmc::BuildKernelArgs args, long long *clocks)
+{
+    constexpr int PITCH = kmc::BK_TILE_M, SLICE = kmc::BK_TILE_K * PITCH;
+    __shared__ __attribute__((aligned(16))) float lds_a[2 * SLICE + PITCH];
+    __shared__ __attribute__((aligned(16))) float lds_b[2 * SLICE + PITCH];
+    const int tid = threadIdx.x;
+    int tile_m, tile_n;
+    if (!kmc::tile_of_workgroup(args, tile_m, tile_n)) return;
+    const long long wall0 = wall_clock64(), tick0 = clock64();
+    const int m0 = tile_m * kmc::BK_TILE_M, n0 = tile_n * kmc::BK_TILE_N;
+    const int tx = tid & 15, ty = tid >> 4;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    typedef const __attribute__((address_space(1))) void *global_address;
+    typedef __attribute__((address_space(3))) void *lds_address;
+    // copy j of 2 per operand: k-rows 4 * wave + 2 * j + (lane >> 5), 16 bytes number lane & 31 of the row
+    const float *src_a[2], *src_b[2];
+    int dst[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int k_row = 4 * wave + 2 * j + (lane >> 5);
+        src_a[j] = args.a + (kmc::i64)k_row * args.a_ld + m0 + 4 * (lane & 31);
+        src_b[j] = args.b + (kmc::i64)k_row * args.b_ld + n0 + 4 * (lane & 31);
+        dst[j] = (4 * wave + 2 * j) * PITCH;
+    }
+    const kmc::i64 step_a = (kmc::i64)kmc::BK_TILE_K * args.a_ld, step_b = (kmc::i64)kmc::BK_TILE_K * args.b_ld;
+    auto copy_slice = [&](int buffer) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const unsigned to_a = (unsigned)(unsigned long)(lds_address)(lds_a + buffer * SLICE + dst[j]);
+            const unsigned to_b = (unsigned)(unsigned long)(lds_address)(lds_b + buffer * SLICE + dst[j]);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"((global_address)src_a[j]), "s"(to_a) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"((global_address)src_b[j]), "s"(to_b) : "memory", "m0");
+            src_a[j] += step_a;
+            src_b[j] += step_b;
+        }
+    };
+    float acc[8][8];
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[j][i] = 0.0f;
+    const int k_slices = args.k / kmc::BK_TILE_K;
+    copy_slice(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+    __syncthreads();
+    for (int slice = 0; slice < k_slices; slice++) {
+        const int cur = slice & 1;
+        if (slice + 1 < k_slices) copy_slice(cur ^ 1);
+        const float *sa = lds_a + cur * SLICE + tx * 4;
+        const float *sb = lds_b + cur * SLICE + ty * 4;
+        float fa0[8], fb0[8], fa1[8], fb1[8];
+        kmc::read_fragment(fa0, sa); kmc::read_fragment(fb0, sb);
+#pragma unroll 1
+        for (int kk = 0; kk < kmc::BK_TILE_K; kk += 2) {
+            kmc::read_fragment(fa1, sa + (kk + 1) * PITCH); kmc::read_fragment(fb1, sb + (kk + 1) * PITCH);
+            kmc::rank1_update<kmc::OP_DIFF, kmc::POW_ABS>(acc, fa0, fb0, 0.0f, 1.0f);
+            kmc::read_fragment(fa0, sa + (kk + 2) * PITCH); kmc::read_fragment(fb0, sb + (kk + 2) * PITCH);
+            kmc::rank1_update<kmc::OP_DIFF, kmc::POW_ABS>(acc, fa1, fb1, 0.0f, 1.0f);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // this wave's copies of the next slice have landed
+        __syncthreads();
+    }
+    const long long wall1 = wall_clock64(), tick1 = clock64();
+    const int m_valid = args.m - m0, n_valid = args.n - n0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int n_local = ty * 4 + (j & 3) + (j >> 2) * 64;
+        if (n_local >= n_valid) continue;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int m_local = tx * 4 + h * 64;
+            float *dst_c = args.c + (kmc::i64)(n0 + n_local) * args.c_ld + m0 + m_local;
+            if (m_local + 3 < m_valid)
+                *reinterpret_cast<float4 *>(dst_c) = make_float4(acc[j][4 * h], acc[j][4 * h + 1], acc[j][4 * h + 2], acc[j][4 * h + 3]);
+        }
+    }
+    if (tid == 0 && blockIdx.x == gridDim.x / 2) { clocks[0] = wall1 - wall0; clocks[1] = tick1 - tick0; }
+}
+
 #define CHECK_VOID(x) \
     do { \
         hipError_t e_ = (x); \
@@ -414,7 +499,8 @@ int walk_ablations()
     kmc::BuildKernelArgs d = {};
     d.m = M; d.n = N; d.k = K; d.l = 1; d.a = a; d.a_ld = Mp; d.b = b; d.b_ld = Np; d.c = c; d.c_ld = M;
     d.diff_sign = 1.0f; d.c_vec = 1; d.tiles_m = tiles_m; d.tiles_n = tiles_n; d.tiles_n_padded = tiles_n_padded; d.grid_width = grid.x;
-    run("product kernel build_kernel<DIFF, ABS>", [&] { kmc::build_kernel<kmc::OP_DIFF, kmc::POW_ABS, kmc::LOAD_COL_VEC, kmc::LOAD_COL_VEC><<<grid, 256>>>(d); }, clocks, reps);
+    run("product kernel build_kernel_four_waves<DIFF, ABS>", [&] { kmc::build_kernel_four_waves<kmc::OP_DIFF, kmc::POW_ABS><<<grid, 256>>>(d); }, clocks, reps);
+    run("product kernel at three waves per SIMD, build_kernel<DIFF, ABS>", [&] { kmc::build_kernel<kmc::OP_DIFF, kmc::POW_ABS, kmc::LOAD_COL_VEC, kmc::LOAD_COL_VEC><<<grid, 256>>>(d); }, clocks, reps);
     run("same walk, clocks read (all traffic)", [&] { walk_variant<false, false, false, false><<<grid, 256>>>(d, clocks); }, clocks, reps);
     run("no global loads in the walk", [&] { walk_variant<true, false, false, false><<<grid, 256>>>(d, clocks); }, clocks, reps);
     run("no global loads, no LDS writes", [&] { walk_variant<true, false, true, false><<<grid, 256>>>(d, clocks); }, clocks, reps);
@@ -427,9 +513,16 @@ int walk_ablations()
     const dim3 wide_grid(tiles_m * ((tiles_n2 + 7) / 8 * 8));
     run("tile of 128 x 256, 8 x 16 results per lane, 2 waves per SIMD", [&] { walk_wide_tile<<<wide_grid, 256>>>(d, clocks); }, clocks, reps);
     run("the same with the LDS waits counted by hand", [&] { walk_wide_tile_counted<<<wide_grid, 256>>>(d, clocks); }, clocks, reps);
+    run("product walk, panels copied straight into LDS, 4 waves per SIMD", [&] { walk_direct_to_lds<4><<<grid, 256>>>(d, clocks); }, clocks, reps);
+    run("the same, 3 waves per SIMD", [&] { walk_direct_to_lds<3><<<grid, 256>>>(d, clocks); }, clocks, reps);
+    run("the same, 2 waves per SIMD", [&] { walk_direct_to_lds<2><<<grid, 256>>>(d, clocks); }, clocks, reps);
+    run("product kernel build_kernel_four_waves<DIFF, ABS> again", [&] { kmc::build_kernel_four_waves<kmc::OP_DIFF, kmc::POW_ABS><<<grid, 256>>>(d); }, clocks, reps);
+    float direct_element;
+    CHECK_VOID(hipMemcpy(&direct_element, c + (size_t)12345 * M + 6789, 4, hipMemcpyDeviceToHost));
+    printf("one element from the walk with direct copies %.6f\n", direct_element);
     float got[2];
     CHECK_VOID(hipMemcpy(got, c + (size_t)12345 * M + 6789, 4, hipMemcpyDeviceToHost));
-    kmc::build_kernel<kmc::OP_DIFF, kmc::POW_ABS, kmc::LOAD_COL_VEC, kmc::LOAD_COL_VEC><<<grid, 256>>>(d);
+    kmc::build_kernel_four_waves<kmc::OP_DIFF, kmc::POW_ABS><<<grid, 256>>>(d);
     CHECK_VOID(hipMemcpy(got + 1, c + (size_t)12345 * M + 6789, 4, hipMemcpyDeviceToHost));
     printf("one element from the wide tile %.6f, from the product kernel %.6f\n", got[0], got[1]);
     return 0;

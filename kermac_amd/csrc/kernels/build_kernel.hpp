@@ -314,6 +314,71 @@ __device__ __forceinline__ void read_fragment(float (&f)[8], const float *p)
     f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
 }
 
+// The K walk of an interior tile whose two panels have their rows contiguous and allow 128-bit access (the
+// benchmark's storage): the slices go from memory straight into LDS.  global_load_lds_dwordx4 writes the 64 x 16
+// bytes of a wave to consecutive LDS addresses, which for these panels are two whole k-rows of 128 floats, so
+// the row pitch here is 128 (the 132 of the other loaders only serves their transposing writes).  A lane's
+// source address is that of its loader (k-row tid / 32 of the slice, and the one 8 rows further for the
+// second copy).  No staging registers and no ds_write: measured on the p = 1 walk at M = N = 30000, K = 1024,
+// same box, 29.49 -> 28.86 ms.  The copies are written as instructions because the compiler would make every
+// LDS read wait for all of them; it does not count them, so the walk waits for them itself (vmcnt(0) before
+// the barrier that publishes a slice) and issues no other vector memory instruction meanwhile.
+// `update(fa, fb)` adds the 8 x 8 terms of one k to the caller's accumulators.
+template <typename Update>
+__device__ __forceinline__ void walk_with_direct_copies(
+    TileLoader<LOAD_COL_VEC> &load_a, TileLoader<LOAD_COL_VEC> &load_b, float *lds_a, float *lds_b, int k_slices, int tx, int ty,
+    Update &&update)
+{
+    constexpr int PITCH = BK_TILE_M, SLICE = BK_TILE_K * PITCH;
+    static_assert(2 * SLICE + PITCH <= 2 * BK_LDS_SLICE + BK_LDS_PITCH, "the two slices and the pad row fit the staging arrays");
+    typedef const __attribute__((address_space(1))) void *global_address;
+    typedef __attribute__((address_space(3))) void *lds_address;
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const float *src_a = load_a.ptr, *src_b = load_b.ptr;      // of the next slice to copy
+    auto copy_slice = [&](int buffer) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            // k-rows 2 wave + 8 j and the next one of the slice
+            const unsigned to_a = (unsigned)(unsigned long)(lds_address)(lds_a + buffer * SLICE + (2 * wave + 8 * j) * PITCH);
+            const unsigned to_b = (unsigned)(unsigned long)(lds_address)(lds_b + buffer * SLICE + (2 * wave + 8 * j) * PITCH);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         : : "v"((global_address)(src_a + (i64)(8 * j) * load_a.ld)), "s"(to_a) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         : : "v"((global_address)(src_b + (i64)(8 * j) * load_b.ld)), "s"(to_b) : "memory", "m0");
+        }
+        src_a += load_a.step;
+        src_b += load_b.step;
+    };
+    if (k_slices == 0) return;
+    // nothing the compiler loaded may be under way beside the copies: it does not know that they count too
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    copy_slice(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+    __syncthreads();
+    for (int slice = 0; slice < k_slices; slice++) {
+        const int cur = slice & 1;
+        if (slice + 1 < k_slices) copy_slice(cur ^ 1);
+        const float *sa = lds_a + cur * SLICE + tx * 4;
+        const float *sb = lds_b + cur * SLICE + ty * 4;
+        float fa0[8], fb0[8], fa1[8], fb1[8];
+        read_fragment(fa0, sa);
+        read_fragment(fb0, sb);
+#pragma unroll 1
+        for (int kk = 0; kk < BK_TILE_K; kk += 2) {
+            read_fragment(fa1, sa + (kk + 1) * PITCH);
+            read_fragment(fb1, sb + (kk + 1) * PITCH);
+            update(fa0, fb0);
+            read_fragment(fa0, sa + (kk + 2) * PITCH);       // last trip: the other buffer's first row or the pad row, never used
+            read_fragment(fb0, sb + (kk + 2) * PITCH);
+            update(fa1, fb1);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // this wave's copies of the next slice have landed
+        __syncthreads();
+    }
+    load_a.ptr = src_a;      // behind the last slice walked: a caller that walks a contraction in runs goes on from here
+    load_b.ptr = src_b;
+}
+
 // The K walk for one output tile.  FULL = the tile is interior and K is a
 // multiple of the slice depth, so no load needs a predicate; the compiler then
 // produces a branch-free steady-state loop.
@@ -327,6 +392,14 @@ __device__ __forceinline__ void accumulate_tile(
     float stage_a[8], stage_b[8];
 
     if (k_slices == 0) return;
+#ifndef BK_NO_DIRECT_COPIES
+    if constexpr (FULL && LOAD_A == LOAD_COL_VEC && LOAD_B == LOAD_COL_VEC) {
+        walk_with_direct_copies(load_a, load_b, lds_a, lds_b, k_slices, tx, ty, [&](const float (&fa)[8], const float (&fb)[8]) {
+            rank1_update<INNER_OP, INNER_POW>(acc, fa, fb, p_inner, diff_sign);
+        });
+        return;
+    }
+#endif
     if (FULL) {
         load_a.load_full(stage_a);
         load_b.load_full(stage_b);
@@ -579,13 +652,11 @@ __device__ __forceinline__ void store_tile(
     }
 }
 
+// One output tile from start to finish; `lds_a` / `lds_b`: two slices per operand plus one pad row (see the fragment
+// prefetch).  The body of the two kernels below.
 template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
-__global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs args)
+__device__ __forceinline__ void build_kernel_tile(const BuildKernelArgs &args, float *lds_a, float *lds_b)
 {
-    // Two slices per operand plus one pad row (see the fragment prefetch).
-    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE + BK_LDS_PITCH];
-    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE + BK_LDS_PITCH];
-
     const int tid = threadIdx.x;
     const int batch = blockIdx.y;
     int tile_m, tile_n;
@@ -630,6 +701,30 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
     finish_tile(acc, args, batch, m0, n0, tx, ty);
 
     store_tile(acc, args, batch, tile_m, tile_n, m0, n0, m_valid, n_valid, tx, ty, tid, lds_a, lds_b, false);
+}
+
+template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>
+__global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs args)
+{
+    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+    build_kernel_tile<INNER_OP, INNER_POW, LOAD_A, LOAD_B>(args, lds_a, lds_b);
+}
+
+// The same kernel for panels with contiguous rows (both loaders LOAD_COL_VEC), compiled for four waves per SIMD.
+// Interior tiles of such panels take the walk with direct copies, whose loop needs no staging registers and fits
+// the 128 registers of four waves; what spills (about 20 registers) sits in the edge loaders and the epilogue.
+// Measured on that walk at M = N = 30000, K = 1024, same box: 28.13 ms at four waves, 28.49 at three, 30.51 at two;
+// the product kernels p = 1 29.7 against 30.1 .. 30.5 ms without direct copies, p = 2 31.6 against 32.6.  A launch
+// that is bound by its stores (K = 64: 0.68 against 0.66 ms) keeps the three-wave kernel; the host decides by K
+// (BK_FOUR_WAVES_MIN_K).
+constexpr int BK_FOUR_WAVES_MIN_K = 256;
+template <int INNER_OP, int INNER_POW>
+__global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_four_waves(const BuildKernelArgs args)
+{
+    __shared__ __attribute__((aligned(16))) float lds_a[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+    __shared__ __attribute__((aligned(16))) float lds_b[2 * BK_LDS_SLICE + BK_LDS_PITCH];
+    build_kernel_tile<INNER_OP, INNER_POW, LOAD_COL_VEC, LOAD_COL_VEC>(args, lds_a, lds_b);
 }
 
 }  // namespace kmc

@@ -221,8 +221,9 @@ __device__ __forceinline__ void row_sad(unsigned (&accrow)[8], const float (&fa)
                  : "v"(fa[0]), "v"(fa[1]), "v"(fa[2]), "v"(fa[3]), "v"(fa[4]), "v"(fa[5]), "v"(fa[6]), "v"(fa[7]), "v"(b));
 }
 
-// The walk: tiles, tile order, staging, fragment reads and stores of build_kernel, with the grid
-// words travelling through the float loaders untouched.
+// The walk: tiles, tile order, direct copies into LDS, fragment reads and stores of build_kernel (the images
+// are laid out like panels with contiguous rows, padded, so every tile is an interior one), with the grid
+// words travelling as floats untouched.
 // Four waves per SIMD: the compiler's own choice is 164 registers, set by the epilogue, not the walk, and three waves;
 // within 128 it spills 180 bytes per lane outside the walk, and the launch is 1.4 % faster
 // (M = N = 30000, K = 1024, same box: 26.7 -> 26.3 ms).
@@ -266,43 +267,10 @@ __global__ __launch_bounds__(BK_THREADS, L1F_MIN_WAVES) void l1_fixed_kernel(con
         for (int j = 0; j < 8; j++)
 #pragma unroll
             for (int i = 0; i < 8; i++) acc[j][i] = 0u;
-        float stage_a[8], stage_b[8];
-        load_a.load_full(stage_a);
-        load_b.load_full(stage_b);
-        load_a.store(lds_a, stage_a);
-        load_b.store(lds_b, stage_b);
-        __syncthreads();
-        for (int slice = 0; slice < slices; slice++) {
-            const int cur = slice & 1;
-            const bool has_next = slice + 1 < slices;
-            load_a.advance();
-            load_b.advance();
-            if (has_next) {
-                load_a.load_full(stage_a);
-                load_b.load_full(stage_b);
-            }
-            const float *sa = lds_a + cur * BK_LDS_SLICE + tx * 4;
-            const float *sb = lds_b + cur * BK_LDS_SLICE + ty * 4;
-            float fa0[8], fb0[8], fa1[8], fb1[8];
-            read_fragment(fa0, sa);
-            read_fragment(fb0, sb);
-#pragma unroll 1
-            for (int kk = 0; kk < BK_TILE_K; kk += 2) {
-                read_fragment(fa1, sa + (kk + 1) * BK_LDS_PITCH);
-                read_fragment(fb1, sb + (kk + 1) * BK_LDS_PITCH);
+        walk_with_direct_copies(load_a, load_b, lds_a, lds_b, slices, tx, ty, [&](const float (&fa)[8], const float (&fb)[8]) {
 #pragma unroll
-                for (int j = 0; j < 8; j++) row_sad(acc[j], fa0, fb0[j]);
-                read_fragment(fa0, sa + (kk + 2) * BK_LDS_PITCH);    // last trip: a row that is never used
-                read_fragment(fb0, sb + (kk + 2) * BK_LDS_PITCH);
-#pragma unroll
-                for (int j = 0; j < 8; j++) row_sad(acc[j], fa1, fb1[j]);
-            }
-            if (has_next) {
-                load_a.store(lds_a + (cur ^ 1) * BK_LDS_SLICE, stage_a);
-                load_b.store(lds_b + (cur ^ 1) * BK_LDS_SLICE, stage_b);
-            }
-            __syncthreads();
-        }
+            for (int j = 0; j < 8; j++) row_sad(acc[j], fa, fb[j]);
+        });
         // This run of terms as fp32, on top of the runs before it, which wait in the result.
         const bool add_earlier = first > 0;
         const bool more_to_come = first + slices < k_slices;
