@@ -464,6 +464,9 @@ def main():
     parser.add_argument("--l2-mode", choices=["auto", "direct", "gram", "gram_bf16"], default=None,
                         help="how squared differences (p = 2) are evaluated in the timed step; default: the library's "
                              "default, 'auto' (matrix cores with repair of ill-conditioned tiles for large problems)")
+    parser.add_argument("--l1-mode", choices=["direct", "fixed"], default=None,
+                        help="how absolute differences (p = 1) are evaluated in the timed step; default: the library's default, "
+                             "'direct' (fp32 on the vector ALU); 'fixed' is the opt-in fixed-point route (for profiling it)")
     parser.add_argument("--workload", choices=["cdist", "cdist_grad", "kernel_coef"], default="cdist",
                         help="cdist (default, the headline metric, with the other two configurations as extra keys); "
                              "cdist_grad = only the Laplace-kernel RFM gradient configuration; kernel_coef = only the "
@@ -482,6 +485,8 @@ def main():
 
     if args.l2_mode is not None:
         kermac.set_l2_mode(args.l2_mode)
+    if args.l1_mode is not None:
+        kermac.set_l1_mode(args.l1_mode)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     if args.workload != "cdist":
@@ -665,9 +670,12 @@ def main():
             other_configs[name]["steps"], other_configs[name]["warmup"] = side_steps, 1
 
     achieved = OPS_PER_CALL / kernel_ms / 1e9
-    traffic, traffic_source = measured_traffic() if headline_p == 1.0 else (None, None)
+    traffic, traffic_source = measured_traffic() if headline_p == 1.0 and kermac.get_l1_mode() == "direct" else (None, None)
     inner = {1.0: "POW_ABS", 2.0: "POW_SQUARE"}.get(headline_p, "POW_POW")
-    headline_kernel = f"kmc::build_kernel<OP_DIFF,{inner},LOAD_COL_VEC,LOAD_COL_VEC>"
+    headline_kernel = (f"kmc::build_kernel_four_waves<OP_DIFF,{inner}>" if inner != "POW_POW"
+                       else f"kmc::build_kernel<OP_DIFF,{inner},LOAD_COL_VEC,LOAD_COL_VEC>")
+    if headline_p == 1.0 and kermac.get_l1_mode() == "fixed":
+        headline_kernel = "kmc::l1_fixed_kernel (l1 mode fixed)"
     if headline_p == 2.0 and kermac.get_l2_mode() != "direct":
         headline_kernel = "kmc::gram_f16_wide / kmc::gram_bf16_l2_kernel / kmc::gram_l2_kernel (l2 mode %s)" % kermac.get_l2_mode()
     line = {
