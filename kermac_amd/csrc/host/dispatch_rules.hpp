@@ -1,6 +1,6 @@
 // Every threshold by which the library decides, from the shape of a call alone, whether a route
-// through a workspace applies.  This table is the only place where these numbers live: the rules
-// (wide_pays in kernels/gram_f16_wide_inst.hip, fixed_pays in kernels/l1_fixed_inst.hip, f16_pays in
+// through a workspace applies, and which variant of the direct kernel is launched.  This table is the only place where these numbers live: the rules
+// (launch_one in kernels/build_kernel_inst.hip, wide_pays in kernels/gram_f16_wide_inst.hip, fixed_pays in kernels/l1_fixed_inst.hip, f16_pays in
 // kernels/norm_gradient_f16_inst.hip, gradient_l2_pays in kernels/gram_f16_wide_inst.hip) read them
 // from here, kmc_dispatch_rules() prints them, and the Python layer builds its "which kernel runs
 // when" table from that print-out.  Where each number comes from (the sweeps) is told next to the rule
@@ -33,6 +33,8 @@
     X(PROBE_MIN_TILES_TIMES_SLICES, 65536)                                                              \
     X(PROBE_PAIRS, 16384)                                                                               \
     X(PROBE_BAIL_PER_16384, 4)                                                                          \
+    /* the direct kernel compiled for four waves per SIMD (k-major panels, no fractional power) */       \
+    X(DIRECT_FOUR_WAVES_MIN_K, 256)                                                                     \
     /* absolute differences on fixed point (KMC_FLAG_L1_FIXED): tiles of 128 x 128 over the batch */    \
     X(L1_FIXED_MIN_TILES, 2048)                                                                         \
     X(L1_FIXED_MIN_K, 128)                                                                              \

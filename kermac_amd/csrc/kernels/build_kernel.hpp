@@ -717,8 +717,7 @@ __global__ __launch_bounds__(BK_THREADS) void build_kernel(const BuildKernelArgs
 // Measured on that walk at M = N = 30000, K = 1024, same box: 28.13 ms at four waves, 28.49 at three, 30.51 at two;
 // the product kernels p = 1 29.7 against 30.1 .. 30.5 ms without direct copies, p = 2 31.6 against 32.6.  A launch
 // that is bound by its stores (K = 64: 0.68 against 0.66 ms) keeps the three-wave kernel; the host decides by K
-// (BK_FOUR_WAVES_MIN_K).
-constexpr int BK_FOUR_WAVES_MIN_K = 256;
+// (DIRECT_FOUR_WAVES_MIN_K of host/dispatch_rules.hpp).
 template <int INNER_OP, int INNER_POW>
 __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_four_waves(const BuildKernelArgs args)
 {

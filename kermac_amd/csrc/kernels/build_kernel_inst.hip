@@ -5,6 +5,7 @@
 
 #include "launch.hpp"
 #include "build_kernel.hpp"
+#include "../host/dispatch_rules.hpp"
 
 #ifndef KMC_INNER_OP
 #error "compile with -DKMC_INNER_OP=<0|1> -DKMC_INNER_POW=<0..4>"
@@ -22,7 +23,7 @@ static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStr
     // contiguous rows on both sides, a contraction long enough for the walk to set the time, and an inner term
     // without transcendentals (whose loop needs more registers): the variant compiled for four waves per SIMD
     if constexpr (LOAD_A == kmc::LOAD_COL_VEC && LOAD_B == kmc::LOAD_COL_VEC && KMC_INNER_POW != kmc::POW_POW) {
-        if (args.k >= kmc::BK_FOUR_WAVES_MIN_K && !args.repair_only)
+        if (args.k >= kmc_rules::DIRECT_FOUR_WAVES_MIN_K && !args.repair_only)
             return launch(kmc::build_kernel_four_waves<KMC_INNER_OP, KMC_INNER_POW>, grid, dim3(kmc::BK_THREADS), stream, args);
     }
     return launch(kmc::build_kernel<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);

@@ -76,6 +76,10 @@ _ROWS = (
     ("any other descriptor (fractional p, signed differences, …)", "always",
      "direct `build_kernel` (ahead of time for DIFF + NOOP/ABS/SQUARE/POW and DOT + NOOP, else compiled on first use); scalar p of 0.5, 1.5, 3, 4 on "
      "the exact-form variants"),
+    ("every direct launch",
+     "both operands with m / n contiguous and 16-byte aligned, K ≥ {DIRECT_FOUR_WAVES_MIN_K}, inner power not fractional, not a repair launch",
+     "`build_kernel_four_waves` (128 registers, four waves per SIMD; interior tiles copy their slices straight into LDS)"),
+    ("", "otherwise", "`build_kernel` (three waves per SIMD; interior tiles of such operands copy straight into LDS all the same)"),
     ("every direct launch, unbatched",
      "fewer than {build_a_kernel.CUT_BELOW_TILES} tiles of 128 × 128 (of one triangle for a set against itself), K ≥ {build_a_kernel.CUT_MIN_K}, and the "
      "launch-time model promises {cut_percent} % (ranges of ≥ {build_a_kernel.CUT_MIN_DEPTH} k)",
