@@ -142,12 +142,14 @@ enum kmc_flags {
      * The reference has no such path (include/build_a_kernel.cuh:339-370 is fp32 only). */
     KMC_FLAG_L1_FIXED = 512,
     /* The route through gram_workspace for squared differences first samples 16384 pairs (m, n) over
-     * the batch, from the pieces it has just made, and counts those below the trust threshold.  From
-     * 4 in 16384 on, nearly every 128 x 128 part of the result holds such a pair and would be
-     * recomputed by the direct kernel anyway (sets of near-duplicates, tight clusters far apart), so the
-     * matrix-core kernel then only stamps the parts and the call costs the direct kernel's time plus
-     * the split (at M = N = 30000, K = 1024: 32.5 ms instead of 6 + 32).  This flag leaves the sample
-     * out: every part is multiplied, checked and, if need be, recomputed. */
+     * the batch -- 16 from each of 1024 parts of 128 x 128 -- from the pieces it has just made, and counts
+     * those below the trust threshold and the sampled parts that show one.  From 4 in 16384 on, spread
+     * over the parts, nearly every part of the result holds such a pair and would be recomputed by the
+     * direct kernel anyway (sets of near-duplicates, tight clusters in any order), so the matrix-core
+     * kernel then only stamps the parts and the call costs the direct kernel's time plus the split (at
+     * M = N = 30000, K = 1024: 32.5 ms instead of 6 + 32).  Pairs packed into few parts (points stored
+     * cluster by cluster) leave the call on the matrix cores.  This flag leaves the sample out: every
+     * part is multiplied, checked and, if need be, recomputed. */
     KMC_FLAG_NO_PROBE = 1024
 };
 

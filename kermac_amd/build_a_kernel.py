@@ -743,6 +743,8 @@ def _attach_gram_workspace(params, device, switch="KERMAC_AMD_L2_WORKSPACE"):
     if workspace is None:
         return None             # no room for it, or the caller's limit: the one-step kernel needs none
     params.gram_workspace, params.gram_workspace_bytes = workspace.data_ptr(), needed
+    if os.environ.get("KERMAC_AMD_L2_PROBE", "1") in ("", "0"):
+        params.flags |= _backend.FLAG_NO_PROBE      # no sample of pairs in front of the product kernel
     return workspace
 
 

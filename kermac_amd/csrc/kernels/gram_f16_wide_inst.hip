@@ -34,7 +34,7 @@ struct WideLayout {
     int slices, slices_per_range, ranges;
     int tiles_m, tiles_n, tiles_n_padded;
     OperandRegions a, b;
-    int64_t probe;          // byte offset of the two counters of gram_probe_pairs
+    int64_t probe;          // byte offset of the three counters of gram_probe_pairs
     int64_t bytes;
 };
 
@@ -277,11 +277,11 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     if (!products && !(p->flags & KMC_FLAG_NO_PROBE) &&
         static_cast<int64_t>(layout.tiles_m) * layout.tiles_n * args.l * layout.slices >= kmc_rules::PROBE_MIN_TILES_TIMES_SLICES) {      // 0.5 ms and more: the sample is 10 us
         wide.probe = reinterpret_cast<unsigned *>(workspace + layout.probe);
-        wide.probe_pairs = kmc::GW_PROBE_PAIRS / args.l > 1024 ? kmc::GW_PROBE_PAIRS / args.l : 1024;
+        wide.probe_pairs = kmc::GW_PROBE_PAIRS / args.l > 1024 ? kmc::GW_PROBE_PAIRS / args.l / kmc::GW_PROBE_GROUP * kmc::GW_PROBE_GROUP : 1024;
         void *clear_args[] = {&wide.probe};
         status = hipLaunchKernel(reinterpret_cast<const void *>(kmc::gram_probe_clear<0>), dim3(1), dim3(64), clear_args, 0, stream);
         if (status != hipSuccess) return status;
-        status = launch(kmc::gram_probe_pairs<0>, dim3((wide.probe_pairs + 3) / 4, args.l), dim3(256), stream, wide);
+        status = launch(kmc::gram_probe_pairs<0>, dim3(wide.probe_pairs / kmc::GW_PROBE_GROUP, args.l), dim3(kmc::GW_PROBE_GROUP * 64), stream, wide);
         if (status != hipSuccess) return status;
     }
     if (args.symmetric) {

@@ -55,7 +55,7 @@ _ROWS = (
      "{WIDE_K_CONTIGUOUS_MIN_ROWS}",
      "`gram_row_stats` + `gram_f16_split` per operand, `gram_f16_wide` (fp16 pieces, 256 × 256 tiles), repair launch of the direct kernel; "
      "from tiles · slices ≥ {PROBE_MIN_TILES_TIMES_SLICES} on `gram_probe_pairs` first: {PROBE_BAIL_PER_16384} of {PROBE_PAIRS} sampled pairs "
-     "below the trust threshold send the whole call to the direct kernel"),
+     "below the trust threshold, spread over the sampled parts and not packed into few of them, send the whole call to the direct kernel"),
     ("",
      "K ≥ {build_a_kernel.AUTO_ONE_STEP_MIN_K} ({build_a_kernel.AUTO_ONE_STEP_MIN_K_ROWS_CONTIGUOUS} with the rows contiguous in both operands), trust < 1, "
      "and not (fewer than 128 tiles of 128 × 128 and a call the direct path would cut over k)",

@@ -272,10 +272,12 @@ def test_a_batch_of_panels_against_themselves_with_near_twins(device, wide):
     assert_close_to_truth(d_self, oracle.cdist(y.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30, what="near duplicates")
 
 
-def clustered(rows, middle, device, seed):
+def clustered(rows, middle, device, seed, cluster_by_cluster=False):
     """Every row one of the points `middle` plus noise of 1e-3: two rows of one cluster are near-duplicates."""
     g = torch.Generator().manual_seed(seed)
     which = torch.randint(0, middle.size(0), (rows,), generator=g)
+    if cluster_by_cluster:
+        which = which.sort().values
     return (middle[which] + 1e-3 * torch.randn(rows, middle.size(1), generator=g)).to(device)
 
 
@@ -306,6 +308,32 @@ def test_sets_of_near_duplicates_go_to_the_direct_kernel_whole(device):
         plain2 = kermac.cdist(a2, b2, p=2.0)
     assert not torch.equal(got2, plain2)
     assert_close_to_truth(got2[0][:512, :768], torch.cdist(a2[:512].double(), b2[:768].double(), p=2.0), rtol=1e-5, what="spread-out data")
+
+
+def test_near_duplicates_stored_cluster_by_cluster_stay_on_the_matrix_cores(device):
+    """The same 64 clusters with the points stored cluster by cluster: as many pairs are near-duplicates, but they fill
+    the blocks on the diagonal (one part in 64) instead of sitting in every part.  The sample tells the two apart by
+    the number of sampled parts that show such a pair, the matrix-core kernel does its work, and the repair launch
+    recomputes the blocks on the diagonal only: parts between different clusters carry the matrix cores' bits, parts
+    inside a cluster the direct kernel's, and everything keeps the tolerance."""
+    M, N, K = 8192, 8192, 1024
+    middle = 10.0 * torch.randn(64, K, generator=torch.Generator().manual_seed(4))
+    a = clustered(M, middle, device, 5, cluster_by_cluster=True)
+    b = clustered(N, middle, device, 6, cluster_by_cluster=True)
+    at, bt = a.t().contiguous().t(), b.t().contiguous().t()
+    assert kermac.get_l2_mode() == "auto"
+    got = kermac.cdist(at, bt, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        plain = kermac.cdist(at, bt, p=2.0)[0]
+    same = (got == plain)
+    # first cluster against first cluster: near-duplicates, recomputed by the direct kernel
+    assert same[:64, :64].all()
+    # first cluster against last: far apart, trusted, the matrix cores' own rounding
+    assert not same[:64, -64:].all()
+    assert 0.2 < (~same).float().mean().item()
+    rows = torch.cat([torch.arange(0, 384), torch.arange(M - 128, M)]).to(device)
+    truth = torch.cdist(a[rows].double(), b[:768].double(), p=2.0)
+    assert_close_to_truth(got[rows][:, :768], truth, rtol=1e-5, atol=1e-30, what="clusters stored one after the other")
 
 
 def test_the_kept_split_is_made_again_when_it_is_not_the_one_needed(device, wide):
