@@ -22,7 +22,7 @@
 // back and added to after the next 1024).
 //
 // Steps on the stream (host side: l1_fixed_inst.hip): clear the header, largest magnitude of a and of
-// b (l1_fixed_range), a sample of pairs that predicts whether the tiles will be trusted at all
+// b (l1_fixed_range), a sample of tiles that predicts what share of them will be trusted
 // (l1_fixed_sample), both operands to the grid in one layout -- rows contiguous, rows padded to 128
 // and k to 16 with the image of zero, so the walk has no edges and needs one loader
 // (l1_fixed_convert) -- the walk (l1_fixed_kernel), and the repair launch.
@@ -37,8 +37,28 @@ struct L1FixedHeader {
     unsigned max_bits;        // bits of the largest |x| in a and b (a NaN or an infinity compares above every number)
     unsigned sampled;         // pairs sampled
     unsigned sampled_below;   // of them, those below the trust threshold
-    unsigned unused[13];
+    unsigned sampled_tiles;         // 128 x 128 tiles they were sampled from
+    unsigned sampled_tiles_below;   // of them, those that showed such a pair
+    unsigned unused[11];
 };
+
+// What the sample says: true when the walk would be wasted.  A tile with one element below the threshold is
+// recomputed whole, and the walk takes 0.87 of the direct kernel's time, so the route pays while fewer than
+// one tile in eight is recomputed.  The share of such tiles is estimated two ways.  Pairs below the threshold
+// that are spread evenly (density d) sit in 1 - exp(-16384 d) of the tiles -- one such pair in 100000 is
+// already one tile in seven.  Pairs packed into few tiles (points stored cluster by cluster: the blocks on the
+// diagonal) sit in the share of sampled tiles that showed one.  Which it is tells the number of sampled tiles
+// with such a pair: spread evenly, `below` pairs land in tiles (1 - exp(-below / tiles)) different ones,
+// packed, in far fewer.
+__device__ __forceinline__ bool l1_fixed_left_to_the_direct_kernel(const L1FixedHeader &header)
+{
+    if (header.sampled_below == 0u) return false;
+    const float pairs = (float)header.sampled, below = (float)header.sampled_below;
+    const float tiles = (float)header.sampled_tiles, tiles_below = (float)header.sampled_tiles_below;
+    const bool spread = tiles_below >= 0.7f * tiles * (1.0f - __expf(-below / tiles));
+    const float share = spread ? 1.0f - __expf(-(float)(BK_TILE_M * BK_TILE_N) * below / pairs) : tiles_below / tiles;
+    return share > 0.125f;
+}
 
 // The grid of one batch entry, derived from the header by every kernel that needs it.
 struct L1FixedGrid {
@@ -85,7 +105,7 @@ struct L1FixedArgs {
     int bits;
     int k_padded;
     float tolerance;              // relative error a trusted element may carry
-    int sample_pairs;
+    int sample_tiles;             // per batch entry
 };
 
 constexpr int L1F_THREADS = 256;
@@ -135,31 +155,64 @@ __device__ __forceinline__ float l1_fixed_element(const L1FixedPanel &panel, int
     return panel.majorness == 0 ? x[(i64)kk * panel.ld + row] : x[(i64)row * panel.ld + kk];
 }
 
-// A sample of (m, n) pairs, one wave each, summed in fp32: how many of them would not be trusted.  The walk
-// looks at the count before it does anything: when more than one pair in 64 falls below the threshold, nearly
-// every 128 x 128 tile holds such a pair and would be recomputed anyway, so the walk only stamps the tiles.
+// A sample of the result, summed in fp32 from the operands as the caller holds them: how much of it would not be
+// trusted.  A workgroup takes one 128 x 128 tile (blockIdx.x counts the sampled tiles of a batch entry,
+// blockIdx.y the batch entries), 16 consecutive rows of a and 16 of b from it, and a lane sums one of their 256
+// pairs over all of k; the rows pass through LDS in chunks of 128 k, loaded along whichever direction is
+// contiguous.  The conversion and the walk look at the counts before they do anything.
+constexpr int L1F_SAMPLE_ROWS = 16;
+constexpr int L1F_SAMPLE_CHUNK = 128;
 __global__ __launch_bounds__(L1F_THREADS) void l1_fixed_sample(const L1FixedArgs args)
 {
+    __shared__ float rows_a[L1F_SAMPLE_CHUNK][L1F_SAMPLE_ROWS + 1];      // + 1: no bank is hit twice whichever way the rows are loaded
+    __shared__ float rows_b[L1F_SAMPLE_CHUNK][L1F_SAMPLE_ROWS + 1];
+    __shared__ unsigned below_in_tile;
     const int batch = blockIdx.y;
-    const int lane = threadIdx.x & 63;
-    const int pair = blockIdx.x * (L1F_THREADS / 64) + (threadIdx.x >> 6);
-    if (pair >= args.sample_pairs) return;
+    const int t = threadIdx.x;
     const L1FixedGrid grid = l1_fixed_grid(args.header[batch].max_bits, args.bits);
     if (!grid.usable) return;
-    unsigned h = (unsigned)pair * 2654435761u + 0x9e3779b9u * (unsigned)(batch + 1);
+    if (t == 0) below_in_tile = 0u;
+    unsigned h = (unsigned)blockIdx.x * 2654435761u + 0x9e3779b9u * (unsigned)(batch + 1);
     h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 13;
-    const int m = (int)(h % (unsigned)args.kernel.m);
+    const int m0 = (int)(h % (unsigned)((args.kernel.m + BK_TILE_M - 1) / BK_TILE_M)) * BK_TILE_M + (int)((h >> 20) & 7u) * L1F_SAMPLE_ROWS;
     h = h * 0x7feb352du + 0x1234567u; h ^= h >> 16;
-    const int n = (int)(h % (unsigned)args.kernel.n);
+    const int n0 = (int)(h % (unsigned)((args.kernel.n + BK_TILE_N - 1) / BK_TILE_N)) * BK_TILE_N + (int)((h >> 20) & 7u) * L1F_SAMPLE_ROWS;
+    // rows beyond the panel repeat its last row: a pair counted twice biases nothing that matters here
+    const int row_a = args.a.majorness == 0 ? t % L1F_SAMPLE_ROWS : t / L1F_SAMPLE_ROWS;
+    const int k_a = args.a.majorness == 0 ? t / L1F_SAMPLE_ROWS : t % L1F_SAMPLE_ROWS;
+    const int row_b = args.b.majorness == 0 ? t % L1F_SAMPLE_ROWS : t / L1F_SAMPLE_ROWS;
+    const int k_b = args.b.majorness == 0 ? t / L1F_SAMPLE_ROWS : t % L1F_SAMPLE_ROWS;
+    const int m = min(m0 + row_a, args.kernel.m - 1), n = min(n0 + row_b, args.kernel.n - 1);
+    const int i = t % L1F_SAMPLE_ROWS, j = t / L1F_SAMPLE_ROWS;      // this lane's pair: row i of a, row j of b
     float sum = 0.0f;
-    for (int kk = lane; kk < args.kernel.k; kk += 64)
-        sum += __builtin_fabsf(l1_fixed_element(args.b, batch, n, kk) - l1_fixed_element(args.a, batch, m, kk));
+    for (int k0 = 0; k0 < args.kernel.k; k0 += L1F_SAMPLE_CHUNK) {
+        float va[L1F_SAMPLE_CHUNK / 16], vb[L1F_SAMPLE_CHUNK / 16];
 #pragma unroll
-    for (int offset = 32; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
-    if (lane == 0) {
-        const float threshold = (float)args.kernel.k / args.tolerance * grid.inv_scale;
-        atomicAdd(&args.header[batch].sampled, 1u);
-        if (!(sum >= threshold)) atomicAdd(&args.header[batch].sampled_below, 1u);
+        for (int u = 0; u < L1F_SAMPLE_CHUNK / 16; u++) {
+            const int ka = k0 + k_a + 16 * u, kb = k0 + k_b + 16 * u;
+            va[u] = ka < args.kernel.k ? l1_fixed_element(args.a, batch, m, ka) : 0.0f;
+            vb[u] = kb < args.kernel.k ? l1_fixed_element(args.b, batch, n, kb) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < L1F_SAMPLE_CHUNK / 16; u++) {
+            rows_a[k_a + 16 * u][row_a] = va[u];
+            rows_b[k_b + 16 * u][row_b] = vb[u];
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int q = 0; q < L1F_SAMPLE_CHUNK; q++) sum += __builtin_fabsf(rows_b[q][j] - rows_a[q][i]);
+    }
+    const float threshold = (float)args.kernel.k / args.tolerance * grid.inv_scale;
+    if (!(sum >= threshold)) atomicAdd(&below_in_tile, 1u);
+    __syncthreads();
+    if (t == 0) {
+        atomicAdd(&args.header[batch].sampled, (unsigned)L1F_THREADS);
+        atomicAdd(&args.header[batch].sampled_tiles, 1u);
+        if (below_in_tile > 0u) {
+            atomicAdd(&args.header[batch].sampled_below, below_in_tile);
+            atomicAdd(&args.header[batch].sampled_tiles_below, 1u);
+        }
     }
 }
 
@@ -177,6 +230,7 @@ __global__ __launch_bounds__(L1F_THREADS) void l1_fixed_convert(const L1FixedPan
 {
     __shared__ float block[64][65];
     const int batch = blockIdx.z;
+    if (l1_fixed_left_to_the_direct_kernel(header[batch])) return;       // the walk will not read the image
     const L1FixedGrid grid = l1_fixed_grid(header[batch].max_bits, bits);
     const int row0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
     const int fast = threadIdx.x & 63, slow = threadIdx.x >> 6;       // 64 x 4 lanes
@@ -246,8 +300,8 @@ __global__ __launch_bounds__(BK_THREADS, L1F_MIN_WAVES) void l1_fixed_kernel(con
 
     const L1FixedHeader header = fixed.header[batch];
     const L1FixedGrid grid = l1_fixed_grid(header.max_bits, fixed.bits);
-    if (!grid.usable || header.sampled_below * 64u > header.sampled) {
-        // nothing here would be trusted: leave the whole tile to the repair launch
+    if (!grid.usable || l1_fixed_left_to_the_direct_kernel(header)) {
+        // nothing here would be trusted, or too little to pay for the walk: leave the whole tile to the repair launch
         if (tid == 0) c_tile[(i64)n0 * args.c_ld + m0] = __uint_as_float(BK_REPAIR_MARKER);
         return;
     }

@@ -12,7 +12,7 @@ namespace kmc_host {
 namespace {
 
 constexpr int64_t REGION_ALIGN = 256;
-constexpr int SAMPLE_PAIRS = 1024;
+constexpr int SAMPLE_TILES = 1024;      // over the batch, 256 pairs each; at least 64 per batch entry
 
 // Whether the route pays: it adds seven small launches and two passes over the operands (about
 // 16 bytes per operand element) to a walk that takes 0.85 of the direct kernel's time, so it needs
@@ -109,7 +109,7 @@ hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKer
     fixed.bits = layout.bits;
     fixed.k_padded = layout.k_padded;
     fixed.tolerance = p->gram_trust > 0.0f && p->gram_trust < 1.0f ? p->gram_trust : 8e-6f;
-    fixed.sample_pairs = SAMPLE_PAIRS;
+    fixed.sample_tiles = SAMPLE_TILES / args.l > 64 ? SAMPLE_TILES / args.l : 64;
 
     void *clear_args[] = {&fixed.header, const_cast<int *>(&args.l)};
     hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(kmc::l1_fixed_clear), dim3((args.l * 16 + kmc::L1F_THREADS - 1) / kmc::L1F_THREADS),
@@ -124,7 +124,7 @@ hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKer
                             dim3(kmc::L1F_THREADS), range_args, 0, stream);
         if (e != hipSuccess) return e;
     }
-    e = launch(kmc::l1_fixed_sample, dim3((SAMPLE_PAIRS + 3) / 4, args.l), dim3(kmc::L1F_THREADS), stream, fixed);
+    e = launch(kmc::l1_fixed_sample, dim3(fixed.sample_tiles, args.l), dim3(kmc::L1F_THREADS), stream, fixed);
     if (e != hipSuccess) return e;
     for (int side = 0; side < (layout.same_panel ? 1 : 2); side++) {
         kmc::L1FixedPanel &panel = side == 0 ? fixed.a : fixed.b;
