@@ -698,9 +698,16 @@ __device__ __forceinline__ void build_kernel_tile(const BuildKernelArgs &args, f
             acc, load_a, load_b, lds_a, lds_b, k_here, m_valid, n_valid, p_inner, args.diff_sign, tx, ty);
     }
 
-    finish_tile(acc, args, batch, m0, n0, tx, ty);
+    // What the epilogue derives from the lane's position is derived here, from a copy of the lane id that the
+    // compiler cannot see through: otherwise it computes store addresses before the walk and, in the variant
+    // held to 128 registers, parks them in scratch memory for the walk's duration.
+    int tid_after = tid;
+    asm volatile("" : "+v"(tid_after));
+    const int tx_after = tid_after & 15, ty_after = tid_after >> 4;
 
-    store_tile(acc, args, batch, tile_m, tile_n, m0, n0, m_valid, n_valid, tx, ty, tid, lds_a, lds_b, false);
+    finish_tile(acc, args, batch, m0, n0, tx_after, ty_after);
+
+    store_tile(acc, args, batch, tile_m, tile_n, m0, n0, m_valid, n_valid, tx_after, ty_after, tid_after, lds_a, lds_b, false);
 }
 
 template <int INNER_OP, int INNER_POW, int LOAD_A, int LOAD_B>

@@ -353,22 +353,28 @@ __global__ __launch_bounds__(BK_THREADS, L1F_MIN_WAVES) void l1_fixed_kernel(con
     for (int j = 0; j < 8; j++)
 #pragma unroll
         for (int i = 0; i < 8; i++) result[j][i] = __uint_as_float(acc[j][i]);
+    // What the epilogue derives from the lane's position is derived here, from a copy of the lane id that the
+    // compiler cannot see through: otherwise it computes the store addresses before the walk and parks them in
+    // scratch memory for its duration (27 dwords per lane, written and read back by every tile).
+    int tid_after = tid;
+    asm volatile("" : "+v"(tid_after));
+    const int tx_after = tid_after & 15, ty_after = tid_after >> 4;
 
     // Trust: an element is off by at most K grid steps.
     const float threshold = (float)args.k / fixed.tolerance * grid.inv_scale;
     int distrust = 0;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        const int n_local = ty * 4 + (j & 3) + (j >> 2) * 64;
+        const int n_local = ty_after * 4 + (j & 3) + (j >> 2) * 64;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const int m_local = tx * 4 + (i & 3) + (i >> 2) * 64;
+            const int m_local = tx_after * 4 + (i & 3) + (i >> 2) * 64;
             if (n_local < n_valid && m_local < m_valid && !(result[j][i] >= threshold)) distrust = 1;
         }
     }
     const bool distrusted = __syncthreads_or(distrust) != 0;
-    finish_tile(result, args, batch, m0, n0, tx, ty);
-    store_tile(result, args, batch, tile_m, tile_n, m0, n0, m_valid, n_valid, tx, ty, tid, lds_a, lds_b, distrusted);
+    finish_tile(result, args, batch, m0, n0, tx_after, ty_after);
+    store_tile(result, args, batch, tile_m, tile_n, m0, n0, m_valid, n_valid, tx_after, ty_after, tid_after, lds_a, lds_b, distrusted);
 }
 
 }  // namespace kmc
