@@ -141,15 +141,16 @@ enum kmc_flags {
      * query reports 0 for, the direct kernel runs.  Not with k_total.
      * The reference has no such path (include/build_a_kernel.cuh:339-370 is fp32 only). */
     KMC_FLAG_L1_FIXED = 512,
-    /* The route through gram_workspace for squared differences first samples 16384 pairs (m, n) over
-     * the batch -- 16 from each of 1024 parts of 128 x 128 -- from the pieces it has just made, and counts
-     * those below the trust threshold and the sampled parts that show one.  From 4 in 16384 on, spread
-     * over the parts, nearly every part of the result holds such a pair and would be recomputed by the
-     * direct kernel anyway (sets of near-duplicates, tight clusters in any order), so the matrix-core
-     * kernel then only stamps the parts and the call costs the direct kernel's time plus the split (at
-     * M = N = 30000, K = 1024: 32.5 ms instead of 6 + 32).  Pairs packed into few parts (points stored
-     * cluster by cluster) leave the call on the matrix cores.  This flag leaves the sample out: every
-     * part is multiplied, checked and, if need be, recomputed. */
+    /* Matrix-core launches for squared differences that are given a workspace first take a sample of
+     * the result from the operands (one small launch): 256 tiles of 128 x 128 over the batch, 256
+     * pairs (m, n) of each, judged by the trust rule on up to 128 of the k.  Pairs below the
+     * threshold that are spread over the sampled tiles mean that nearly every part of the result
+     * holds such a pair and would be recomputed by the direct kernel anyway (sets of near-duplicates,
+     * tight clusters in any order): from 2 in 16384 on, the matrix-core kernel only stamps its parts
+     * and the call costs the direct kernel's time plus little (at M = N = 30000, K = 1024: 32.5 ms
+     * instead of 6 + 32; at 2048 x 2048 x 1024 0.19 instead of 0.37 ms).  Pairs packed into few tiles
+     * (points stored cluster by cluster) leave the call on the matrix cores.  This flag leaves the
+     * sample out: every part is multiplied, checked and, if need be, recomputed. */
     KMC_FLAG_NO_PROBE = 1024
 };
 
@@ -215,7 +216,11 @@ typedef struct kmc_build_kernel_params {
      * then 256 x 256 tiles on the fp16 matrix instruction; same trust rule, same repair launch,
      * same tolerance: at M = N = 30000, K = 1024 6.1 ms instead of 10).  NULL, too small, or a
      * problem for which kmc_gram_workspace_bytes reports 0: the one-step kernel runs.  The
-     * contents after the call do not matter; calls that share a workspace must be ordered. */
+     * contents after the call do not matter; calls that share a workspace must be ordered.
+     * With KMC_FLAG_L2_GRAM or KMC_FLAG_L2_GRAM_BF16 on a problem that runs a one-step kernel, a
+     * workspace of at least KMC_SAMPLE_BYTES lets the library look before it multiplies (see
+     * KMC_FLAG_NO_PROBE); kmc_gram_workspace_bytes does not ask for it, a caller who wants the
+     * sample for every size hands over max(KMC_SAMPLE_BYTES, what the query reports). */
     void *gram_workspace;
     int64_t gram_workspace_bytes;
 } kmc_build_kernel_params;
@@ -286,6 +291,11 @@ int kmc_sample_mean(const float *x, int32_t majorness, int32_t rows, int32_t k, 
  * before capturing calls into a HIP graph.  The stream must belong to the current device.
  */
 #define KMC_STATIC_SCRATCH_BYTES (64u << 20)
+
+/* What the sample in front of a matrix-core launch for squared differences takes of gram_workspace
+ * (KMC_FLAG_NO_PROBE); the route through the workspace counts it in what kmc_gram_workspace_bytes
+ * reports, the one-step kernels use it when the caller hands it over. */
+#define KMC_SAMPLE_BYTES 1024
 int kmc_build_kernel_cut_static(const kmc_build_kernel_params *params, int32_t ranges, void *stream);
 
 /*

@@ -44,6 +44,7 @@ FLAG_DOT_PIECES = 128
 FLAG_GRAM_WORKSPACE_ANY_SIZE = 256
 FLAG_L1_FIXED = 512
 FLAG_NO_PROBE = 1024
+SAMPLE_BYTES = 1024             # KMC_SAMPLE_BYTES: what the sample in front of a matrix-core launch takes of the workspace
 
 _float_p = c_void_p  # device pointers are passed as integers
 

@@ -729,6 +729,14 @@ def _workspace_route_applies(params, flags):
         params.flags = kept
 
 
+# The sample that the library takes in front of a one-step matrix-core kernel when it is handed KMC_SAMPLE_BYTES of
+# workspace is one more launch, 5 to 8 us on the stream.  On data whose near-duplicates sit in every tile it saves the
+# matrix cores' work (4096 x 4096 x 512: 441 -> 362 us where the direct kernel takes 319; 2048 x 2048 x 1024 374 -> 300
+# against 193, the repair launch being the direct kernel uncut), on every other call it is a tax: 38 -> 46 us at
+# 1024 x 1024 x 256.  From 4e9 terms on the tax is below a tenth.
+_L2_SAMPLE_MIN_TERMS = 4_000_000_000
+
+
 def _attach_gram_workspace(params, device, switch="KERMAC_AMD_L2_WORKSPACE"):
     """Large squared-difference problems in the split-bf16 mode go through a workspace (include/
     kermac_amd.h, gram_workspace: both operands split once into fp16 pieces, then 256 x 256 tiles);
@@ -736,15 +744,18 @@ def _attach_gram_workspace(params, device, switch="KERMAC_AMD_L2_WORKSPACE"):
     KERMAC_AMD_L2_WORKSPACE=0 keeps every call on the one-step kernel."""
     if os.environ.get(switch, "1") in ("", "0"):
         return None
+    if os.environ.get("KERMAC_AMD_L2_PROBE", "1") in ("", "0"):
+        params.flags |= _backend.FLAG_NO_PROBE      # no sample of the result in front of the matrix-core kernel
     needed = _backend.gram_workspace_bytes(params)
+    if (needed == 0 and (params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16)) and not (params.flags & _backend.FLAG_NO_PROBE)
+            and params.m * params.n * params.k * params.l >= _L2_SAMPLE_MIN_TERMS):
+        needed = _backend.SAMPLE_BYTES              # a one-step kernel: room for the sample that is taken in front of it
     if needed == 0:
         return None
     workspace = _scratch.allocate(needed, device)
     if workspace is None:
         return None             # no room for it, or the caller's limit: the one-step kernel needs none
     params.gram_workspace, params.gram_workspace_bytes = workspace.data_ptr(), needed
-    if os.environ.get("KERMAC_AMD_L2_PROBE", "1") in ("", "0"):
-        params.flags |= _backend.FLAG_NO_PROBE      # no sample of pairs in front of the product kernel
     return workspace
 
 

@@ -109,6 +109,7 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
     args->k_total = p->k_total;
     args->centre = nullptr;
     args->centre_bs = 0;
+    args->sample = nullptr;
     if ((p->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16)) && p->gram_centre) {
         if (!aligned16(p->gram_centre) || p->gram_centre_bs % 4 != 0 || p->gram_centre_bs < 0)
             return fail(KMC_ERR_INVALID_ARGUMENT, "gram_centre must be 16-byte aligned with a batch stride that is a multiple of 4");
@@ -144,6 +145,7 @@ hipError_t launch_gram_l2(int load_a, int load_b, const kmc::BuildKernelArgs &ar
 hipError_t launch_gram_bf16_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
 int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
 hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
+hipError_t launch_gram_probe(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, unsigned *sample, hipStream_t stream);
 int64_t l1_fixed_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
 hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
 hipError_t launch_finish_partials(const kmc::BuildKernelArgs &kernel, const float *partials, int64_t partial_ld,
@@ -235,6 +237,15 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
         hipError_t g = launch_gram_f16_wide(params, args, static_cast<hipStream_t>(stream), &wide);
         if (g != hipSuccess) return fail_hip(g, "gram_f16_wide launches");
         if (!wide) {
+            // The one-step kernels: with KMC_SAMPLE_BYTES of workspace, a sample of the result first (gram_probe.hip),
+            // so that data whose near-duplicates sit in every tile costs the direct kernel's time, not both.
+            if (!(params->flags & KMC_FLAG_NO_PROBE) && params->gram_workspace && params->gram_workspace_bytes >= KMC_SAMPLE_BYTES &&
+                (reinterpret_cast<uintptr_t>(params->gram_workspace) & 255) == 0 && args.k > 0) {
+                unsigned *sample = static_cast<unsigned *>(params->gram_workspace);
+                g = launch_gram_probe(params, args, sample, static_cast<hipStream_t>(stream));
+                if (g != hipSuccess) return fail_hip(g, "gram_probe_operands launch");
+                args.sample = sample;
+            }
             g = (params->flags & KMC_FLAG_L2_GRAM_BF16)
                     ? launch_gram_bf16_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream))
                     : launch_gram_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));

@@ -29,10 +29,9 @@
     X(DOT_LONG_MIN_TILES_BATCHED, 32)                                                                   \
     X(DOT_LONG_MIN_TILES_SINGLE, 64)                                                                    \
     X(DOT_LONG_MIN_TILES_TIMES_K, 24576)                                                                \
-    /* the sample of pairs in front of the squared-difference product kernel */                         \
-    X(PROBE_MIN_TILES_TIMES_SLICES, 65536)                                                              \
-    X(PROBE_PAIRS, 16384)                                                                               \
-    X(PROBE_BAIL_PER_16384, 4)                                                                          \
+    /* the sample of the result in front of the matrix-core kernels for squared differences */           \
+    X(SAMPLE_TILES, 256)                   /* of 128 x 128, 256 pairs each */                           \
+    X(SAMPLE_LEAVE_PER_16384, 2)           /* pairs below the trust threshold, spread over the tiles */ \
     /* the direct kernel compiled for four waves per SIMD (k-major panels, no fractional power) */       \
     X(DIRECT_FOUR_WAVES_MIN_K, 256)                                                                     \
     /* absolute differences on fixed point (KMC_FLAG_L1_FIXED): tiles of 128 x 128 over the batch */    \

@@ -55,9 +55,45 @@ struct BuildKernelArgs {
     // GRAM_CENTRE_PAD floats, 16-byte aligned) that is subtracted from both operands while they are
     // staged; null: nothing is subtracted.
     const float *centre; i64 centre_bs;
+    // Matrix-core kernels for squared differences only, or null: what a sample of the result said before the
+    // launch (gram_probe.hip fills it, sample_leaves_it_to_the_direct_kernel reads it).
+    const unsigned *sample;
 };
 
 constexpr int GRAM_CENTRE_PAD = 64;
+
+// The sample taken in front of a matrix-core launch for squared differences: BK_SAMPLE_TILES tiles of 128 x 128
+// of the result, 16 rows of each operand from each, their 256 pairs.  One word per sampled tile: pairs below
+// the trust threshold in the low half, 1 in the high half when there are any.
+constexpr int BK_SAMPLE_TILES = 256;
+constexpr int BK_SAMPLE_ROWS = 16;
+constexpr int BK_SAMPLE_BYTES = BK_SAMPLE_TILES * 4;
+constexpr int BK_SAMPLE_LEAVE_PER_16384 = 2;     // pairs below the threshold, spread over the tiles: leave the call to the direct kernel
+
+// What the sample says: true when the matrix cores' work would be thrown away.  A 128 x 128 part with one pair
+// below the trust threshold is recomputed whole by the repair launch, so pairs below the threshold cost the
+// matrix cores' work when they sit in (nearly) every part: 2 such pairs in 16384, spread evenly, already put one
+// into six parts of seven.  The same share of pairs packed into few parts -- points stored cluster by cluster,
+// whose near-duplicates fill the blocks on the diagonal -- costs the repair of those parts only.  The two are
+// told apart by the number of sampled tiles that show such a pair: spread evenly over the sampled tiles, `below`
+// pairs land in tiles (1 - exp(-below / tiles)) different ones; packed, in far fewer.
+// Every lane of a wave calls it; the answer is the same for every wave of the launch.
+__device__ __forceinline__ bool sample_leaves_it_to_the_direct_kernel(const unsigned *sample)
+{
+    static_assert(BK_SAMPLE_TILES == 256, "a lane reads four words");
+    const uint4 words = reinterpret_cast<const uint4 *>(sample)[threadIdx.x & 63];
+    unsigned below = (words.x & 0xffffu) + (words.y & 0xffffu) + (words.z & 0xffffu) + (words.w & 0xffffu);
+    unsigned tiles_below = (words.x >> 16) + (words.y >> 16) + (words.z >> 16) + (words.w >> 16);
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        below += (unsigned)__shfl_xor((int)below, offset);
+        tiles_below += (unsigned)__shfl_xor((int)tiles_below, offset);
+    }
+    const float pairs = (float)(BK_SAMPLE_TILES * BK_SAMPLE_ROWS * BK_SAMPLE_ROWS);
+    if ((float)below * 16384.0f < (float)BK_SAMPLE_LEAVE_PER_16384 * pairs) return false;
+    const float spread = (float)BK_SAMPLE_TILES * (1.0f - __expf(-(float)below / (float)BK_SAMPLE_TILES));
+    return (float)tiles_below >= 0.7f * spread;
+}
 
 constexpr int BK_TILE_M = 128;
 constexpr int BK_TILE_N = 128;

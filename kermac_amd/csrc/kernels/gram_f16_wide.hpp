@@ -95,32 +95,7 @@ struct GramWideArgs {
     const float *gradient_g; i64 gradient_g_ld, gradient_g_bs;
     const float *gradient_shift; i64 gradient_shift_bs;
     int gradient_n;
-    // GW_EPILOGUE_DISTANCE only, or null: three counters that gram_probe_pairs fills before the product
-    // kernel starts -- pairs sampled, those of them below the trust threshold, and sampled 128 x 128
-    // parts that hold such a pair (probe_leaves_it_to_the_direct_kernel reads them).
-    unsigned *probe;
-    int probe_pairs;        // per batch entry, a multiple of GW_PROBE_GROUP
 };
-
-constexpr int GW_PROBE_PAIRS = 16384;
-constexpr int GW_PROBE_GROUP = 16;          // pairs sampled from one 128 x 128 part of the result
-constexpr int GW_PROBE_SLICES = 32;         // of each sampled pair, this many 16-deep slices spread over K
-constexpr unsigned GW_PROBE_BAIL = 4;       // per GW_PROBE_PAIRS
-
-// What the sample says.  Pairs below the trust threshold cost the product kernel's work only when they sit
-// in (nearly) every 128 x 128 part: 4 such pairs in 16384, spread evenly, already mean one per part on average.
-// The same share of pairs packed into few parts -- points stored cluster by cluster, whose near-duplicates
-// fill the blocks on the diagonal -- costs the repair of those parts only (64 clusters at 30000 x 30000 x 1024:
-// 6.1 ms, where the direct kernel takes 29).  The two are told apart by the number of sampled parts that
-// show such a pair: spread evenly over `groups` parts, `below` pairs land in groups (1 - exp(-below / groups))
-// different ones; packed, in far fewer.
-__device__ __forceinline__ bool probe_leaves_it_to_the_direct_kernel(const unsigned *probe)
-{
-    const float pairs = (float)probe[0], below = (float)probe[1], parts = (float)probe[2];
-    if (below == 0.0f || below * (float)GW_PROBE_PAIRS < (float)GW_PROBE_BAIL * pairs) return false;
-    const float groups = pairs / (float)GW_PROBE_GROUP;
-    return parts >= 0.7f * groups * (1.0f - __expf(-below / groups));
-}
 
 constexpr int GW_MAX_RANGES = 9;      // ranges of K per row: ceil(slices / 8) up to 71 slices, 8 beyond
 
@@ -250,68 +225,6 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsA
     }
 }
 
-template <int UNUSED = 0>
-__global__ void gram_probe_clear(unsigned *probe)
-{
-    if (threadIdx.x < 3) probe[threadIdx.x] = 0u;
-}
-
-// Would the product kernel's results be trusted?  A workgroup samples one 128 x 128 part of the result
-// (blockIdx.x counts the sampled parts of a batch entry, blockIdx.y the batch entries), one wave per pair
-// (m, n) of it: squared distance and norms over up to GW_PROBE_SLICES slices spread over K, from the first
-// fp16 piece of every value (2^-11 of the row's largest magnitude: ample for a threshold that is a quarter
-// of the norms or more).  The criterion is that of the product kernel on these k alone; near-duplicate
-// points fail it on any subset of k.  The counters are per launch.
-template <int UNUSED = 0>
-__global__ __launch_bounds__(GW_PROBE_GROUP * 64) void gram_probe_pairs(const GramWideArgs args)
-{
-    __shared__ unsigned below_in_part;
-    const int batch = blockIdx.y;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    if (threadIdx.x == 0) below_in_part = 0u;
-    __syncthreads();
-    unsigned h = (unsigned)blockIdx.x * 2654435761u + 0x9e3779b9u * (unsigned)(batch + 1);
-    h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 13;
-    const int m0 = (int)(h % (unsigned)((args.kernel.m + 127) / 128)) * 128;
-    h = h * 0x7feb352du + 0x1234567u; h ^= h >> 16;
-    const int n0 = (int)(h % (unsigned)((args.kernel.n + 127) / 128)) * 128;
-    h = (h + (unsigned)wave) * 0x9e3779b1u; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 13;
-    const int m = m0 + (int)((h & 0xffffu) % (unsigned)min(128, args.kernel.m - m0));
-    const int n = n0 + (int)((h >> 16) % (unsigned)min(128, args.kernel.n - n0));
-    // lane = 2 * (sampled slice) + half
-    const int sampled = min(args.slices, GW_PROBE_SLICES);
-    const int s = lane >> 1, half = lane & 1;
-    float d2 = 0.0f, norms = 0.0f;
-    if (s < sampled) {
-        const int slice = (int)((long long)s * args.slices / sampled);
-        const gram_chunk ca = args.pieces_a[batch * args.pieces_a_bs + ((i64)slice * GW_SEGMENTS + half) * args.rows_pad_a + m];
-        const gram_chunk cb = args.pieces_b[batch * args.pieces_b_bs + ((i64)slice * GW_SEGMENTS + half) * args.rows_pad_b + n];
-        const float ua = args.unscale_a[batch * args.unscale_a_bs + m], ub = args.unscale_b[batch * args.unscale_b_bs + n];
-        const gram_half8 ha = __builtin_bit_cast(gram_half8, ca), hb = __builtin_bit_cast(gram_half8, cb);
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const float a = (float)ha[e] * ua, b = (float)hb[e] * ub;
-            d2 += (b - a) * (b - a);
-            norms += a * a + b * b;
-        }
-    }
-#pragma unroll
-    for (int offset = 32; offset > 0; offset >>= 1) {
-        d2 += __shfl_xor(d2, offset);
-        norms += __shfl_xor(norms, offset);
-    }
-    if (lane == 0 && !(d2 >= args.kernel.gram_trust * norms)) atomicAdd(&below_in_part, 1u);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        atomicAdd(&args.probe[0], (unsigned)GW_PROBE_GROUP);
-        if (below_in_part > 0u) {
-            atomicAdd(&args.probe[1], below_in_part);
-            atomicAdd(&args.probe[2], 1u);
-        }
-    }
-}
-
 // Workgroup -> tile, as tile_of_workgroup of build_kernel.hpp with bands of GW_BAND_N tiles: a
 // CU holds one workgroup, so the 32 of an XCD cover 4 n tiles x 8 m tiles of a band at a time.
 // SYMMETRIC (a panel against itself): the ids count through the tiles on and below the diagonal,
@@ -388,9 +301,9 @@ __global__ __launch_bounds__(GW_THREADS) void gram_f16_wide(const GramWideArgs a
     const int n_valid = args.kernel.n - n0;
 
     if constexpr (EPILOGUE == GW_EPILOGUE_DISTANCE) {
-        // The sample of pairs says that the repair launch would redo (nearly) every part: stamp them all
-        // and leave (the branch is uniform over the launch: every workgroup reads the same three counters).  Parts above the diagonal of a symmetric result belong to nobody.
-        if (args.probe && probe_leaves_it_to_the_direct_kernel(args.probe)) {
+        // The sample of the result says that the repair launch would redo (nearly) every part: stamp them all
+        // and leave (the branch is uniform over the launch: every workgroup reads the same words).  Parts above the diagonal of a symmetric result belong to nobody.
+        if (args.kernel.sample && sample_leaves_it_to_the_direct_kernel(args.kernel.sample)) {
             if (tid < 4) {
                 const int part_m = tid & 1, part_n = tid >> 1;
                 const bool above = SYMMETRIC && tile_m == tile_n && part_m < part_n;

@@ -20,8 +20,6 @@ namespace kmc_host {
 namespace {
 
 constexpr int64_t REGION_ALIGN = 256;
-static_assert(kmc::GW_PROBE_PAIRS == kmc_rules::PROBE_PAIRS && kmc::GW_PROBE_BAIL == kmc_rules::PROBE_BAIL_PER_16384,
-              "the device constants of the sample of pairs are those of the table of rules");
 
 struct OperandRegions {
     int rows_pad, batches;
@@ -34,7 +32,7 @@ struct WideLayout {
     int slices, slices_per_range, ranges;
     int tiles_m, tiles_n, tiles_n_padded;
     OperandRegions a, b;
-    int64_t probe;          // byte offset of the three counters of gram_probe_pairs
+    int64_t sample;         // byte offset of the words of gram_probe_operands
     int64_t bytes;
 };
 
@@ -124,7 +122,7 @@ bool place_wide(int m, int n, int k, int l, bool a_once, bool b_once, bool symme
     place_operand(layout->a, m, a_once, l, *layout, cursor);
     if (symmetric) layout->b = layout->a;      // one panel, split once
     else place_operand(layout->b, n, b_once, l, *layout, cursor);
-    layout->probe = place(cursor, 256);
+    layout->sample = place(cursor, kmc::BK_SAMPLE_BYTES);
     layout->bytes = cursor;
     return true;
 }
@@ -214,6 +212,8 @@ void forget_split_in(const void *workspace)
 }
 
 // Statistics and split of one operand (also used by the gradient's fp16 route).
+hipError_t launch_gram_probe(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, unsigned *sample, hipStream_t stream);   // gram_probe.hip
+
 hipError_t launch_gram_rows(const kmc::GramRowsArgs &rows_of, int batches, hipStream_t stream)
 {
     const dim3 grid(rows_of.rows_pad / kmc::GW_ROW_THREADS, rows_of.ranges, batches);
@@ -271,18 +271,14 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     wide.slices = layout.slices; wide.ranges = layout.ranges;
     wide.wide_tiles_m = layout.tiles_m; wide.wide_tiles_n = layout.tiles_n; wide.wide_tiles_n_padded = layout.tiles_n_padded;
     const bool products = p->inner_operator == KMC_OP_DOT;
-    // Squared differences of problems whose walk is long against a launch: a sample of pairs first, so
-    // that data the trust rule would reject wholesale (sets of near-duplicates) costs the direct
-    // kernel's time and little more, instead of both.  KMC_FLAG_NO_PROBE leaves it out.
-    if (!products && !(p->flags & KMC_FLAG_NO_PROBE) &&
-        static_cast<int64_t>(layout.tiles_m) * layout.tiles_n * args.l * layout.slices >= kmc_rules::PROBE_MIN_TILES_TIMES_SLICES) {      // 0.5 ms and more: the sample is 10 us
-        wide.probe = reinterpret_cast<unsigned *>(workspace + layout.probe);
-        wide.probe_pairs = kmc::GW_PROBE_PAIRS / args.l > 1024 ? kmc::GW_PROBE_PAIRS / args.l / kmc::GW_PROBE_GROUP * kmc::GW_PROBE_GROUP : 1024;
-        void *clear_args[] = {&wide.probe};
-        status = hipLaunchKernel(reinterpret_cast<const void *>(kmc::gram_probe_clear<0>), dim3(1), dim3(64), clear_args, 0, stream);
+    // Squared differences: a sample of the result first, so that data the trust rule would reject wholesale
+    // (sets of near-duplicates) costs the direct kernel's time and little more, instead of both.
+    // KMC_FLAG_NO_PROBE leaves it out.
+    if (!products && !(p->flags & KMC_FLAG_NO_PROBE)) {
+        unsigned *sample = reinterpret_cast<unsigned *>(workspace + layout.sample);
+        status = launch_gram_probe(p, wide.kernel, sample, stream);
         if (status != hipSuccess) return status;
-        status = launch(kmc::gram_probe_pairs<0>, dim3(wide.probe_pairs / kmc::GW_PROBE_GROUP, args.l), dim3(kmc::GW_PROBE_GROUP * 64), stream, wide);
-        if (status != hipSuccess) return status;
+        wide.kernel.sample = sample;
     }
     if (args.symmetric) {
         const dim3 grid(static_cast<unsigned>(layout.tiles_m) * (layout.tiles_m + 1) / 2, args.l, 1);

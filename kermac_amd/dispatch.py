@@ -53,16 +53,19 @@ _ROWS = (
      "{WIDE_MIN_TILES_PER_SIDE_X2} · (tiles_m + tiles_n), ≤ {WIDE_MAX_PADDING_PERCENT} % of the tiles' area padding; with k contiguous in both "
      "operands instead: K ≥ {WIDE_K_CONTIGUOUS_MIN_K}, ≥ {WIDE_K_CONTIGUOUS_MIN_TILES} tiles, tiles · K ≥ {WIDE_K_CONTIGUOUS_MIN_TILES_TIMES_K}, M and N ≥ "
      "{WIDE_K_CONTIGUOUS_MIN_ROWS}",
-     "`gram_row_stats` + `gram_f16_split` per operand, `gram_f16_wide` (fp16 pieces, 256 × 256 tiles), repair launch of the direct kernel; "
-     "from tiles · slices ≥ {PROBE_MIN_TILES_TIMES_SLICES} on `gram_probe_pairs` first: {PROBE_BAIL_PER_16384} of {PROBE_PAIRS} sampled pairs "
-     "below the trust threshold, spread over the sampled parts and not packed into few of them, send the whole call to the direct kernel"),
+     "`gram_probe_operands`, `gram_row_stats` + `gram_f16_split` per operand, `gram_f16_wide` (fp16 pieces, 256 × 256 tiles), repair launch "
+     "of the direct kernel"),
     ("",
      "K ≥ {build_a_kernel.AUTO_ONE_STEP_MIN_K} ({build_a_kernel.AUTO_ONE_STEP_MIN_K_ROWS_CONTIGUOUS} with the rows contiguous in both operands), trust < 1, "
      "and not (fewer than 128 tiles of 128 × 128 and a call the direct path would cut over k)",
      "one-step matrix-core kernel: `gram_l2_kernel` (fp32 matrix instruction) with k contiguous in an operand and K ≥ {build_a_kernel.AUTO_FP32_MIN_K} on "
      "{build_a_kernel.AUTO_FP32_MIN_TILES} … {build_a_kernel.AUTO_FP32_MAX_TILES} tiles, or one dimension ≤ 128 with ≥ {build_a_kernel.AUTO_FP32_MIN_TILES} "
-     "tiles; else `gram_bf16_l2_kernel` (three bf16 pieces); repair launch behind either"),
+     "tiles; else `gram_bf16_l2_kernel` (three bf16 pieces); from M · N · K · L ≥ {build_a_kernel.L2_SAMPLE_MIN_TERMS} on `gram_probe_operands` in front "
+     "of either; repair launch behind"),
     ("", "otherwise", "direct `build_kernel<DIFF, SQUARE>`"),
+    ("", "whichever matrix-core kernel runs: the sample of `gram_probe_operands` ({SAMPLE_TILES} tiles of the result, 256 pairs each) shows "
+     "{SAMPLE_LEAVE_PER_16384} pairs in 16384 below the trust threshold, spread over the sampled tiles and not packed into few of them",
+     "the matrix-core kernel only stamps its parts: the repair launch, i.e. the direct kernel, computes everything"),
     ("`run_kernel` of DOT + NOOP (sums of products) into a stored matrix; l2 mode `\"auto\"`",
      "K ≥ {build_a_kernel.L2_DEFAULT_MIN_K} and the library's rule: K ≥ {DOT_MIN_K}, ≥ {DOT_MIN_TILES} tiles, tiles · K ≥ {DOT_MIN_TILES_TIMES_K}, "
      "≤ {WIDE_MAX_PADDING_PERCENT} % padding; or K ≥ {DOT_LONG_K}, tiles · K ≥ {DOT_LONG_MIN_TILES_TIMES_K}, ≥ {DOT_LONG_MIN_TILES_BATCHED} tiles "

@@ -297,3 +297,59 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
         assert torch.equal(got, kermac.cdist(points, points.clone(), p=2.0)[0])
     assert_close_to_truth(got, oracle.cdist(points.cpu(), points.cpu(), p=2.0)[0], rtol=1e-5, atol=1e-30,
                           what="auto, near-duplicate points")
+
+
+def test_the_one_step_kernels_look_before_they_multiply(device, monkeypatch):
+    """A problem of 8.6e9 terms that the default mode gives to a one-step matrix-core kernel (256 tiles of 256 x 256 at
+    K = 512: too few for the route through a workspace): the Python layer hands the library KMC_SAMPLE_BYTES of workspace,
+    and the library samples the result first.  Points drawn around 64 centres in any order have a near-duplicate pair in
+    every tile: the kernel only stamps its tiles, and the result is the direct kernel's bit for bit.  The same points stored
+    cluster by cluster have them in the blocks on the diagonal only: the matrix cores keep the call.  Without the sample
+    (KERMAC_AMD_L2_PROBE=0) every tile is multiplied, checked and recomputed: the same bits as with it."""
+    from kermac_amd import _backend, build_a_kernel as module
+    M = N = 4096
+    K = 512
+    g = torch.Generator().manual_seed(21)
+    middle = 10.0 * torch.randn(64, K, generator=g)
+
+    def clustered(rows, cluster_by_cluster):
+        which = torch.randint(0, 64, (rows,), generator=g)
+        if cluster_by_cluster:
+            which = which.sort().values
+        # rows contiguous (the benchmark's storage): with k contiguous this shape would take the route through a workspace
+        return (middle[which] + 1e-3 * torch.randn(rows, K, generator=g)).to(device).t().contiguous().t()
+
+    assert kermac.get_l2_mode() == "auto"
+    a, b = clustered(M, False), clustered(N, False)
+    plan = module._plan_run_kernel(kermac.kernel_descriptor_l2_norm, a, b, None, None, None, None, None, None, None, 0, 0, False)
+    plan.params.flags = (plan.params.flags & ~(_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16)) | module._auto_matrix_core_flags(
+        plan.params, plan.params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16))
+    assert plan.params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16) and _backend.gram_workspace_bytes(plan.params) == 0
+    workspace = module._attach_gram_workspace(plan.params, device)
+    assert workspace is not None and workspace.numel() == _backend.SAMPLE_BYTES
+
+    got = kermac.cdist(a, b, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        plain = kermac.cdist(a, b, p=2.0)[0]
+    assert torch.equal(got, plain)
+    assert_close_to_truth(got[:256, :256], torch.cdist(a[:256].double(), b[:256].double()), rtol=1e-5, atol=1e-30, what="clusters, any order")
+    monkeypatch.setenv("KERMAC_AMD_L2_PROBE", "0")
+    assert torch.equal(kermac.cdist(a, b, p=2.0)[0], plain)
+    monkeypatch.delenv("KERMAC_AMD_L2_PROBE")
+
+    a, b = clustered(M, True), clustered(N, True)
+    got = kermac.cdist(a, b, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        plain = kermac.cdist(a, b, p=2.0)[0]
+    same = got == plain
+    assert same[:32, :32].all() and not same[:64, -64:].all() and (~same).float().mean().item() > 0.2
+    rows = torch.cat([torch.arange(0, 256), torch.arange(M - 128, M)]).to(device)
+    assert_close_to_truth(got[rows][:, :512], torch.cdist(a[rows].double(), b[:512].double()), rtol=1e-5, atol=1e-30,
+                          what="clusters stored one after the other")
+
+    # spread-out data of the same shape: the sample finds nothing, the matrix cores' bits
+    x, y = torch.randn(K, M, generator=g).to(device).t(), torch.randn(K, N, generator=g).to(device).t()
+    got = kermac.cdist(x, y, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        assert not torch.equal(got, kermac.cdist(x, y, p=2.0)[0])
+    assert_close_to_truth(got[:256, :256], torch.cdist(x[:256].double(), y[:256].double()), rtol=1e-5, what="spread-out data")
