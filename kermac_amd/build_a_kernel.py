@@ -672,23 +672,33 @@ def _attach_gram_centre(params, stream, device):
 #   * the route through a workspace wherever the library takes it (kmc_gram_workspace_bytes: large
 #     problems from K = 64 on; 10000 x 10000 x 96 413 / 304, 4096 x 4096 x 4096 2400 cut / 530, 4096 x 4096 x 20000
 #     12500 / 2300), sums of products nowhere else (they have no one-step kernel);
-#   * the one-step kernels from K = 192 on (128 x 128 x 200 65 / 37, 8 x 256 x 256 x 512 141 / 54, 2000 x 2000 x 200
-#     71 / 52; at K = 64 .. 160 the direct kernel is as fast or faster: 4096 x 4096 x 64 59 / 83, 1000 x 30000 x 128
-#     178 / 233, 8 x 1000 x 1000 x 160 67 / 81), unless the direct path would cut the call over k and the
-#     grid is below 128 tiles (1024 x 1024 x 32768: 1400 cut / 10000; 1536 x 1536 x 4096 380 cut / 250), or the
+#   * the one-step kernels from K = 128 on (128 x 128 x 200 65 / 37, 8 x 256 x 256 x 512 141 / 54, 2000 x 2000 x 200
+#     71 / 52; at K = 128 over ten shapes, k contiguous: 512 x 512 40 / 31, 1000 x 30000 165 / 127, 32 x 256 x 256 41 / 32,
+#     4096 x 4096 90 / 86, 2000 x 2000 44 / 46, 2500 x 2500 50 / 59, the one that loses more than a tenth; with the rows
+#     contiguous 2000 x 2000 45 / 36, 5000 x 5000 146 / 116; at K = 96 the direct kernel is ahead, 0.73 .. 0.97, but for
+#     few rows against many: 1000 x 30000 x 96 130 / 115), unless the direct path would cut the call over k and the grid is
+#     below 192 tiles (1024 x 1024 x 32768: 1400 cut / 10000; 1500 x 1500 x 3072 312 cut / 408), or the
 #     contraction is so long that they trust nothing they compute (K > 18000: every tile would be redone);
 #   * of the one-step kernels the fp32 one for K >= 384 on 128 to 768 tiles (2000 x 2000 x 784 fp32 135 / split 171,
 #     8 x 1000 x 1000 x 3072 634 / 855), the split one otherwise (K = 200: 47 .. 55 / 37 .. 44; 4096 x 4096 x 512 212 / 161;
 #     8 x 256 x 256 x 512, 32 tiles, 69 / 55), and for a single row of 128 tiles or more (4 x 100 x 50000
 #     x 784 fp32 558 / split 857, at K = 256 252 / 340);
 #   * the numbers above are for operands with k contiguous, as torch allocates them.  With the rows contiguous
-#     (the kernels' own order) the split kernel stages faster: it is taken from K = 128 on (5000 x 5000 x 128 155 /
-#     119, 30000 x 1500 x 128 242 / 165) and instead of the fp32 one (2500 x 2500 x 1024 fp32 198 / split 137).
-_AUTO_ONE_STEP_MIN_K = 192
-_AUTO_ONE_STEP_MIN_K_ROWS_CONTIGUOUS = 128
+#     (the kernels' own order) the split kernel stages faster: it is taken instead of the fp32 one (2500 x 2500 x 1024
+#     fp32 198 / split 137), and uncut from 128 tiles on.
+_AUTO_ONE_STEP_MIN_K = 128
 _AUTO_FP32_MIN_K = 384
 _AUTO_FP32_MIN_TILES = 128
 _AUTO_FP32_MAX_TILES = 768
+# ... and only for batch entries of 32 tiles and more: on batches of small entries the split kernel is far ahead
+# (8 x 512 x 512 x 1024, k contiguous: fp32 108 / split 69 us; 32 x 256 x 256 x 3072 280 / 163; 8 x 700 x 700 x 1024 216 / 228)
+_AUTO_FP32_MIN_TILES_PER_ENTRY = 32
+# A call that the direct path would cut over k stays there below this many tiles: the matrix cores run it uncut.
+# With k contiguous the one-step kernels stage more slowly and need more tiles to be ahead (1500 x 1500, 144 tiles:
+# direct, cut / fp32 at K = 784 107 / 130 us, at K = 3072 312 / 408; 500 x 5000, 160 tiles, 125 / 121 and 343 / 396;
+# 2000 x 2000, 256 tiles, 157 / 130 and 493 / 408; with the rows contiguous 1536 x 1536 x 4096 380 / 250).
+_AUTO_UNCUT_MIN_TILES = 128
+_AUTO_UNCUT_MIN_TILES_K_CONTIGUOUS = 192
 
 
 def _auto_matrix_core_flags(params, asked):
@@ -697,11 +707,10 @@ def _auto_matrix_core_flags(params, asked):
         return asked
     # operands with the rows contiguous (m or n, the kernels' own order) stage faster in the split kernel
     rows_contiguous = params.a_majorness == _backend.COL_MAJOR and params.b_majorness == _backend.COL_MAJOR
-    one_step_min_k = _AUTO_ONE_STEP_MIN_K_ROWS_CONTIGUOUS if rows_contiguous else _AUTO_ONE_STEP_MIN_K
-    if not asked & _backend.FLAG_L2_GRAM or params.k < one_step_min_k or params.gram_trust >= 1.0:
+    if not asked & _backend.FLAG_L2_GRAM or params.k < _AUTO_ONE_STEP_MIN_K or params.gram_trust >= 1.0:
         return 0
     tiles = -(-params.m // 128) * -(-params.n // 128)
-    if tiles < 128:
+    if tiles < (_AUTO_UNCUT_MIN_TILES if rows_contiguous else _AUTO_UNCUT_MIN_TILES_K_CONTIGUOUS):
         kept = params.flags
         params.flags &= ~asked                  # the question is what the direct path would do
         try:
@@ -710,7 +719,8 @@ def _auto_matrix_core_flags(params, asked):
         finally:
             params.flags = kept
     if not rows_contiguous:
-        if params.k >= _AUTO_FP32_MIN_K and _AUTO_FP32_MIN_TILES <= tiles * params.l <= _AUTO_FP32_MAX_TILES:
+        if (params.k >= _AUTO_FP32_MIN_K and _AUTO_FP32_MIN_TILES <= tiles * params.l <= _AUTO_FP32_MAX_TILES
+                and tiles >= _AUTO_FP32_MIN_TILES_PER_ENTRY):
             return _backend.FLAG_L2_GRAM
         if min(params.m, params.n) <= 128 and tiles * params.l >= _AUTO_FP32_MIN_TILES:      # one long row of tiles
             return _backend.FLAG_L2_GRAM

@@ -56,10 +56,12 @@ _ROWS = (
      "`gram_probe_operands`, `gram_row_stats` + `gram_f16_split` per operand, `gram_f16_wide` (fp16 pieces, 256 × 256 tiles), repair launch "
      "of the direct kernel"),
     ("",
-     "K ≥ {build_a_kernel.AUTO_ONE_STEP_MIN_K} ({build_a_kernel.AUTO_ONE_STEP_MIN_K_ROWS_CONTIGUOUS} with the rows contiguous in both operands), trust < 1, "
-     "and not (fewer than 128 tiles of 128 × 128 and a call the direct path would cut over k)",
+     "K ≥ {build_a_kernel.AUTO_ONE_STEP_MIN_K}, trust < 1, "
+     "and not (a call the direct path would cut over k on fewer than {build_a_kernel.AUTO_UNCUT_MIN_TILES_K_CONTIGUOUS} tiles of 128 × 128, "
+     "{build_a_kernel.AUTO_UNCUT_MIN_TILES} with the rows contiguous)",
      "one-step matrix-core kernel: `gram_l2_kernel` (fp32 matrix instruction) with k contiguous in an operand and K ≥ {build_a_kernel.AUTO_FP32_MIN_K} on "
-     "{build_a_kernel.AUTO_FP32_MIN_TILES} … {build_a_kernel.AUTO_FP32_MAX_TILES} tiles, or one dimension ≤ 128 with ≥ {build_a_kernel.AUTO_FP32_MIN_TILES} "
+     "{build_a_kernel.AUTO_FP32_MIN_TILES} … {build_a_kernel.AUTO_FP32_MAX_TILES} tiles over the batch and ≥ {build_a_kernel.AUTO_FP32_MIN_TILES_PER_ENTRY} per entry, "
+     "or one dimension ≤ 128 with ≥ {build_a_kernel.AUTO_FP32_MIN_TILES} "
      "tiles; else `gram_bf16_l2_kernel` (three bf16 pieces); from M · N · K · L ≥ {build_a_kernel.L2_SAMPLE_MIN_TERMS} on `gram_probe_operands` in front "
      "of either; repair launch behind"),
     ("", "otherwise", "direct `build_kernel<DIFF, SQUARE>`"),

@@ -323,7 +323,7 @@ def test_l2_mode_sets_the_gram_flag_only_for_squared_differences():
 def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
     """The l2 mode "auto" decides from the parameter block (and the library's answer about its
     workspace route, which needs no device): the route through a workspace where the library takes
-    it, the one-step kernels from K = 192 on (the fp32 one for long contractions over few tiles),
+    it, the one-step kernels from K = 128 on (the fp32 one for long contractions over few tiles),
     the direct kernel for short contractions, for grids it would rather cut over k, and for
     contractions so long that the one-step kernels would trust nothing."""
     from kermac_amd import build_a_kernel as module
@@ -344,20 +344,24 @@ def test_auto_mode_picks_the_kernel_by_shape_without_a_gpu(monkeypatch):
 
     assert chosen(128, 128, 200) == core                         # one step, split pieces
     assert chosen(100, 50000, 256, l=4) == _backend.FLAG_L2_GRAM   # one long row of tiles: fp32
-    assert chosen(1500, 1500, 784) == _backend.FLAG_L2_GRAM      # one step, fp32: a long contraction over 144 tiles
+    assert chosen(1500, 1500, 384) == _backend.FLAG_L2_GRAM      # one step, fp32: 144 tiles, a contraction the direct path does not cut
+    assert chosen(1500, 1500, 784) == 0                          # ... one it does cut: 144 tiles with k contiguous stay with it
+    assert chosen(512, 512, 1024, l=8) == core                   # 128 tiles in entries of 16: split pieces, not fp32
+    assert chosen(700, 700, 1024, l=4) == _backend.FLAG_L2_GRAM  # 144 tiles in entries of 36: fp32
     assert chosen(2000, 2000, 784) == core                       # 64 tiles of 256 x 256, k contiguous: the workspace route
     assert chosen(4096, 4096, 512) == core                       # 1024 tiles: split pieces
-    assert chosen(4096, 4096, 64) == 0 and chosen(1000, 30000, 160) == 0
+    assert chosen(4096, 4096, 64) == 0 and chosen(1000, 30000, 120) == 0 and chosen(1000, 30000, 128) == core
     assert chosen(10000, 10000, 96) == core                      # the library's workspace route
     assert chosen(4096, 4096, 4096) == core                      # ... also where the direct path would cut over k
     assert chosen(4096, 4096, 20000) == core                     # ... and for contractions the one-step kernels would not trust
     assert chosen(1500, 1500, 20000) == 0
     assert chosen(1024, 1024, 32768) == 0                        # 64 tiles: cut over k by the direct path
-    assert chosen(1536, 1536, 4096) == _backend.FLAG_L2_GRAM     # 144 tiles: uncut on the matrix cores
+    assert chosen(1536, 1536, 4096) == 0                         # 144 tiles, k contiguous: cut over k as well
+    assert chosen(1536, 1536, 4096, rows_contiguous=True) == core  # rows contiguous: uncut on the matrix cores from 128 tiles on
     assert chosen(256, 256, 512, l=8) == core
-    # operands stored with the rows contiguous: the split kernel from K = 128 on, and instead of the fp32 one
-    assert chosen(5000, 5000, 128, rows_contiguous=True) == core and chosen(5000, 5000, 128) == 0
-    assert chosen(1500, 1500, 1024, rows_contiguous=True) == core and chosen(1500, 1500, 1024) == _backend.FLAG_L2_GRAM
+    # operands stored with the rows contiguous: the split kernel instead of the fp32 one
+    assert chosen(5000, 5000, 128, rows_contiguous=True) == core and chosen(5000, 5000, 128) == core and chosen(5000, 5000, 112) == 0
+    assert chosen(1500, 1500, 1024, rows_contiguous=True) == core and chosen(1500, 1500, 400) == _backend.FLAG_L2_GRAM
     assert chosen(2000, 2000, 784, rows_contiguous=True) == core              # the split one-step kernel there
     assert chosen(8192, 4096, 512, dot=True) == _backend.FLAG_DOT_PIECES
     assert chosen(300, 300, 512, dot=True) == 0

@@ -257,8 +257,8 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
     big = planned(8000, 8000, 128)
     assert big.l2_auto and big.params.flags & core == core and big.params.gram_trust > 0
     assert chosen(8000, 8000, 128) == core                                       # the route through a workspace
-    assert chosen(500, 500, 128) == 0                                            # a short contraction: direct
-    assert chosen(500, 500, 256) == core                                         # one step, from K = 192 on
+    assert chosen(500, 500, 112) == 0                                            # a short contraction: direct
+    assert chosen(500, 500, 256) == core                                         # one step, from K = 128 on
     assert planned(16000, 16000, 32).params.flags & core == 0                    # K below min_k: direct
     assert planned(8000, 8000, 128, kermac.kernel_descriptor_l1_norm).params.flags & core == 0
     assert chosen(8000, 8000, 128, kermac.kernel_descriptor_laplace_l2, bandwidth=2.0) == core
@@ -275,18 +275,20 @@ def test_auto_mode_picks_the_kernel_by_shape(device):
     with kermac.l2_mode("direct"):
         assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0])
     assert_close_to_truth(got, oracle.cdist(x.cpu(), y.cpu(), p=2.0)[0], rtol=1e-5, what="auto, long contraction")
-    # results the direct path would cut over k, but large enough for the matrix cores uncut: 144 tiles of
-    # 128 x 128 on the one-step kernel (36 of 256 x 256 are too few for the route through a workspace; of the
-    # one-step kernels the fp32 one here: a long contraction with k contiguous), 144 tiles of 256 x 256 on that route
-    for rows, depth, mode in ((1500, 2048, "gram"), (3000, 2048, "gram_bf16")):
+    # results the direct path would cut over k, but large enough for the matrix cores uncut: with the rows contiguous
+    # 144 tiles of 128 x 128 on the split one-step kernel (36 of 256 x 256 are too few for the route through a
+    # workspace); with k contiguous 144 tiles of 256 x 256 on that route, and 144 of 128 x 128 left to the direct path
+    for rows, depth, mode, rows_contiguous in ((1500, 2048, "gram_bf16", True), (3000, 2048, "gram_bf16", False), (1500, 2048, "direct", False)):
         x = torch.randn(rows, depth, generator=g).to(device)
         y = torch.randn(rows, depth, generator=g).to(device)
+        if rows_contiguous:
+            x, y = x.t().contiguous().t(), y.t().contiguous().t()
         assert module._cut_over_contraction(planned(rows, rows, depth, kermac.kernel_descriptor_l1_norm).params) is not None
         got = kermac.cdist(x, y, p=2.0)[0]
         with kermac.l2_mode(mode):
-            assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0]), f"{rows} x {rows} x {depth}: expected the matrix cores"
+            assert torch.equal(got, kermac.cdist(x, y, p=2.0)[0]), f"{rows} x {rows} x {depth}: expected {mode}"
         truth = torch.cdist(x[:64].double(), y[:64].double(), p=2.0)
-        assert_close_to_truth(got[:64, :64], truth, rtol=1e-5, what="auto, uncut on the matrix cores")
+        assert_close_to_truth(got[:64, :64], truth, rtol=1e-5, what="auto on results the direct path would cut")
     # a large problem in auto mode equals the explicit split-bf16 mode, near-duplicate tiles included
     g = torch.Generator().manual_seed(6)
     points = torch.randn(4400, 256, generator=g)
