@@ -870,12 +870,13 @@ def test_scratch_memory_is_handed_out_within_the_limit_or_from_the_callers_buffe
 def test_the_dispatch_table_of_the_design_is_the_generated_one():
     """One source of truth for "which kernel runs when": the thresholds live in csrc/host/dispatch_rules.hpp (read by the
     library's rules, printed by kmc_dispatch_rules) and in the Python layer's module constants; kermac_amd.dispatch renders the
-    table from them, and the copy in DESIGN.md must be that rendering.  The rules themselves must flip at the printed numbers."""
+    table from them, and the copy in the design document at the repository root must be that rendering.  The rules themselves
+    must flip at the printed numbers."""
     from kermac_amd import dispatch
     known = dispatch.rules()
     table = dispatch.table_markdown()
     design = (ROOT / "DESIGN.md").read_text()
-    assert table in design, "DESIGN.md: regenerate the dispatch table with `python -m kermac_amd.dispatch`"
+    assert table in design, "the design document's copy of the dispatch table is stale: regenerate it with `python -m kermac_amd.dispatch`"
     header = (ROOT / "include" / "kermac_amd.h").read_text()
     assert "kmc_dispatch_rules" in header and "147456" not in header and "36864" not in header      # pointed to, not restated
     fake = 4096
