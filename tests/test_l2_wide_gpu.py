@@ -336,6 +336,34 @@ def test_near_duplicates_stored_cluster_by_cluster_stay_on_the_matrix_cores(devi
     assert_close_to_truth(got[rows][:, :768], truth, rtol=1e-5, atol=1e-30, what="clusters stored one after the other")
 
 
+def test_a_clustered_set_against_itself_and_a_batch_of_clustered_sets(device):
+    """The sample in front of the product kernel on a panel against itself (only the tiles on and below the diagonal are
+    stamped; the repair launch computes them and mirrors them) and on a batch (the sampled tiles are spread over the
+    entries): clustered points in any order, so everything is left to the direct kernel -- its bits, a symmetric result,
+    the tolerance."""
+    K = 1024
+    middle = 10.0 * torch.randn(64, K, generator=torch.Generator().manual_seed(14))
+    x = clustered(8192, middle, device, 15).t().contiguous().t()
+    assert kermac.get_l2_mode() == "auto"
+    got = kermac.cdist(x, x, p=2.0)[0]
+    with kermac.l2_mode("direct"):
+        plain = kermac.cdist(x, x, p=2.0)[0]
+    assert torch.equal(got, plain) and torch.equal(got, got.t())
+    truth = torch.cdist(x[:256].double(), x[4096:4608].double(), p=2.0)
+    assert_close_to_truth(got[:256, 4096:4608], truth, rtol=1e-5, atol=1e-30, what="a clustered set against itself")
+
+    a = torch.stack([clustered(4096, middle, device, 16 + i) for i in range(4)]).transpose(1, 2).contiguous().transpose(1, 2)
+    b = torch.stack([clustered(4096, middle, device, 26 + i) for i in range(4)]).transpose(1, 2).contiguous().transpose(1, 2)
+    with kermac.l2_mode("gram_bf16"):
+        assert workspace_bytes(a, b) > 0
+    got = kermac.cdist(a, b, p=2.0)
+    with kermac.l2_mode("direct"):
+        plain = kermac.cdist(a, b, p=2.0)
+    assert torch.equal(got, plain)
+    truth = torch.cdist(a[3, :256].double(), b[3, :256].double(), p=2.0)
+    assert_close_to_truth(got[3, :256, :256], truth, rtol=1e-5, atol=1e-30, what="a batch of clustered sets")
+
+
 def test_the_kept_split_is_made_again_when_it_is_not_the_one_needed(device, wide):
     """KMC_FLAG_GRAM_A_KEPT on a workspace that holds no split of this `a` (never used, used for another `a`, used by
     another route in between): the library notices from its record of the workspace and makes the split; the result is
