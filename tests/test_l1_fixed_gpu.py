@@ -180,6 +180,50 @@ def test_batches_kernels_and_offsets(device, fixed):
     assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-7, what="laplace, batch of 3")
 
 
+def test_the_sample_tells_near_duplicates_everywhere_from_near_duplicates_in_few_tiles(device):
+    """4096 tiles by the route's own rule.  Points drawn around 64 centres in any order: every tile holds pairs whose
+    distance is a few grid steps, the sample sees them spread over its tiles, the conversion and the walk do nothing and
+    the result is the direct kernel's.  The same points stored cluster by cluster: those pairs fill the blocks on the
+    diagonal, one tile in 64, the walk runs and only those blocks are recomputed.  Every other feature constant: one
+    pair in two thousand just below the threshold, spread evenly -- eight per tile -- and the call is left to the
+    direct kernel as well.  The tolerance holds in all three."""
+    M = N = 8192
+    K = 512
+    g = torch.Generator().manual_seed(33)
+    middle = 10.0 * torch.randn(64, K, generator=g)
+
+    def clustered(rows, cluster_by_cluster):
+        which = torch.randint(0, 64, (rows,), generator=g)
+        if cluster_by_cluster:
+            which = which.sort().values
+        return (middle[which] + 1e-3 * torch.randn(rows, K, generator=g)).to(device).t().contiguous().t()
+
+    def both(a, b):
+        with kermac.l1_mode("fixed"):
+            assert workspace_bytes(a, b) > 0         # the route applies by its own rule
+            got = kermac.cdist(a, b, p=1.0)[0]
+        return got, direct(lambda: kermac.cdist(a, b, p=1.0))[0]
+
+    a, b = clustered(M, False), clustered(N, False)
+    got, plain = both(a, b)
+    assert torch.equal(got, plain)
+    assert_close_to_truth(got[:200, :300], l1_distances_float64(a[:200], b[:300]), rtol=1e-5, atol=1e-30, what="clusters in any order")
+
+    a, b = clustered(M, True), clustered(N, True)
+    got, plain = both(a, b)
+    same = got == plain
+    assert same[:32, :32].all() and not same[:64, -64:].all() and (~same).float().mean().item() > 0.2
+    rows = torch.cat([torch.arange(0, 150), torch.arange(M - 50, M)]).to(device)
+    assert_close_to_truth(got[rows][:, :300], l1_distances_float64(a[rows], b[:300]), rtol=1e-5, atol=1e-30, what="clusters one after the other")
+
+    a = torch.randn(K, M, generator=g); a[::2] = 3.0
+    b = torch.randn(K, N, generator=g); b[::2] = 3.0
+    a, b = a.to(device).t(), b.to(device).t()
+    got, plain = both(a, b)
+    assert torch.equal(got, plain)
+    assert_close_to_truth(got[:200, :300], l1_distances_float64(a[:200], b[:300]), rtol=1e-5, what="every other feature constant")
+
+
 def test_a_tighter_tolerance_repairs_more(device, monkeypatch):
     monkeypatch.setenv("KERMAC_AMD_L1_FIXED_ANY_SIZE", "1")
     g = torch.Generator().manual_seed(3)
