@@ -34,6 +34,10 @@
     X(SAMPLE_LEAVE_PER_16384, 2)           /* pairs below the trust threshold, spread over the tiles */ \
     /* the direct kernel compiled for four waves per SIMD (k-major panels, no fractional power) */       \
     X(DIRECT_FOUR_WAVES_MIN_K, 256)                                                                     \
+    /* ... and the one with b in scalar registers (absolute and squared differences, K and N multiples of 16): */ \
+    /* tiles of 256 x 64 in every batch entry */                                                         \
+    X(DIRECT_SCALAR_B_MIN_TILES, 1800)                                                                  \
+    X(DIRECT_SCALAR_B_MIN_K, 64)                                                                        \
     /* absolute differences on fixed point (KMC_FLAG_L1_FIXED): tiles of 128 x 128 over the batch */    \
     X(L1_FIXED_MIN_TILES, 2048)                                                                         \
     X(L1_FIXED_MIN_K, 128)                                                                              \

@@ -3,8 +3,11 @@
 // Compiled several times with different -DKMC_INNER_OP / -DKMC_INNER_POW.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "launch.hpp"
 #include "build_kernel.hpp"
+#include "build_kernel_scalar_b.hpp"
 #include "../host/dispatch_rules.hpp"
 
 #ifndef KMC_INNER_OP
@@ -17,9 +20,44 @@
 
 namespace kmc_host {
 
+// Whether the call is one for build_kernel_scalar_b (its header says what the kernel assumes): enough tiles of
+// 256 x 64 in every batch entry to fill the chip twice.  From a sweep against build_kernel / build_kernel_four_waves
+// (their time / this kernel's, p = 1 and p = 2, K = 64 .. 4096): 2256 tiles (6000 x 6000) 1.02 .. 1.07 and 1.05 .. 1.10,
+// 1876 (1000 x 30000) 1.01 .. 1.02 and 1.03 .. 1.07, 3776 (30000 x 2000) 1.04 .. 1.21, 55342 (30000 x 30000) 1.02 .. 1.05 and
+// 1.05 .. 1.08; 1024 tiles (4096 x 4096) 0.96 .. 1.03, and batches of small entries lose: 8 x 2048 x 2048 0.95 .. 1.0,
+// 64 x 512 x 512 0.91 .. 1.0 for p = 1.
+// KERMAC_AMD_SCALAR_B_MIN_TILES=n replaces the size rule by "at least n tiles over the batch, any k" (read on every
+// call, so that a test can send small shapes to the kernel).
+static bool scalar_b_applies(const kmc::BuildKernelArgs &args, int64_t *tiles_m, int64_t *tiles_n)
+{
+    if (args.k < 16 || args.k % kmc::BK_TILE_K != 0 || args.n % kmc::SB_WAVE_N != 0 || args.k_total != 0 || args.repair_only || args.symmetric)
+        return false;
+    *tiles_m = (static_cast<int64_t>(args.m) + kmc::SB_TILE_M - 1) / kmc::SB_TILE_M;
+    *tiles_n = (static_cast<int64_t>(args.n) + kmc::SB_TILE_N - 1) / kmc::SB_TILE_N;
+    const int64_t tiles = *tiles_m * *tiles_n;
+    if (tiles > 0x7fffffff) return false;
+    const char *text = std::getenv("KERMAC_AMD_SCALAR_B_MIN_TILES");
+    const int forced = text ? std::atoi(text) : 0;
+    if (forced > 0) return tiles * args.l >= forced;
+    return tiles >= kmc_rules::DIRECT_SCALAR_B_MIN_TILES && args.k >= kmc_rules::DIRECT_SCALAR_B_MIN_K;
+}
+
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)
 {
+    // absolute and squared differences of large problems whose rows are contiguous on both sides: b in scalar registers
+    if constexpr (LOAD_A == kmc::LOAD_COL_VEC && LOAD_B == kmc::LOAD_COL_VEC && KMC_INNER_OP == kmc::OP_DIFF &&
+                  (KMC_INNER_POW == kmc::POW_ABS || KMC_INNER_POW == kmc::POW_SQUARE)) {
+        int64_t tiles_m = 0, tiles_n = 0;
+        if (scalar_b_applies(args, &tiles_m, &tiles_n)) {
+            kmc::BuildKernelArgs copy = args;
+            const float *a = args.a, *b = args.b;
+            float *c = args.c;
+            void *kernel_args[] = {&copy, &a, &b, &c};
+            return hipLaunchKernel(reinterpret_cast<const void *>(kmc::build_kernel_scalar_b<KMC_INNER_OP, KMC_INNER_POW>),
+                                   dim3(static_cast<unsigned>(tiles_m * tiles_n), args.l), dim3(kmc::BK_THREADS), kernel_args, 0, stream);
+        }
+    }
     // contiguous rows on both sides, a contraction long enough for the walk to set the time, and an inner term
     // without transcendentals (whose loop needs more registers): the variant compiled for four waves per SIMD
     if constexpr (LOAD_A == kmc::LOAD_COL_VEC && LOAD_B == kmc::LOAD_COL_VEC && KMC_INNER_POW != kmc::POW_POW) {

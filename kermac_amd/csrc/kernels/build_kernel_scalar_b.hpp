@@ -1,0 +1,209 @@
+// The direct kernel for large problems whose panels have their rows contiguous: the b operand in scalar registers.
+//
+// build_kernel (build_kernel.hpp) stages both operands in LDS and every lane reads 16 floats of fragments per k
+// for its 8 x 8 results -- a quarter of a float per term, 1 TB per launch at M = N = 30000, K = 1024, and with the
+// copies that feed them the reason why the kernel runs at 2.1 GHz where its arithmetic alone runs at 2.37.  Here
+// a wave owns 16 columns n and ALL its lanes share them, so b[n, k] is the same for every lane: it is loaded by
+// scalar loads into scalar registers and enters the vector instructions as their scalar operand, which costs no
+// LDS traffic at all.  A lane owns 4 consecutive rows m x those 16 columns: one 16-byte LDS read per k for 128
+// vector instructions (a sixteenth of a float per term), and only a passes through LDS (copied straight from
+// memory by global_load_lds_dwordx4, 1 KB per k-row of the 256 x 64 tile).  Workgroup 4 waves = 256 (m) x 64 (n),
+// 92 registers, 33 KB of LDS, four workgroups per CU.  Measured on the walk alone, same box, M = N = 30000,
+// K = 1024: 27.4 ms against 28.3 ms for build_kernel_four_waves (8 waves per workgroup on 256 x 128: 28.7; the
+// 8 x 8 lane tile with b in scalar registers, 512 x 64: 28.4; five waves per SIMD: 27.6; tile order in bands of
+// 8 tile rows: 28.0).
+//
+// What the host guarantees before it launches this kernel (build_kernel_inst.hip): both operands with rows
+// contiguous and 16-byte aligned (the LOAD_COL_VEC loaders), K a multiple of 16, N a multiple of 16 (a wave's 16
+// columns exist or do not), no ranges of one contraction (k_total = 0), not a repair launch, not the triangle of
+// a symmetric result.  The last tile row may be ragged in m: lanes beyond M copy nothing and store nothing.
+// Results are those of build_kernel bit for bit: every element sums its terms over k in the same order.
+// The reference has one kernel for all shapes (include/build_a_kernel.cuh:339-462).
+#pragma once
+
+#include "build_kernel.hpp"
+
+namespace kmc {
+
+constexpr int SB_TILE_M = 256;      // 64 lanes x 4 rows
+constexpr int SB_WAVE_N = 16;       // columns of a wave: 16 scalars per k
+constexpr int SB_TILE_N = 4 * SB_WAVE_N;
+constexpr int SB_CHUNK = 4;         // k per group of scalar loads (64 scalar registers)
+
+// Two columns at a time: 8 independent subtractions (scalar minus vector), then 8 independent accumulations, as
+// in row_abs_diff / row_square_diff of build_kernel.hpp.
+#define KMC_SB_SUB8 \
+    "v_sub_f32 %8, %20, %16\n\tv_sub_f32 %9, %20, %17\n\tv_sub_f32 %10, %20, %18\n\tv_sub_f32 %11, %20, %19\n\t" \
+    "v_sub_f32 %12, %21, %16\n\tv_sub_f32 %13, %21, %17\n\tv_sub_f32 %14, %21, %18\n\tv_sub_f32 %15, %21, %19\n\t"
+#define KMC_SB_OPERANDS \
+    : "+v"(acc0[0]), "+v"(acc0[1]), "+v"(acc0[2]), "+v"(acc0[3]), "+v"(acc1[0]), "+v"(acc1[1]), "+v"(acc1[2]), "+v"(acc1[3]), \
+      "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7) \
+    : "v"(fa[0]), "v"(fa[1]), "v"(fa[2]), "v"(fa[3]), "s"(b0), "s"(b1)
+
+template <int INNER_POW>
+__device__ __forceinline__ void scalar_b_pair(float (&acc0)[4], float (&acc1)[4], const float (&fa)[4], float b0, float b1)
+{
+    static_assert(INNER_POW == POW_ABS || INNER_POW == POW_SQUARE, "absolute and squared differences only");
+    float t0, t1, t2, t3, t4, t5, t6, t7;
+    if (INNER_POW == POW_ABS) {
+        asm volatile(KMC_SB_SUB8
+                     "v_add_f32 %0, |%8|, %0\n\tv_add_f32 %1, |%9|, %1\n\tv_add_f32 %2, |%10|, %2\n\tv_add_f32 %3, |%11|, %3\n\t"
+                     "v_add_f32 %4, |%12|, %4\n\tv_add_f32 %5, |%13|, %5\n\tv_add_f32 %6, |%14|, %6\n\tv_add_f32 %7, |%15|, %7"
+                     KMC_SB_OPERANDS);
+    } else {
+        asm volatile(KMC_SB_SUB8
+                     "v_fmac_f32 %0, %8, %8\n\tv_fmac_f32 %1, %9, %9\n\tv_fmac_f32 %2, %10, %10\n\tv_fmac_f32 %3, %11, %11\n\t"
+                     "v_fmac_f32 %4, %12, %12\n\tv_fmac_f32 %5, %13, %13\n\tv_fmac_f32 %6, %14, %14\n\tv_fmac_f32 %7, %15, %15"
+                     KMC_SB_OPERANDS);
+    }
+}
+
+__device__ __forceinline__ void scalar_b_fragment(float (&f)[4], const float *p)
+{
+    const float4 v = *reinterpret_cast<const float4 *>(p);
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+
+// The operands come in twice: inside `args`, and as restrict-qualified parameters, which is what lets the compiler
+// prove that nothing the kernel writes (the copies into LDS, the result) can change b, and so load it with scalar
+// loads (through args.b it takes vector loads of one address for all lanes, and the kernel spills).
+template <int INNER_OP, int INNER_POW>
+__global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const BuildKernelArgs args, const float *__restrict__ operand_a,
+                                                                      const float *__restrict__ operand_b, float *__restrict__ result)
+{
+    static_assert(INNER_OP == OP_DIFF, "differences only");
+    // two slices of 16 k-rows, and one row that the fragment read ahead of the last k of the second slice touches
+    __shared__ __attribute__((aligned(16))) float lds_a[(2 * BK_TILE_K + 1) * SB_TILE_M];
+    const int tid = threadIdx.x;
+    const int batch = blockIdx.y;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // consecutive workgroups walk n: the ~128 of them resident on an XCD share one or two row blocks of a through its L2
+    const int tiles_n = (args.n + SB_TILE_N - 1) / SB_TILE_N;
+    const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x - tile_m * tiles_n;
+    const int m0 = tile_m * SB_TILE_M;
+    const int n0 = tile_n * SB_TILE_N + SB_WAVE_N * wave;        // uniform over the wave
+    const int m_valid = args.m - m0;
+    const bool wave_has_columns = n0 < args.n;                   // all 16 or none: n is a multiple of 16
+    const bool lane_copies = 4 * lane < m_valid;                 // the 16 bytes lie inside the row: its length is a multiple of 4 floats
+
+    typedef const __attribute__((address_space(1))) void *global_address;
+    typedef __attribute__((address_space(3))) void *lds_address;
+    // copy j of 4 per slice and wave: k-row 4 * wave + j, 256 floats = 64 lanes x 16 bytes
+    const float *src[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) src[j] = operand_a + batch * args.a_bs + (i64)(4 * wave + j) * args.a_ld + m0 + 4 * lane;
+    const i64 step_a = (i64)BK_TILE_K * args.a_ld;
+    auto copy_slice = [&](int buffer) {
+        if (lane_copies) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const unsigned to = (unsigned)(unsigned long)(lds_address)(lds_a + (buffer * BK_TILE_K + 4 * wave + j) * SB_TILE_M);
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"((global_address)src[j]), "s"(to) : "memory", "m0");
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) src[j] += step_a;
+    };
+
+    float acc[SB_WAVE_N][4];
+#pragma unroll
+    for (int j = 0; j < SB_WAVE_N; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[j][i] = 0.0f;
+
+    const int k_slices = args.k / BK_TILE_K;
+    const float *b_columns = operand_b + batch * args.b_bs + n0;    // uniform: the loads below are scalar loads
+    copy_slice(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+    __syncthreads();
+    for (int slice = 0; slice < k_slices; slice++) {
+        const int cur = slice & 1;
+        if (slice + 1 < k_slices) copy_slice(cur ^ 1);
+        if (wave_has_columns) {
+            const float *sa = lds_a + cur * BK_TILE_K * SB_TILE_M + 4 * lane;
+            const float *bk = b_columns + (i64)slice * BK_TILE_K * args.b_ld;
+            float fa0[4], fa1[4];
+            scalar_b_fragment(fa0, sa);
+#pragma unroll 1
+            for (int kk = 0; kk < BK_TILE_K; kk += SB_CHUNK) {
+                float sb[SB_CHUNK][SB_WAVE_N];
+#pragma unroll
+                for (int q = 0; q < SB_CHUNK; q++) {
+                    const float4 *row = reinterpret_cast<const float4 *>(bk + (i64)(kk + q) * args.b_ld);
+#pragma unroll
+                    for (int v = 0; v < SB_WAVE_N / 4; v++) {
+                        const float4 x = row[v];
+                        sb[q][4 * v] = x.x; sb[q][4 * v + 1] = x.y; sb[q][4 * v + 2] = x.z; sb[q][4 * v + 3] = x.w;
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < SB_CHUNK; q += 2) {
+                    scalar_b_fragment(fa1, sa + (kk + q + 1) * SB_TILE_M);
+#pragma unroll
+                    for (int j = 0; j < SB_WAVE_N; j += 2) scalar_b_pair<INNER_POW>(acc[j], acc[j + 1], fa0, sb[q][j], sb[q][j + 1]);
+                    scalar_b_fragment(fa0, sa + (kk + q + 2) * SB_TILE_M);       // past the slice on its last k: read, never used
+#pragma unroll
+                    for (int j = 0; j < SB_WAVE_N; j += 2) scalar_b_pair<INNER_POW>(acc[j], acc[j + 1], fa1, sb[q + 1][j], sb[q + 1][j + 1]);
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // this wave's copies of the next slice have landed
+        __syncthreads();
+    }
+    if (!wave_has_columns) return;
+
+    // Epilogue: outer power, epsilon mask, kernel function, regularised diagonal -- finish_tile of build_kernel.hpp on
+    // this kernel's 16 x 4 results per lane.  What depends on the lane's position is derived from a copy of the lane
+    // id that the compiler cannot see through, so that it is not computed before the walk and kept through it.
+    int lane_after = lane;
+    asm volatile("" : "+v"(lane_after));
+    const int outer_power = args.outer_power;
+    const int kernel_type = args.kernel_type;
+    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
+    if (outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
+    if (kernel_type != KERNEL_NONE) {
+        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
+        neg_gamma = kernel_neg_gamma(kernel_type, bw);
+        regularization = args.regularization ? args.regularization[batch * args.regularization_bs] : args.regularization_value;
+    }
+    const float epsilon = args.epsilon;
+    auto for_each = [&](auto &&f) {
+#pragma unroll
+        for (int j = 0; j < SB_WAVE_N; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[j][i] = f(acc[j][i]);
+    };
+    switch (outer_power) {
+    case POW_ABS: for_each([](float v) { return __builtin_fabsf(v); }); break;
+    case POW_SQUARE: for_each([](float v) { return v * v; }); break;
+    case POW_SQRT: for_each([](float v) { return __builtin_amdgcn_sqrtf(v); }); break;
+    case POW_POW: for_each([p_outer](float v) { return exp2f(p_outer * log2f(v)); }); break;
+    default: break;
+    }
+    if (kernel_type != KERNEL_NONE)
+        for_each([epsilon, neg_gamma](float v) { return expf((v < epsilon ? 0.0f : v) * neg_gamma); });
+    const int m_first = m0 + 4 * lane_after;
+    if (kernel_type != KERNEL_NONE && regularization != 0.0f) {
+        const float diagonal_value = 1.0f + regularization;
+#pragma unroll
+        for (int j = 0; j < SB_WAVE_N; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (args.reg_off_x + m_first + i == args.reg_off_y + n0 + j) acc[j][i] = diagonal_value;
+    }
+    // Stores: a wave writes 1 KB of consecutive m for each of its 16 columns.
+    float *c_rows = result + batch * args.c_bs + (i64)n0 * args.c_ld + m_first;
+    if (args.c_vec && m_first + 3 < args.m) {
+#pragma unroll
+        for (int j = 0; j < SB_WAVE_N; j++)
+            *reinterpret_cast<float4 *>(c_rows + (i64)j * args.c_ld) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+    } else {
+#pragma unroll
+        for (int j = 0; j < SB_WAVE_N; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (m_first + i < args.m) c_rows[(i64)j * args.c_ld + i] = acc[j][i];
+    }
+}
+
+}  // namespace kmc

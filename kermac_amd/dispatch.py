@@ -82,6 +82,10 @@ _ROWS = (
      "direct `build_kernel` (ahead of time for DIFF + NOOP/ABS/SQUARE/POW and DOT + NOOP, else compiled on first use); scalar p of 0.5, 1.5, 3, 4 on "
      "the exact-form variants"),
     ("every direct launch",
+     "absolute or squared differences, both operands with m / n contiguous and 16-byte aligned, K and N multiples of 16, K ≥ {DIRECT_SCALAR_B_MIN_K}, "
+     "≥ {DIRECT_SCALAR_B_MIN_TILES} tiles of 256 × 64 in every batch entry, not ranges of one contraction, not a repair launch, not a set against itself",
+     "`build_kernel_scalar_b` (b in scalar registers, only a through LDS; 92 registers, four waves per SIMD)"),
+    ("",
      "both operands with m / n contiguous and 16-byte aligned, K ≥ {DIRECT_FOUR_WAVES_MIN_K}, inner power not fractional, not a repair launch",
      "`build_kernel_four_waves` (128 registers, four waves per SIMD; interior tiles copy their slices straight into LDS)"),
     ("", "otherwise", "`build_kernel` (three waves per SIMD; interior tiles of such operands copy straight into LDS all the same)"),

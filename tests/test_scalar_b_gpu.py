@@ -1,0 +1,109 @@
+"""GPU tests of the direct kernel's variant that keeps the b operand in scalar registers (csrc/kernels/
+build_kernel_scalar_b.hpp): absolute and squared differences of operands whose rows are contiguous, K and N
+multiples of 16.  By its own rule the library launches it from 1800 tiles of 256 x 64 per batch entry and K = 64 on;
+KERMAC_AMD_SCALAR_B_MIN_TILES=1 sends the small shapes of these tests to it.  It sums the terms of every element in
+the order of the ordinary kernel (include/build_a_kernel.cuh:339-370 has one kernel for all shapes), so beside the
+oracle the tests ask for that kernel's bits.
+"""
+import pytest
+import torch
+
+import kermac_amd as kermac
+from oracle import oracle
+from tests.helpers import assert_close_to_truth, l1_distances_float64
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def scalar_b(monkeypatch):
+    monkeypatch.setenv("KERMAC_AMD_SCALAR_B_MIN_TILES", "1")
+    kermac.set_l2_mode("direct")
+    yield monkeypatch
+    kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
+
+
+def panels(M, N, K, device, seed, L=None):
+    g = torch.Generator().manual_seed(seed)
+    shape = (lambda rows: (K, rows)) if L is None else (lambda rows: (L, K, rows))
+    a = torch.randn(shape(M), generator=g).to(device).transpose(-1, -2)
+    b = torch.randn(shape(N), generator=g).to(device).transpose(-1, -2)
+    return a, b
+
+
+def ordinary(monkeypatch, call):
+    monkeypatch.delenv("KERMAC_AMD_SCALAR_B_MIN_TILES")
+    try:
+        return call()
+    finally:
+        monkeypatch.setenv("KERMAC_AMD_SCALAR_B_MIN_TILES", "1")
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 64, 16), (300, 80, 32), (1000, 912, 64), (257, 16, 48), (3, 160, 16), (1, 16, 1024),
+                                   (515, 1040, 208), (1024, 1024, 256), (2047, 2000, 1040)])
+@pytest.mark.parametrize("p", [1.0, 2.0])
+def test_matches_truth_and_the_ordinary_kernel(device, scalar_b, M, N, K, p):
+    a, b = panels(M, N, K, device, 7 * M + N + K)
+    out = torch.empty(N, M, device=device).t()
+    got = kermac.cdist(a, b, out=out, p=p)
+    truth = l1_distances_float64(a, b) if p == 1.0 else torch.cdist(a.double(), b.double(), p=2.0, compute_mode="donot_use_mm_for_euclid_dist")
+    assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-30, what=f"p={p} {M}x{N}x{K}")
+    plain = ordinary(scalar_b, lambda: kermac.cdist(a, b, p=p))
+    assert torch.equal(got, plain.reshape(got.shape)), "not the ordinary kernel's bits"
+
+
+def test_it_is_the_kernel_that_ran(device, scalar_b):
+    """Shapes the kernel cannot take (N or K not a multiple of 16, a set against itself, rows not contiguous) run the
+    ordinary kernels and give the same numbers; a misaligned operand does too."""
+    for M, N, K in ((300, 81, 32), (300, 80, 40), (128, 128, 24)):
+        a, b = panels(M, N, K, device, M + N + K)
+        truth = l1_distances_float64(a, b)
+        assert_close_to_truth(kermac.cdist(a, b, p=1.0)[0], truth, rtol=1e-5, what=f"{M}x{N}x{K}")
+    a, b = panels(400, 400, 64, device, 3)
+    assert_close_to_truth(kermac.cdist(a, a, p=1.0)[0], l1_distances_float64(a, a), rtol=1e-5, atol=1e-30, what="a against itself")
+    rows = a.contiguous()
+    assert_close_to_truth(kermac.cdist(rows, b, p=1.0)[0], l1_distances_float64(a, b), rtol=1e-5, what="k contiguous")
+    store = torch.randn(64 * 404 + 1, device=device)[1:].view(64, 404)
+    odd = store[:, :400].t()
+    assert_close_to_truth(kermac.cdist(odd, b, p=1.0)[0], l1_distances_float64(odd, b), rtol=1e-5, what="misaligned a")
+
+
+def test_kernel_functions_batches_and_offsets(device, scalar_b):
+    """Laplace and Gaussian kernels with a regularised off-diagonal, a batch with a broadcast operand and per-entry
+    bandwidths, a result with padded rows; against the oracle and the ordinary kernel."""
+    L, M, N, K = 3, 520, 336, 48
+    a, _ = panels(M, N, K, device, 11, L=L)
+    _, b = panels(M, N, K, device, 12)
+    bandwidth = torch.tensor([3.0, 7.0, 1.5], device=device)
+    store = torch.empty(L, N, M + 4, device=device)
+    out = store[:, :, :M].transpose(1, 2)
+    for descriptor, names in ((kermac.kernel_descriptor_laplace_l1, ("DIFF", "ABS", "NOOP", "LAPLACE")),
+                              (kermac.kernel_descriptor_laplace_l2, ("DIFF", "SQUARE", "SQRT", "LAPLACE"))):
+        got = kermac.run_kernel(descriptor, a, b, out=out, bandwidth=bandwidth, regularization=0.25,
+                                regularization_offset_x=3, regularization_offset_y=1)
+        truth = oracle.run_kernel(*names, a.cpu(), b.cpu(), bandwidth=bandwidth.cpu(), regularization=0.25,
+                                  regularization_offset_x=3, regularization_offset_y=1)
+        assert_close_to_truth(got, truth, rtol=1e-5, atol=1e-7, what=str(descriptor))
+        plain = ordinary(scalar_b, lambda: kermac.run_kernel(descriptor, a, b, bandwidth=bandwidth, regularization=0.25,
+                                                             regularization_offset_x=3, regularization_offset_y=1))
+        assert torch.equal(got, plain)
+    gaussian = kermac.KernelDescriptor(kermac.InnerOperator.DIFF, kermac.PowerType.SQUARE, kermac.PowerType.NOOP, kermac.KernelType.GAUSSIAN)
+    got = kermac.run_kernel(gaussian, a[0], b, bandwidth=4.0)
+    plain = ordinary(scalar_b, lambda: kermac.run_kernel(gaussian, a[0], b, bandwidth=4.0))
+    assert torch.equal(got, plain)
+
+
+def test_a_large_problem_takes_the_kernel_by_itself(device):
+    """16384 x 16384 x 256 is 16384 tiles of 256 x 64: the library's own rule.  Float64 slabs, and the rows and columns at
+    the edges of a ragged problem of the same size."""
+    with kermac.l2_mode("direct"):
+        for M, N in ((16384, 16384), (16000 + 37, 16000)):
+            a, b = panels(M, N, 256, device, 5)
+            out = torch.empty(N, M, device=device).t()
+            for p in (1.0, 2.0):
+                kermac.cdist(a, b, out=out, p=p)
+                rows = torch.cat([torch.arange(0, 96), torch.arange(M - 64, M)]).to(device)
+                columns = torch.cat([torch.arange(0, 64), torch.arange(N - 80, N)]).to(device)
+                x, y = a[rows], b[columns]
+                truth = l1_distances_float64(x, y) if p == 1.0 else torch.cdist(x.double(), y.double(), p=2.0, compute_mode="donot_use_mm_for_euclid_dist")
+                assert_close_to_truth(out[rows][:, columns], truth, rtol=1e-5, what=f"p={p} {M}x{N}")
