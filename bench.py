@@ -687,7 +687,7 @@ def main():
     achieved = OPS_PER_CALL / kernel_ms / 1e9
     traffic, traffic_source = measured_traffic() if headline_p == 1.0 and kermac.get_l1_mode() == "direct" else (None, None)
     inner = {1.0: "POW_ABS", 2.0: "POW_SQUARE"}.get(headline_p, "POW_POW")
-    headline_kernel = (f"kmc::build_kernel_four_waves<OP_DIFF,{inner}>" if inner != "POW_POW"
+    headline_kernel = (f"kmc::build_kernel_scalar_b<OP_DIFF,{inner}>" if inner != "POW_POW"
                        else f"kmc::build_kernel<OP_DIFF,{inner},LOAD_COL_VEC,LOAD_COL_VEC>")
     if headline_p == 1.0 and kermac.get_l1_mode() == "fixed":
         headline_kernel = "kmc::l1_fixed_kernel (l1 mode fixed)"

@@ -26,6 +26,7 @@
 #include <cstring>
 
 #include "kermac_amd/csrc/kernels/build_kernel.hpp"
+#include "kermac_amd/csrc/kernels/build_kernel_scalar_b.hpp"
 
 #define CHECK(x) \
     do { \
@@ -499,6 +500,8 @@ int walk_ablations()
     kmc::BuildKernelArgs d = {};
     d.m = M; d.n = N; d.k = K; d.l = 1; d.a = a; d.a_ld = Mp; d.b = b; d.b_ld = Np; d.c = c; d.c_ld = M;
     d.diff_sign = 1.0f; d.c_vec = 1; d.tiles_m = tiles_m; d.tiles_n = tiles_n; d.tiles_n_padded = tiles_n_padded; d.grid_width = grid.x;
+    const dim3 scalar_b_grid(((M + kmc::SB_TILE_M - 1) / kmc::SB_TILE_M) * ((N + kmc::SB_TILE_N - 1) / kmc::SB_TILE_N));
+    run("product kernel build_kernel_scalar_b<DIFF, ABS> (b in scalar registers)", [&] { kmc::build_kernel_scalar_b<kmc::OP_DIFF, kmc::POW_ABS><<<scalar_b_grid, 256>>>(d, a, b, c); }, clocks, reps);
     run("product kernel build_kernel_four_waves<DIFF, ABS>", [&] { kmc::build_kernel_four_waves<kmc::OP_DIFF, kmc::POW_ABS><<<grid, 256>>>(d); }, clocks, reps);
     run("product kernel at three waves per SIMD, build_kernel<DIFF, ABS>", [&] { kmc::build_kernel<kmc::OP_DIFF, kmc::POW_ABS, kmc::LOAD_COL_VEC, kmc::LOAD_COL_VEC><<<grid, 256>>>(d); }, clocks, reps);
     run("same walk, clocks read (all traffic)", [&] { walk_variant<false, false, false, false><<<grid, 256>>>(d, clocks); }, clocks, reps);
@@ -517,6 +520,7 @@ int walk_ablations()
     run("the same, 3 waves per SIMD", [&] { walk_direct_to_lds<3><<<grid, 256>>>(d, clocks); }, clocks, reps);
     run("the same, 2 waves per SIMD", [&] { walk_direct_to_lds<2><<<grid, 256>>>(d, clocks); }, clocks, reps);
     run("product kernel build_kernel_four_waves<DIFF, ABS> again", [&] { kmc::build_kernel_four_waves<kmc::OP_DIFF, kmc::POW_ABS><<<grid, 256>>>(d); }, clocks, reps);
+    run("product kernel build_kernel_scalar_b<DIFF, ABS> again", [&] { kmc::build_kernel_scalar_b<kmc::OP_DIFF, kmc::POW_ABS><<<scalar_b_grid, 256>>>(d, a, b, c); }, clocks, reps);
     float direct_element;
     CHECK_VOID(hipMemcpy(&direct_element, c + (size_t)12345 * M + 6789, 4, hipMemcpyDeviceToHost));
     printf("one element from the walk with direct copies %.6f\n", direct_element);
