@@ -29,6 +29,10 @@ constexpr int SB_TILE_M = 256;      // 64 lanes x 4 rows
 constexpr int SB_WAVE_N = 16;       // columns of a wave: 16 scalars per k
 constexpr int SB_TILE_N = 4 * SB_WAVE_N;
 constexpr int SB_CHUNK = 4;         // k per group of scalar loads (64 scalar registers)
+#ifndef KMC_SB_XCD_ROWS
+#define KMC_SB_XCD_ROWS 2
+#endif
+constexpr int SB_XCD_ROWS = KMC_SB_XCD_ROWS;   // row blocks of a that one XCD works on at a time
 
 // Two columns at a time: 8 independent subtractions (scalar minus vector), then 8 independent accumulations, as
 // in row_abs_diff / row_square_diff of build_kernel.hpp.
@@ -77,9 +81,33 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
     const int tid = threadIdx.x;
     const int batch = blockIdx.y;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // consecutive workgroups walk n: the ~128 of them resident on an XCD share one or two row blocks of a through its L2
+    // Tile order.  The hardware deals workgroups to the 8 XCDs round-robin by their launch-wide id.  Bands of 8 row
+    // blocks of a: inside a band XCD x owns row block x and walks n, so the ~128 workgroups resident on an XCD share ONE
+    // 1 MB panel of a through its L2 (which the b panels streaming past cannot push out), and the 8 XCDs ask for the same
+    // b panel at about the same time.  The row blocks that do not fill a band are walked n fastest across all XCDs:
+    // a band of fewer than 8 would leave XCDs idle for its whole length.
     const int tiles_n = (args.n + SB_TILE_N - 1) / SB_TILE_N;
-    const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x - tile_m * tiles_n;
+    int tile_m, tile_n;
+    {
+        constexpr int band_rows = 8 * SB_XCD_ROWS;
+        const int banded_rows = ((args.m + SB_TILE_M - 1) / SB_TILE_M) / band_rows * band_rows;
+        const int banded = banded_rows * tiles_n;                    // a multiple of 8
+        const int id = blockIdx.x;
+        if (id < banded) {
+            // the XCD of this workgroup: gridDim.x * blockIdx.y + id mod 8 -- a permutation of every 8 consecutive ids
+            const int xcd = (id + (int)((gridDim.x % 8u) * (blockIdx.y % 8u))) & 7;
+            const int sequence = id >> 3;                            // position in that XCD's queue
+            const int band = sequence / (SB_XCD_ROWS * tiles_n);
+            const int in_band = sequence - band * (SB_XCD_ROWS * tiles_n);
+            tile_n = in_band / SB_XCD_ROWS;
+            tile_m = band * band_rows + xcd * SB_XCD_ROWS + (in_band - tile_n * SB_XCD_ROWS);
+        } else {
+            const int rest = id - banded;
+            const int row = rest / tiles_n;
+            tile_n = rest - row * tiles_n;
+            tile_m = banded_rows + row;
+        }
+    }
     const int m0 = tile_m * SB_TILE_M;
     const int n0 = tile_n * SB_TILE_N + SB_WAVE_N * wave;        // uniform over the wave
     const int m_valid = args.m - m0;
