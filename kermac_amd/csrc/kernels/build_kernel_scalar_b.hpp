@@ -10,8 +10,7 @@
 // memory by global_load_lds_dwordx4, 1 KB per k-row of the 256 x 64 tile).  Workgroup 4 waves = 256 (m) x 64 (n),
 // 92 registers, 33 KB of LDS, four workgroups per CU.  Measured on the walk alone, same box, M = N = 30000,
 // K = 1024: 27.4 ms against 28.3 ms for build_kernel_four_waves (8 waves per workgroup on 256 x 128: 28.7; the
-// 8 x 8 lane tile with b in scalar registers, 512 x 64: 28.4; five waves per SIMD: 27.6; tile order in bands of
-// 8 tile rows: 28.0).
+// 8 x 8 lane tile with b in scalar registers, 512 x 64: 28.4; five waves per SIMD: 27.6).
 //
 // What the host guarantees before it launches this kernel (build_kernel_inst.hip): both operands with rows
 // contiguous and 16-byte aligned (the LOAD_COL_VEC loaders), K a multiple of 16, N a multiple of 16 (a wave's 16
@@ -29,10 +28,7 @@ constexpr int SB_TILE_M = 256;      // 64 lanes x 4 rows
 constexpr int SB_WAVE_N = 16;       // columns of a wave: 16 scalars per k
 constexpr int SB_TILE_N = 4 * SB_WAVE_N;
 constexpr int SB_CHUNK = 4;         // k per group of scalar loads (64 scalar registers)
-#ifndef KMC_SB_XCD_ROWS
-#define KMC_SB_XCD_ROWS 2
-#endif
-constexpr int SB_XCD_ROWS = KMC_SB_XCD_ROWS;   // row blocks of a that one XCD works on at a time
+constexpr int SB_XCD_ROWS = 2;      // row blocks of a that one XCD works on at a time
 
 // Two columns at a time: 8 independent subtractions (scalar minus vector), then 8 independent accumulations, as
 // in row_abs_diff / row_square_diff of build_kernel.hpp.
@@ -81,11 +77,14 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
     const int tid = threadIdx.x;
     const int batch = blockIdx.y;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Tile order.  The hardware deals workgroups to the 8 XCDs round-robin by their launch-wide id.  Bands of 8 row
-    // blocks of a: inside a band XCD x owns row block x and walks n, so the ~128 workgroups resident on an XCD share ONE
-    // 1 MB panel of a through its L2 (which the b panels streaming past cannot push out), and the 8 XCDs ask for the same
-    // b panel at about the same time.  The row blocks that do not fill a band are walked n fastest across all XCDs:
-    // a band of fewer than 8 would leave XCDs idle for its whole length.
+    // Tile order.  The hardware deals workgroups to the 8 XCDs round-robin by their launch-wide id.  Bands of 16 row
+    // blocks of a: inside a band XCD x owns row blocks 2x and 2x + 1 and walks n with the row block fastest, so the ~128
+    // workgroups resident on an XCD share 2 MB of a through its L2, and the two workgroups that stream the same b panel
+    // (by scalar loads, which nothing but the L2 can share) run side by side: the second finds it there.  Measured at
+    // M = N = 30000, K = 1024: 19 GB fetched from memory per launch against 31 GB with n fastest over the whole launch
+    // or one row block per XCD, and 19.7 GB with three (3 MB of a no longer stay in a 4 MB L2 beside the stream).
+    // The row blocks that do not fill a band are walked n fastest across all XCDs: a band of fewer than 16 would
+    // leave XCDs idle for its whole length.
     const int tiles_n = (args.n + SB_TILE_N - 1) / SB_TILE_N;
     int tile_m, tile_n;
     {

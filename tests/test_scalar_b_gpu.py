@@ -52,6 +52,27 @@ def test_matches_truth_and_the_ordinary_kernel(device, scalar_b, M, N, K, p):
     assert torch.equal(got, plain.reshape(got.shape)), "not the ordinary kernel's bits"
 
 
+@pytest.mark.parametrize("M,N,K,L", [(256 * 15 + 9, 320, 16, None), (256 * 16, 336, 32, None), (256 * 17 + 100, 64 * 7 + 16, 16, None),
+                                     (256 * 35 + 1, 208, 16, None), (256 * 33, 64 * 3, 32, 3), (256 * 18 + 77, 64 * 5 + 48, 16, 5)])
+def test_every_tile_of_the_band_order_is_walked_once(device, scalar_b, M, N, K, L):
+    """Row blocks of a in bands of 16 (two per XCD) and the row blocks that fill no band, with and without a batch
+    whose grid width shifts the XCD of a workgroup from entry to entry: the result is filled with NaN first, and every
+    element is the ordinary kernel's."""
+    a, b = panels(M, N, K, device, M + N + K, L=L)
+    shape = (N, M) if L is None else (L, N, M)
+    out = torch.full(shape, float("nan"), device=device).transpose(-1, -2)
+    got = kermac.cdist(a, b, out=out, p=1.0)
+    assert not torch.isnan(got).any(), "tiles left out"
+    plain = ordinary(scalar_b, lambda: kermac.cdist(a, b, p=1.0))
+    assert torch.equal(got, plain.reshape(got.shape)), "not the ordinary kernel's bits"
+    sample = slice(0, M, 97)
+    if L is None:
+        truth = l1_distances_float64(a[sample], b)
+    else:
+        truth = torch.stack([l1_distances_float64(a[entry, sample], b[entry]) for entry in range(L)])
+    assert_close_to_truth(got[..., sample, :], truth, rtol=1e-5, atol=1e-30, what=f"{M}x{N}x{K}x{L}")
+
+
 def test_it_is_the_kernel_that_ran(device, scalar_b):
     """Shapes the kernel cannot take (N or K not a multiple of 16, a set against itself, rows not contiguous) run the
     ordinary kernels and give the same numbers; a misaligned operand does too."""
