@@ -151,7 +151,21 @@ enum kmc_flags {
      * instead of 6 + 32; at 2048 x 2048 x 1024 0.19 instead of 0.37 ms).  Pairs packed into few tiles
      * (points stored cluster by cluster) leave the call on the matrix cores.  This flag leaves the
      * sample out: every part is multiplied, checked and, if need be, recomputed. */
-    KMC_FLAG_NO_PROBE = 1024
+    KMC_FLAG_NO_PROBE = 1024,
+    /* kmc_build_kernel, inner_operator DIFF with inner_power ABS or SQUARE on the direct kernel (none of the
+     * flags above), with gram_workspace: the fastest direct kernel for large problems (b in scalar registers)
+     * takes its operands as k-major panels (rows contiguous, 16-byte aligned, k a multiple of 16, n a multiple
+     * of 16).  With this flag the library copies operands stored any other way -- k contiguous as torch
+     * allocates them, misaligned views, other k or n -- into such panels in the workspace (padded with zeros:
+     * a zero in both operands adds nothing to a sum, padded columns are not stored) and runs that kernel on
+     * the copies: one read and one write of each copied operand against 5 to 7 % of the kernel's time.  The
+     * sums are the direct kernel's bit for bit.  kmc_gram_workspace_bytes says which calls take the route
+     * (5400 tiles of 256 x 64 per batch entry, k >= 64, an operand that needs a copy, not a panel against
+     * itself, 16-byte aligned c; KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE: any size) and how much memory it wants
+     * (4 bytes per element of the padded copies).  Without a workspace, or for a call the query reports 0
+     * for, the direct kernels run on the operands as they are.  The reference has one kernel for all
+     * storage orders (include/build_a_kernel.cuh:484-539). */
+    KMC_FLAG_DIRECT_PANELS = 2048
 };
 
 /*

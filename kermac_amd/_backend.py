@@ -30,8 +30,11 @@ COL_MAJOR = 0
 ROW_MAJOR = 1
 
 # enum kmc_inner_operator, enum kmc_power_type (the values the Python mirror tests for)
+OP_DIFF = 0
 OP_DOT = 1
 POW_NOOP = 0
+POW_ABS = 1
+POW_SQUARE = 2
 
 FLAG_FORCE_SCALAR_ACCESS = 1
 FLAG_NEGATE_DIFF = 2
@@ -44,6 +47,7 @@ FLAG_DOT_PIECES = 128
 FLAG_GRAM_WORKSPACE_ANY_SIZE = 256
 FLAG_L1_FIXED = 512
 FLAG_NO_PROBE = 1024
+FLAG_DIRECT_PANELS = 2048
 SAMPLE_BYTES = 1024             # KMC_SAMPLE_BYTES: what the sample in front of a matrix-core launch takes of the workspace
 
 _float_p = c_void_p  # device pointers are passed as integers

@@ -55,7 +55,7 @@ EXTRA_DEVICE_SOURCES = ["kernels/norm_gradient_inst.hip", "kernels/gram_kernel_i
                         "kernels/gram_coefficients_inst.hip", "kernels/gram_bf16_kernel_inst.hip",
                         "kernels/finish_partials.hip", "kernels/cut_static_scratch.hip", "kernels/sample_mean.hip", "kernels/gram_probe.hip",
                         "kernels/gram_f16_wide_inst.hip", "kernels/norm_gradient_f16_inst.hip",
-                        "kernels/matrix_times_coefficients.hip", "kernels/l1_fixed_inst.hip"]
+                        "kernels/matrix_times_coefficients.hip", "kernels/l1_fixed_inst.hip", "kernels/panel_copy.hip"]
 
 
 def _hipcc() -> str:

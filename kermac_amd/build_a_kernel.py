@@ -640,6 +640,18 @@ def run_kernel(
     if params.flags & (_backend.FLAG_L2_GRAM | _backend.FLAG_L2_GRAM_BF16):
         plan.keepalive.append(_attach_gram_centre(params, stream, a.device))
         plan.keepalive.append(_attach_gram_workspace(params, a.device))
+    elif (cut is None and not params.flags & (_backend.FLAG_DOT_PIECES | _backend.FLAG_L1_FIXED)
+            and params.inner_operator == _backend.OP_DIFF and params.inner_power in (_backend.POW_ABS, _backend.POW_SQUARE)):
+        # absolute and squared differences on the direct kernel: large problems whose operands its fastest
+        # variant cannot take as they are (k contiguous, as torch allocates them; K or N not multiples of 16) run
+        # on copies that it can, when the library wants room for them (include/kermac_amd.h, KMC_FLAG_DIRECT_PANELS)
+        params.flags |= _backend.FLAG_DIRECT_PANELS
+        if os.environ.get("KERMAC_AMD_DIRECT_PANELS_ANY_SIZE", "0") not in ("", "0"):
+            params.flags |= _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE      # tests send small shapes down the route
+        workspace = _attach_gram_workspace(params, a.device, switch="KERMAC_AMD_DIRECT_PANELS")
+        if workspace is None:
+            params.flags &= ~(_backend.FLAG_DIRECT_PANELS | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE)
+        plan.keepalive.append(workspace)
     if cut is None:
         launch(params)
     else:

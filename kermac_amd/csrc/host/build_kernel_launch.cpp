@@ -110,6 +110,7 @@ int prepare(const kmc_build_kernel_params *p, bool need_c, kmc::BuildKernelArgs 
     args->centre = nullptr;
     args->centre_bs = 0;
     args->sample = nullptr;
+    args->panels = 0;
     if ((p->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16)) && p->gram_centre) {
         if (!aligned16(p->gram_centre) || p->gram_centre_bs % 4 != 0 || p->gram_centre_bs < 0)
             return fail(KMC_ERR_INVALID_ARGUMENT, "gram_centre must be 16-byte aligned with a batch stride that is a multiple of 4");
@@ -148,6 +149,8 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
 hipError_t launch_gram_probe(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, unsigned *sample, hipStream_t stream);
 int64_t l1_fixed_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
 hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
+int64_t direct_panels_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
+hipError_t launch_direct_panels(const kmc_build_kernel_params *p, kmc::BuildKernelArgs *args, hipStream_t stream, bool *taken);
 hipError_t launch_finish_partials(const kmc::BuildKernelArgs &kernel, const float *partials, int64_t partial_ld,
                                   int64_t partial_bs, int64_t partial_slice, int slices, int vec, hipStream_t stream);
 }
@@ -191,6 +194,7 @@ int kmc_gram_workspace_bytes(const kmc_build_kernel_params *params, int64_t *byt
     if (status != KMC_OK) return status;
     *bytes = gram_f16_wide_bytes(&asked, args);
     if (*bytes == 0) *bytes = l1_fixed_bytes(&asked, args);
+    if (*bytes == 0) *bytes = direct_panels_bytes(&asked, args);
     return KMC_OK;
 }
 
@@ -261,6 +265,14 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
         hipError_t g = launch_l1_fixed(params, args, static_cast<hipStream_t>(stream), &fixed);
         if (g != hipSuccess) return fail_hip(g, "l1_fixed launches");
         if (fixed) args.repair_only = 1;
+    }
+    if (params->flags & KMC_FLAG_DIRECT_PANELS) {
+        // Large absolute- and squared-difference problems whose operands the kernel with b in scalar registers cannot
+        // take as they are: copies that it can (panel_copy.hip), then the ordinary launch on the copies.
+        bool copied = false;
+        hipError_t g = launch_direct_panels(params, &args, static_cast<hipStream_t>(stream), &copied);
+        if (g != hipSuccess) return fail_hip(g, "panel_copy launches");
+        if (copied) load_a = load_b = kmc::LOAD_COL_VEC;
     }
     hipError_t e = launch(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail_hip(e, "build_kernel launch");

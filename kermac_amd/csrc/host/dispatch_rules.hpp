@@ -38,6 +38,9 @@
     /* tiles of 256 x 64 in every batch entry */                                                         \
     X(DIRECT_SCALAR_B_MIN_TILES, 1800)                                                                  \
     X(DIRECT_SCALAR_B_MIN_K, 64)                                                                        \
+    /* ... on copies of operands in any other storage (KMC_FLAG_DIRECT_PANELS): the same tiles, per batch entry */ \
+    X(DIRECT_PANELS_MIN_TILES, 5400)                                                                    \
+    X(DIRECT_PANELS_MIN_K, 64)                                                                          \
     /* absolute differences on fixed point (KMC_FLAG_L1_FIXED): tiles of 128 x 128 over the batch */    \
     X(L1_FIXED_MIN_TILES, 2048)                                                                         \
     X(L1_FIXED_MIN_K, 128)                                                                              \

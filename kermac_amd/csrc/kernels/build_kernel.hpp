@@ -58,7 +58,14 @@ struct BuildKernelArgs {
     // Matrix-core kernels for squared differences only, or null: what a sample of the result said before the
     // launch (gram_probe.hip fills it, sample_leaves_it_to_the_direct_kernel reads it).
     const unsigned *sample;
+    // build_kernel_scalar_b only.  BK_PANELS_COPIED: the operands are the copies of panel_copy.hip, made for that
+    // kernel, which therefore runs whatever the size of the problem.  BK_PANELS_B_PADDED: the rows of b hold n rounded
+    // up to 16 columns (zeros past n), so that a wave's 16 columns can always be loaded; columns below n are stored.
+    int panels;
 };
+
+constexpr int BK_PANELS_COPIED = 1;
+constexpr int BK_PANELS_B_PADDED = 2;
 
 constexpr int GRAM_CENTRE_PAD = 64;
 

@@ -30,12 +30,13 @@ namespace kmc_host {
 // call, so that a test can send small shapes to the kernel).
 static bool scalar_b_applies(const kmc::BuildKernelArgs &args, int64_t *tiles_m, int64_t *tiles_n)
 {
-    if (args.k < 16 || args.k % kmc::BK_TILE_K != 0 || args.n % kmc::SB_WAVE_N != 0 || args.k_total != 0 || args.repair_only || args.symmetric)
+    if (args.k < 16 || args.k % kmc::BK_TILE_K != 0 || (args.n % kmc::SB_WAVE_N != 0 && !(args.panels & kmc::BK_PANELS_B_PADDED)) || args.k_total != 0 || args.repair_only || args.symmetric)
         return false;
     *tiles_m = (static_cast<int64_t>(args.m) + kmc::SB_TILE_M - 1) / kmc::SB_TILE_M;
     *tiles_n = (static_cast<int64_t>(args.n) + kmc::SB_TILE_N - 1) / kmc::SB_TILE_N;
     const int64_t tiles = *tiles_m * *tiles_n;
     if (tiles > 0x7fffffff) return false;
+    if (args.panels & kmc::BK_PANELS_COPIED) return true;       // the host made the copies for this kernel
     const char *text = std::getenv("KERMAC_AMD_SCALAR_B_MIN_TILES");
     const int forced = text ? std::atoi(text) : 0;
     if (forced > 0) return tiles * args.l >= forced;

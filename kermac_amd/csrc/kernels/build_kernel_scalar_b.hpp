@@ -13,9 +13,10 @@
 // 8 x 8 lane tile with b in scalar registers, 512 x 64: 28.4; five waves per SIMD: 27.6).
 //
 // What the host guarantees before it launches this kernel (build_kernel_inst.hip): both operands with rows
-// contiguous and 16-byte aligned (the LOAD_COL_VEC loaders), K a multiple of 16, N a multiple of 16 (a wave's 16
-// columns exist or do not), no ranges of one contraction (k_total = 0), not a repair launch, not the triangle of
-// a symmetric result.  The last tile row may be ragged in m: lanes beyond M copy nothing and store nothing.
+// contiguous and 16-byte aligned (the LOAD_COL_VEC loaders), K a multiple of 16, N a multiple of 16 or b a copy
+// whose rows are padded to one (a wave's 16 columns can be loaded or do not exist; panel_copy.hip makes such copies
+// of operands in any other storage), no ranges of one contraction (k_total = 0), not a repair launch, not the triangle
+// of a symmetric result.  The last tile row may be ragged in m: lanes beyond M copy nothing and store nothing.
 // Results are those of build_kernel bit for bit: every element sums its terms over k in the same order.
 // The reference has one kernel for all shapes (include/build_a_kernel.cuh:339-462).
 #pragma once
@@ -110,7 +111,8 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
     const int m0 = tile_m * SB_TILE_M;
     const int n0 = tile_n * SB_TILE_N + SB_WAVE_N * wave;        // uniform over the wave
     const int m_valid = args.m - m0;
-    const bool wave_has_columns = n0 < args.n;                   // all 16 or none: n is a multiple of 16
+    const bool wave_has_columns = n0 < args.n;                   // all 16 can be loaded: n is a multiple of 16, or b a padded copy
+    const int columns = args.n - n0 < SB_WAVE_N ? args.n - n0 : SB_WAVE_N;     // ... and these are stored
     const bool lane_copies = 4 * lane < m_valid;                 // the 16 bytes lie inside the row: its length is a multiple of 4 floats
 
     typedef const __attribute__((address_space(1))) void *global_address;
@@ -223,13 +225,13 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
     if (args.c_vec && m_first + 3 < args.m) {
 #pragma unroll
         for (int j = 0; j < SB_WAVE_N; j++)
-            *reinterpret_cast<float4 *>(c_rows + (i64)j * args.c_ld) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+            if (j < columns) *reinterpret_cast<float4 *>(c_rows + (i64)j * args.c_ld) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
     } else {
 #pragma unroll
         for (int j = 0; j < SB_WAVE_N; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                if (m_first + i < args.m) c_rows[(i64)j * args.c_ld + i] = acc[j][i];
+                if (j < columns && m_first + i < args.m) c_rows[(i64)j * args.c_ld + i] = acc[j][i];
     }
 }
 

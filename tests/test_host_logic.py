@@ -611,6 +611,35 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     monkeypatch.setenv("KERMAC_AMD_GRADIENT_F16_MIN_TERMS", "1")
     assert gradient(3, 2, 1, 5) > 0
 
+    def panels(m, n, k, l=1, power=1, flags=_backend.FLAG_DIRECT_PANELS, k_contiguous=(True, True), same=False, misaligned=False):
+        params = _backend.BuildKernelParams()
+        params.inner_operator, params.inner_power, params.outer_power = 0, power, 0
+        params.m, params.n, params.k, params.l = m, n, k, l
+        params.a, params.a_ld, params.a_bs = fake + (4 if misaligned else 0), (k if k_contiguous[0] else m), m * k
+        params.b, params.b_ld, params.b_bs = (params.a if same else fake + 4 * m * k * l), (k if k_contiguous[1] else n), n * k
+        params.a_majorness = _backend.ROW_MAJOR if k_contiguous[0] else _backend.COL_MAJOR
+        params.b_majorness = _backend.ROW_MAJOR if k_contiguous[1] else _backend.COL_MAJOR
+        params.c_ld, params.c_bs = m, m * n
+        params.flags = flags
+        return _backend.gram_workspace_bytes(params)
+
+    # copies of the operands for the direct kernel with b in scalar registers: 5400 tiles of 256 x 64 per batch entry,
+    # k >= 64, absolute or squared differences, an operand the kernel cannot take as it is; 4 bytes per padded element
+    assert panels(30000, 30000, 1024) == 2 * 1024 * 30016 * 4
+    assert panels(30000, 30000, 1024, power=2) == panels(30000, 30000, 1024) and panels(30000, 30000, 1024, power=4) == 0
+    assert panels(30000, 30000, 1024, k_contiguous=(False, False)) == 0             # the kernel takes these by itself
+    assert panels(30000, 30000, 1024, k_contiguous=(False, True)) == 1024 * 30016 * 4
+    assert panels(30000, 30008, 1024, k_contiguous=(False, False)) == 1024 * 30016 * 4        # n not a multiple of 16: b
+    assert panels(30000, 30000, 1000, k_contiguous=(False, False)) == 2 * 1008 * 30016 * 4    # k not a multiple of 16: both
+    assert panels(30000, 30000, 1024, k_contiguous=(False, False), misaligned=True) == 1024 * 30016 * 4
+    assert panels(10000, 10000, 1024) > 0 and panels(9000, 9000, 1024) == 0         # 6280 and 5076 tiles
+    assert panels(9000, 9000, 1024, l=4) == 0                                       # per batch entry
+    assert panels(30000, 30000, 48) == 0
+    assert panels(30000, 30000, 1024, same=True) == 0                               # a set against itself: half the tiles instead
+    assert panels(30000, 30000, 1024, flags=0) == 0
+    assert panels(30000, 30000, 1024, flags=_backend.FLAG_DIRECT_PANELS | _backend.FLAG_L1_FIXED) == absolute_differences(30000, 30000, 1024)   # that route's own
+    assert panels(300, 200, 5, flags=_backend.FLAG_DIRECT_PANELS | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE) == 16 * (320 + 256) * 4
+
 
 def test_auto_mode_of_the_coefficient_product_without_a_gpu(monkeypatch):
     """l2 mode "auto", run_kernel(..., coefficients=...) of squared differences: panels where the
