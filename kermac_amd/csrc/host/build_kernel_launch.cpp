@@ -145,7 +145,9 @@ namespace kmc_host {
 hipError_t launch_gram_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
 hipError_t launch_gram_bf16_l2(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream);
 int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
-hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
+hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken,
+                                const unsigned **sample = nullptr);
+hipError_t launch_scalar_b_if_the_sample_leaves(int load_a, int load_b, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *launched);
 hipError_t launch_gram_probe(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, unsigned *sample, hipStream_t stream);
 int64_t l1_fixed_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args);
 hipError_t launch_l1_fixed(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken);
@@ -238,8 +240,10 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
             return fail(KMC_ERR_INVALID_ARGUMENT, "KMC_FLAG_L2_GRAM needs inner_operator DIFF and inner_power SQUARE");
         // Matrix-core pass over every tile, then the direct kernel over the tiles it marked.
         bool wide = false;
-        hipError_t g = launch_gram_f16_wide(params, args, static_cast<hipStream_t>(stream), &wide);
+        const unsigned *sample_taken = nullptr;
+        hipError_t g = launch_gram_f16_wide(params, args, static_cast<hipStream_t>(stream), &wide, &sample_taken);
         if (g != hipSuccess) return fail_hip(g, "gram_f16_wide launches");
+        if (wide) args.sample = sample_taken;
         if (!wide) {
             // The one-step kernels: with KMC_SAMPLE_BYTES of workspace, a sample of the result first (gram_probe.hip),
             // so that data whose near-duplicates sit in every tile costs the direct kernel's time, not both.
@@ -254,6 +258,14 @@ int kmc_build_kernel(const kmc_build_kernel_params *params, void *stream)
                     ? launch_gram_bf16_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream))
                     : launch_gram_l2(load_a, load_b, args, grid, static_cast<hipStream_t>(stream));
             if (g != hipSuccess) return fail_hip(g, "gram_l2_kernel launch");
+        }
+        if (args.sample) {
+            // Where the sample left the call to the direct kernel, its fastest variant does the work (if it can take
+            // these operands), and the repair launch behind it finds nothing to do.
+            bool launched = false;
+            g = launch_scalar_b_if_the_sample_leaves(load_a, load_b, args, static_cast<hipStream_t>(stream), &launched);
+            if (g != hipSuccess) return fail_hip(g, "build_kernel_scalar_b launch");
+            args.sample = nullptr;
         }
         args.repair_only = 1;
     }

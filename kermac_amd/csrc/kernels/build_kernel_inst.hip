@@ -52,6 +52,7 @@ static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStr
         int64_t tiles_m = 0, tiles_n = 0;
         if (scalar_b_applies(args, &tiles_m, &tiles_n)) {
             kmc::BuildKernelArgs copy = args;
+            copy.sample = nullptr;          // an ordinary launch computes everything
             const float *a = args.a, *b = args.b;
             float *c = args.c;
             void *kernel_args[] = {&copy, &a, &b, &c};
@@ -67,6 +68,27 @@ static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStr
     }
     return launch(kmc::build_kernel<KMC_INNER_OP, KMC_INNER_POW, LOAD_A, LOAD_B>, grid, dim3(kmc::BK_THREADS), stream, args);
 }
+
+#if KMC_INNER_OP == 0 && KMC_INNER_POW == 2
+// For a matrix-core call for squared differences that took a sample (args.sample): when the direct kernel with b in
+// scalar registers can take the operands as they are, launches it in front of the repair launch, where it computes
+// everything if the sample left the call to the direct kernel and exits at once if not.  Without it the repair launch
+// does that work on the ordinary kernel, 8 % slower.  *launched says whether the call qualified.
+hipError_t launch_scalar_b_if_the_sample_leaves(int load_a, int load_b, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *launched)
+{
+    *launched = false;
+    int64_t tiles_m = 0, tiles_n = 0;
+    if (!args.sample || load_a != kmc::LOAD_COL_VEC || load_b != kmc::LOAD_COL_VEC || !scalar_b_applies(args, &tiles_m, &tiles_n))
+        return hipSuccess;
+    kmc::BuildKernelArgs copy = args;
+    const float *a = args.a, *b = args.b;
+    float *c = args.c;
+    void *kernel_args[] = {&copy, &a, &b, &c};
+    *launched = true;
+    return hipLaunchKernel(reinterpret_cast<const void *>(kmc::build_kernel_scalar_b<KMC_INNER_OP, KMC_INNER_POW>),
+                           dim3(static_cast<unsigned>(tiles_m * tiles_n), args.l), dim3(kmc::BK_THREADS), kernel_args, 0, stream);
+}
+#endif
 
 hipError_t KMC_LAUNCHER_NAME(int load_a, int load_b, const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)
 {

@@ -73,6 +73,10 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
                                                                       const float *__restrict__ operand_b, float *__restrict__ result)
 {
     static_assert(INNER_OP == OP_DIFF, "differences only");
+    // Launched between a matrix-core kernel for squared differences and its repair launch: the whole result when the
+    // sample taken in front of them left the call to the direct kernel (the matrix-core kernel has then only stamped
+    // its tiles, and the repair launch behind finds none of the stamps), nothing otherwise.
+    if (args.sample != nullptr && !sample_leaves_it_to_the_direct_kernel(args.sample)) return;
     // two slices of 16 k-rows, and one row that the fragment read ahead of the last k of the second slice touches
     __shared__ __attribute__((aligned(16))) float lds_a[(2 * BK_TILE_K + 1) * SB_TILE_M];
     const int tid = threadIdx.x;

@@ -231,9 +231,11 @@ int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKe
 
 // Row statistics and split of both operands, then the product kernel.  `*taken` says whether the
 // path applied (and the launches were made); if not, nothing was launched.
-hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken)
+hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *taken,
+                                const unsigned **sample_taken)
 {
     *taken = false;
+    if (sample_taken) *sample_taken = nullptr;
     WideLayout layout;
     if (!p->gram_workspace || !wide_layout(p, args, &layout) || p->gram_workspace_bytes < layout.bytes ||
         (reinterpret_cast<uintptr_t>(p->gram_workspace) & (REGION_ALIGN - 1)) != 0)
@@ -279,6 +281,7 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
         status = launch_gram_probe(p, wide.kernel, sample, stream);
         if (status != hipSuccess) return status;
         wide.kernel.sample = sample;
+        if (sample_taken) *sample_taken = sample;
     }
     if (args.symmetric) {
         const dim3 grid(static_cast<unsigned>(layout.tiles_m) * (layout.tiles_m + 1) / 2, args.l, 1);
