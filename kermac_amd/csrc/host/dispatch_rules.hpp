@@ -38,6 +38,7 @@
     /* tiles of 256 x 64 in every batch entry */                                                         \
     X(DIRECT_SCALAR_B_MIN_TILES, 1800)                                                                  \
     X(DIRECT_SCALAR_B_MIN_K, 64)                                                                        \
+    X(DIRECT_SCALAR_B_MIN_TILES_SYMMETRIC, 16000)    /* a panel against itself: the tiles of its triangle */ \
     /* ... on copies of operands in any other storage (KMC_FLAG_DIRECT_PANELS): the same tiles, per batch entry */ \
     X(DIRECT_PANELS_MIN_TILES, 5400)                                                                    \
     X(DIRECT_PANELS_MIN_K, 64)                                                                          \

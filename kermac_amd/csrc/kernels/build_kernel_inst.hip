@@ -26,21 +26,28 @@ namespace kmc_host {
 // 1876 (1000 x 30000) 1.01 .. 1.02 and 1.03 .. 1.07, 3776 (30000 x 2000) 1.04 .. 1.21, 55342 (30000 x 30000) 1.02 .. 1.05 and
 // 1.05 .. 1.08; 1024 tiles (4096 x 4096) 0.96 .. 1.03, and batches of small entries lose: 8 x 2048 x 2048 0.95 .. 1.0,
 // 64 x 512 x 512 0.91 .. 1.0 for p = 1.
+// A panel against itself (the tiles of one triangle, each stored twice; ordinary kernel's time / this kernel's, p = 1 and
+// p = 2, one box): 30000 x 1024, 27966 tiles, 1.02 and 1.05; 16384 x 512, 8320 tiles, 0.99 and 1.05; 8192 x 1024 0.90 and 1.02;
+// 12000 x 128 1.03 and 1.05; 6000 x 512 level: taken from 16000 tiles on.
 // KERMAC_AMD_SCALAR_B_MIN_TILES=n replaces the size rule by "at least n tiles over the batch, any k" (read on every
 // call, so that a test can send small shapes to the kernel).
-static bool scalar_b_applies(const kmc::BuildKernelArgs &args, int64_t *tiles_m, int64_t *tiles_n)
+static bool scalar_b_applies(const kmc::BuildKernelArgs &args, int64_t *grid_width)
 {
-    if (args.k < 16 || args.k % kmc::BK_TILE_K != 0 || (args.n % kmc::SB_WAVE_N != 0 && !(args.panels & kmc::BK_PANELS_B_PADDED)) || args.k_total != 0 || args.repair_only || args.symmetric)
+    if (args.k < 16 || args.k % kmc::BK_TILE_K != 0 || (args.n % kmc::SB_WAVE_N != 0 && !(args.panels & kmc::BK_PANELS_B_PADDED)) ||
+        args.k_total != 0 || args.repair_only)
         return false;
-    *tiles_m = (static_cast<int64_t>(args.m) + kmc::SB_TILE_M - 1) / kmc::SB_TILE_M;
-    *tiles_n = (static_cast<int64_t>(args.n) + kmc::SB_TILE_N - 1) / kmc::SB_TILE_N;
-    const int64_t tiles = *tiles_m * *tiles_n;
-    if (tiles > 0x7fffffff) return false;
+    const int64_t tiles_m = (static_cast<int64_t>(args.m) + kmc::SB_TILE_M - 1) / kmc::SB_TILE_M;
+    const int64_t tiles_n = (static_cast<int64_t>(args.n) + kmc::SB_TILE_N - 1) / kmc::SB_TILE_N;
+    // a panel against itself: tile row r holds the tiles 0 .. 4 r + 3 that reach the diagonal or lie below it
+    const int64_t tiles = args.symmetric ? 2 * (tiles_m - 1) * tiles_m + (4 * tiles_m < tiles_n ? 4 * tiles_m : tiles_n) : tiles_m * tiles_n;
+    if (tiles > 0x7fffffff || (args.symmetric && args.m != args.n)) return false;
+    *grid_width = tiles;
     if (args.panels & kmc::BK_PANELS_COPIED) return true;       // the host made the copies for this kernel
     const char *text = std::getenv("KERMAC_AMD_SCALAR_B_MIN_TILES");
     const int forced = text ? std::atoi(text) : 0;
     if (forced > 0) return tiles * args.l >= forced;
-    return tiles >= kmc_rules::DIRECT_SCALAR_B_MIN_TILES && args.k >= kmc_rules::DIRECT_SCALAR_B_MIN_K;
+    return tiles >= (args.symmetric ? kmc_rules::DIRECT_SCALAR_B_MIN_TILES_SYMMETRIC : kmc_rules::DIRECT_SCALAR_B_MIN_TILES) &&
+           args.k >= kmc_rules::DIRECT_SCALAR_B_MIN_K;
 }
 
 template <int LOAD_A, int LOAD_B>
@@ -49,15 +56,15 @@ static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStr
     // absolute and squared differences of large problems whose rows are contiguous on both sides: b in scalar registers
     if constexpr (LOAD_A == kmc::LOAD_COL_VEC && LOAD_B == kmc::LOAD_COL_VEC && KMC_INNER_OP == kmc::OP_DIFF &&
                   (KMC_INNER_POW == kmc::POW_ABS || KMC_INNER_POW == kmc::POW_SQUARE)) {
-        int64_t tiles_m = 0, tiles_n = 0;
-        if (scalar_b_applies(args, &tiles_m, &tiles_n)) {
+        int64_t grid_width = 0;
+        if (scalar_b_applies(args, &grid_width)) {
             kmc::BuildKernelArgs copy = args;
             copy.sample = nullptr;          // an ordinary launch computes everything
             const float *a = args.a, *b = args.b;
             float *c = args.c;
             void *kernel_args[] = {&copy, &a, &b, &c};
             return hipLaunchKernel(reinterpret_cast<const void *>(kmc::build_kernel_scalar_b<KMC_INNER_OP, KMC_INNER_POW>),
-                                   dim3(static_cast<unsigned>(tiles_m * tiles_n), args.l), dim3(kmc::BK_THREADS), kernel_args, 0, stream);
+                                   dim3(static_cast<unsigned>(grid_width), args.l), dim3(kmc::BK_THREADS), kernel_args, 0, stream);
         }
     }
     // contiguous rows on both sides, a contraction long enough for the walk to set the time, and an inner term
@@ -77,8 +84,8 @@ static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStr
 hipError_t launch_scalar_b_if_the_sample_leaves(int load_a, int load_b, const kmc::BuildKernelArgs &args, hipStream_t stream, bool *launched)
 {
     *launched = false;
-    int64_t tiles_m = 0, tiles_n = 0;
-    if (!args.sample || load_a != kmc::LOAD_COL_VEC || load_b != kmc::LOAD_COL_VEC || !scalar_b_applies(args, &tiles_m, &tiles_n))
+    int64_t grid_width = 0;
+    if (!args.sample || load_a != kmc::LOAD_COL_VEC || load_b != kmc::LOAD_COL_VEC || !scalar_b_applies(args, &grid_width))
         return hipSuccess;
     kmc::BuildKernelArgs copy = args;
     const float *a = args.a, *b = args.b;
@@ -86,7 +93,7 @@ hipError_t launch_scalar_b_if_the_sample_leaves(int load_a, int load_b, const km
     void *kernel_args[] = {&copy, &a, &b, &c};
     *launched = true;
     return hipLaunchKernel(reinterpret_cast<const void *>(kmc::build_kernel_scalar_b<KMC_INNER_OP, KMC_INNER_POW>),
-                           dim3(static_cast<unsigned>(tiles_m * tiles_n), args.l), dim3(kmc::BK_THREADS), kernel_args, 0, stream);
+                           dim3(static_cast<unsigned>(grid_width), args.l), dim3(kmc::BK_THREADS), kernel_args, 0, stream);
 }
 #endif
 

@@ -15,8 +15,9 @@
 // What the host guarantees before it launches this kernel (build_kernel_inst.hip): both operands with rows
 // contiguous and 16-byte aligned (the LOAD_COL_VEC loaders), K a multiple of 16, N a multiple of 16 or b a copy
 // whose rows are padded to one (a wave's 16 columns can be loaded or do not exist; panel_copy.hip makes such copies
-// of operands in any other storage), no ranges of one contraction (k_total = 0), not a repair launch, not the triangle
-// of a symmetric result.  The last tile row may be ragged in m: lanes beyond M copy nothing and store nothing.
+// of operands in any other storage), no ranges of one contraction (k_total = 0), not a repair launch.  A panel
+// against itself (args.symmetric) runs the tiles that reach the diagonal or lie below it and stores each twice.
+// The last tile row may be ragged in m: lanes beyond M copy nothing and store nothing.
 // Results are those of build_kernel bit for bit: every element sums its terms over k in the same order.
 // The reference has one kernel for all shapes (include/build_a_kernel.cuh:339-462).
 #pragma once
@@ -92,7 +93,16 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
     // leave XCDs idle for its whole length.
     const int tiles_n = (args.n + SB_TILE_N - 1) / SB_TILE_N;
     int tile_m, tile_n;
-    {
+    if (args.symmetric) {
+        // A panel against itself: the tiles that reach the diagonal or lie below it, tile row r holding columns
+        // 0 .. 4 r + 3 (a tile is 256 x 64) and starting at id 2 r (r + 1); every tile is also stored mirrored.
+        const int id = blockIdx.x;
+        int row = (int)((sqrtf(2.0f * (float)id + 1.0f) - 1.0f) * 0.5f);
+        while (2 * row * (row + 1) > id) row--;
+        while (2 * (row + 1) * (row + 2) <= id) row++;
+        tile_m = row;
+        tile_n = id - 2 * row * (row + 1);
+    } else {
         constexpr int band_rows = 8 * SB_XCD_ROWS;
         const int banded_rows = ((args.m + SB_TILE_M - 1) / SB_TILE_M) / band_rows * band_rows;
         const int banded = banded_rows * tiles_n;                    // a multiple of 8
@@ -183,59 +193,101 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
         __builtin_amdgcn_s_waitcnt(0x0F70);      // this wave's copies of the next slice have landed
         __syncthreads();
     }
-    if (!wave_has_columns) return;
+    if (!wave_has_columns && !args.symmetric) return;
 
     // Epilogue: outer power, epsilon mask, kernel function, regularised diagonal -- finish_tile of build_kernel.hpp on
     // this kernel's 16 x 4 results per lane.  What depends on the lane's position is derived from a copy of the lane
     // id that the compiler cannot see through, so that it is not computed before the walk and kept through it.
-    int lane_after = lane;
-    asm volatile("" : "+v"(lane_after));
-    const int outer_power = args.outer_power;
-    const int kernel_type = args.kernel_type;
-    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
-    if (outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
-    if (kernel_type != KERNEL_NONE) {
-        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
-        neg_gamma = kernel_neg_gamma(kernel_type, bw);
-        regularization = args.regularization ? args.regularization[batch * args.regularization_bs] : args.regularization_value;
+    if (wave_has_columns) {
+        int lane_after = lane;
+        asm volatile("" : "+v"(lane_after));
+        const int outer_power = args.outer_power;
+        const int kernel_type = args.kernel_type;
+        float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
+        if (outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
+        if (kernel_type != KERNEL_NONE) {
+            const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
+            neg_gamma = kernel_neg_gamma(kernel_type, bw);
+            regularization = args.regularization ? args.regularization[batch * args.regularization_bs] : args.regularization_value;
+        }
+        const float epsilon = args.epsilon;
+        auto for_each = [&](auto &&f) {
+    #pragma unroll
+            for (int j = 0; j < SB_WAVE_N; j++)
+    #pragma unroll
+                for (int i = 0; i < 4; i++) acc[j][i] = f(acc[j][i]);
+        };
+        switch (outer_power) {
+        case POW_ABS: for_each([](float v) { return __builtin_fabsf(v); }); break;
+        case POW_SQUARE: for_each([](float v) { return v * v; }); break;
+        case POW_SQRT: for_each([](float v) { return __builtin_amdgcn_sqrtf(v); }); break;
+        case POW_POW: for_each([p_outer](float v) { return exp2f(p_outer * log2f(v)); }); break;
+        default: break;
+        }
+        if (kernel_type != KERNEL_NONE)
+            for_each([epsilon, neg_gamma](float v) { return expf((v < epsilon ? 0.0f : v) * neg_gamma); });
+        const int m_first = m0 + 4 * lane_after;
+        if (kernel_type != KERNEL_NONE && regularization != 0.0f) {
+            const float diagonal_value = 1.0f + regularization;
+    #pragma unroll
+            for (int j = 0; j < SB_WAVE_N; j++)
+    #pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (args.reg_off_x + m_first + i == args.reg_off_y + n0 + j) acc[j][i] = diagonal_value;
+        }
+        // Stores: a wave writes 1 KB of consecutive m for each of its 16 columns.
+        float *c_rows = result + batch * args.c_bs + (i64)n0 * args.c_ld + m_first;
+        if (args.c_vec && m_first + 3 < args.m) {
+    #pragma unroll
+            for (int j = 0; j < SB_WAVE_N; j++)
+                if (j < columns) *reinterpret_cast<float4 *>(c_rows + (i64)j * args.c_ld) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+        } else {
+    #pragma unroll
+            for (int j = 0; j < SB_WAVE_N; j++)
+    #pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (j < columns && m_first + i < args.m) c_rows[(i64)j * args.c_ld + i] = acc[j][i];
+        }
     }
-    const float epsilon = args.epsilon;
-    auto for_each = [&](auto &&f) {
-#pragma unroll
-        for (int j = 0; j < SB_WAVE_N; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) acc[j][i] = f(acc[j][i]);
-    };
-    switch (outer_power) {
-    case POW_ABS: for_each([](float v) { return __builtin_fabsf(v); }); break;
-    case POW_SQUARE: for_each([](float v) { return v * v; }); break;
-    case POW_SQRT: for_each([](float v) { return __builtin_amdgcn_sqrtf(v); }); break;
-    case POW_POW: for_each([p_outer](float v) { return exp2f(p_outer * log2f(v)); }); break;
-    default: break;
-    }
-    if (kernel_type != KERNEL_NONE)
-        for_each([epsilon, neg_gamma](float v) { return expf((v < epsilon ? 0.0f : v) * neg_gamma); });
-    const int m_first = m0 + 4 * lane_after;
-    if (kernel_type != KERNEL_NONE && regularization != 0.0f) {
-        const float diagonal_value = 1.0f + regularization;
-#pragma unroll
-        for (int j = 0; j < SB_WAVE_N; j++)
+    if (!args.symmetric) return;
+
+    // The same values at C(n, m).  Through LDS (idle after the walk, which ends with a barrier), 64 rows m at a time: the
+    // lanes that hold them write their 4 x 16 results as [m][n], and the workgroup stores 16 rows of 256 bytes per
+    // instruction.  Elements on the far side of the diagonal that this writes are the ones another tile computes for
+    // itself, from the same terms in the same order: the same bits.
+    constexpr int MIRROR_PITCH = SB_TILE_N + 4;
+    static_assert(64 * MIRROR_PITCH <= (2 * BK_TILE_K + 1) * SB_TILE_M, "a quarter of the tile fits the staging array");
+    float *c_batch = result + batch * args.c_bs;
+    const int n_tile = tile_n * SB_TILE_N;
+#pragma unroll 1
+    for (int quarter = 0; quarter < 4; quarter++) {
+        if ((lane >> 4) == quarter) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                if (args.reg_off_x + m_first + i == args.reg_off_y + n0 + j) acc[j][i] = diagonal_value;
-    }
-    // Stores: a wave writes 1 KB of consecutive m for each of its 16 columns.
-    float *c_rows = result + batch * args.c_bs + (i64)n0 * args.c_ld + m_first;
-    if (args.c_vec && m_first + 3 < args.m) {
 #pragma unroll
-        for (int j = 0; j < SB_WAVE_N; j++)
-            if (j < columns) *reinterpret_cast<float4 *>(c_rows + (i64)j * args.c_ld) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
-    } else {
+                for (int v = 0; v < SB_WAVE_N / 4; v++)
+                    *reinterpret_cast<float4 *>(lds_a + (4 * (lane & 15) + i) * MIRROR_PITCH + SB_WAVE_N * wave + 4 * v) =
+                        make_float4(acc[4 * v][i], acc[4 * v + 1][i], acc[4 * v + 2][i], acc[4 * v + 3][i]);
+        }
+        __syncthreads();
 #pragma unroll
-        for (int j = 0; j < SB_WAVE_N; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (j < columns && m_first + i < args.m) c_rows[(i64)j * args.c_ld + i] = acc[j][i];
+        for (int pass = 0; pass < 4; pass++) {
+            const int row = 16 * pass + (tid >> 4), column = 4 * (tid & 15);
+            const int m = m0 + 64 * quarter + row, n = n_tile + column;
+            if (m < args.m && n < args.n) {
+                const float4 v = *reinterpret_cast<const float4 *>(lds_a + row * MIRROR_PITCH + column);
+                float *to = c_batch + (i64)m * args.c_ld + n;
+                if (args.c_vec && n + 3 < args.n) {
+                    *reinterpret_cast<float4 *>(to) = v;
+                } else {
+                    to[0] = v.x;
+                    if (n + 1 < args.n) to[1] = v.y;
+                    if (n + 2 < args.n) to[2] = v.z;
+                    if (n + 3 < args.n) to[3] = v.w;
+                }
+            }
+        }
+        __syncthreads();
     }
 }
 

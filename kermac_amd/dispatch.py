@@ -83,7 +83,8 @@ _ROWS = (
      "the exact-form variants"),
     ("every direct launch",
      "absolute or squared differences, both operands with m / n contiguous and 16-byte aligned, K and N multiples of 16, K ≥ {DIRECT_SCALAR_B_MIN_K}, "
-     "≥ {DIRECT_SCALAR_B_MIN_TILES} tiles of 256 × 64 in every batch entry, not ranges of one contraction, not a repair launch, not a set against itself",
+     "≥ {DIRECT_SCALAR_B_MIN_TILES} tiles of 256 × 64 in every batch entry ({DIRECT_SCALAR_B_MIN_TILES_SYMMETRIC} tiles of one triangle for a set against itself), "
+     "not ranges of one contraction, not a repair launch",
      "`build_kernel_scalar_b` (b in scalar registers, only a through LDS; 92 registers, four waves per SIMD)"),
     ("",
      "absolute or squared differences of operands that kernel cannot take as they are (k contiguous, misaligned, K or N not multiples of 16), "

@@ -73,9 +73,45 @@ def test_every_tile_of_the_band_order_is_walked_once(device, scalar_b, M, N, K, 
     assert_close_to_truth(got[..., sample, :], truth, rtol=1e-5, atol=1e-30, what=f"{M}x{N}x{K}x{L}")
 
 
+@pytest.mark.parametrize("M,K,L", [(16, 16, None), (48, 32, None), (256, 16, None), (272, 48, None), (1024, 64, None), (1040, 16, None),
+                                   (2000, 32, None), (4112, 16, None), (784, 32, 3)])
+@pytest.mark.parametrize("p", [1.0, 2.0])
+def test_a_panel_against_itself(device, scalar_b, M, K, L, p):
+    """The tiles that reach the diagonal or lie below it, each stored twice: every element is written (the result starts
+    as NaN), the matrix is symmetric bit for bit with a zero diagonal, and it is the ordinary kernels' result."""
+    a, _ = panels(M, 16, K, device, M + K, L=L)
+    shape = (M, M) if L is None else (L, M, M)
+    out = torch.full(shape, float("nan"), device=device).transpose(-1, -2)
+    got = kermac.cdist(a, a, out=out, p=p)
+    assert not torch.isnan(got).any(), "elements left out"
+    assert torch.equal(got, got.transpose(-1, -2)) and (torch.diagonal(got, dim1=-2, dim2=-1) == 0).all()
+    plain = ordinary(scalar_b, lambda: kermac.cdist(a, a, p=p))
+    assert torch.equal(got, plain.reshape(got.shape)), "not the ordinary kernel's bits"
+    rows = slice(0, M, 7)
+    if L is None:
+        truth = l1_distances_float64(a[rows], a) if p == 1.0 else torch.cdist(a[rows].double(), a.double(), p=2.0, compute_mode="donot_use_mm_for_euclid_dist")
+        assert_close_to_truth(got[rows], truth, rtol=1e-5, atol=1e-5, what=f"a against a, p={p} {M}x{K}")
+
+
+def test_a_panel_against_itself_with_a_kernel_function_and_odd_results(device, scalar_b):
+    """Laplace kernel with a regularised diagonal; a result whose rows are padded, and one that is off a 16-byte
+    boundary (32-bit stores on both sides of the diagonal)."""
+    M, K = 600 + 8, 48
+    a, _ = panels(M, 16, K, device, 21)
+    call = lambda **kw: kermac.run_kernel(kermac.kernel_descriptor_laplace_l1, a, a, bandwidth=5.0, regularization=0.5, **kw)
+    plain = ordinary(scalar_b, call)[0]
+    assert (torch.diagonal(plain) == 1.5).all()
+    store = torch.full((M, M + 4), float("nan"), device=device)
+    assert torch.equal(call(out=store[:, :M].t()), plain)
+    odd = torch.full((M * M + 1,), float("nan"), device=device)[1:].view(M, M).t()
+    assert torch.equal(call(out=odd), plain)
+    truth = oracle.run_kernel("DIFF", "ABS", "NOOP", "LAPLACE", a.cpu(), a.cpu(), bandwidth=5.0, regularization=0.5)
+    assert_close_to_truth(plain, truth.reshape(plain.shape), rtol=1e-5, atol=1e-7, what="laplace, a against a")
+
+
 def test_it_is_the_kernel_that_ran(device, scalar_b):
-    """Shapes the kernel cannot take (N or K not a multiple of 16, a set against itself, rows not contiguous) run the
-    ordinary kernels and give the same numbers; a misaligned operand does too."""
+    """Shapes the kernel cannot take (N or K not a multiple of 16, rows not contiguous) run the ordinary kernels and give
+    the same numbers; a misaligned operand does too."""
     for M, N, K in ((300, 81, 32), (300, 80, 40), (128, 128, 24)):
         a, b = panels(M, N, K, device, M + N + K)
         truth = l1_distances_float64(a, b)
