@@ -66,6 +66,112 @@ __device__ __forceinline__ void scalar_b_fragment(float (&f)[4], const float *p)
     f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
 }
 
+// The K walk of one 256 x 64 tile: acc[j][i] += inner(b[n0 + j, k] - a[m0 + 4 lane + i, k]) over k_slices slices of 16 k.
+// `a_lane` points at this lane's 16 bytes of k-row 0 of the tile's rows (a + m0 + 4 lane), `b_columns` at the wave's 16
+// columns of k-row 0 (uniform over the wave: the loads are scalar loads, provided the kernel's operand pointers are
+// restrict-qualified parameters of their own).  `lds_a`: two slices of 16 k-rows of 256 floats and one row more, which
+// the fragment read ahead of the last k of the second slice touches.  Every wave of the workgroup calls it (copies and
+// barriers are the workgroup's); a wave without columns computes nothing.  Ends with a barrier: lds_a is free afterwards.
+template <int INNER_POW>
+__device__ __forceinline__ void scalar_b_walk(float (&acc)[SB_WAVE_N][4], const float *a_lane, i64 a_ld, const float *b_columns, i64 b_ld,
+                                              int k_slices, bool lane_copies, bool wave_has_columns, float *lds_a, int lane, int wave)
+{
+    typedef const __attribute__((address_space(1))) void *global_address;
+    typedef __attribute__((address_space(3))) void *lds_address;
+    // copy j of 4 per slice and wave: k-row 4 * wave + j, 256 floats = 64 lanes x 16 bytes
+    const float *src[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) src[j] = a_lane + (i64)(4 * wave + j) * a_ld;
+    const i64 step_a = (i64)BK_TILE_K * a_ld;
+    auto copy_slice = [&](int buffer) {
+        if (lane_copies) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const unsigned to = (unsigned)(unsigned long)(lds_address)(lds_a + (buffer * BK_TILE_K + 4 * wave + j) * SB_TILE_M);
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"((global_address)src[j]), "s"(to) : "memory", "m0");
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) src[j] += step_a;
+    };
+    copy_slice(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+    __syncthreads();
+    for (int slice = 0; slice < k_slices; slice++) {
+        const int cur = slice & 1;
+        if (slice + 1 < k_slices) copy_slice(cur ^ 1);
+        if (wave_has_columns) {
+            const float *sa = lds_a + cur * BK_TILE_K * SB_TILE_M + 4 * lane;
+            const float *bk = b_columns + (i64)slice * BK_TILE_K * b_ld;
+            float fa0[4], fa1[4];
+            scalar_b_fragment(fa0, sa);
+#pragma unroll 1
+            for (int kk = 0; kk < BK_TILE_K; kk += SB_CHUNK) {
+                float sb[SB_CHUNK][SB_WAVE_N];
+#pragma unroll
+                for (int q = 0; q < SB_CHUNK; q++) {
+                    const float4 *row = reinterpret_cast<const float4 *>(bk + (i64)(kk + q) * b_ld);
+#pragma unroll
+                    for (int v = 0; v < SB_WAVE_N / 4; v++) {
+                        const float4 x = row[v];
+                        sb[q][4 * v] = x.x; sb[q][4 * v + 1] = x.y; sb[q][4 * v + 2] = x.z; sb[q][4 * v + 3] = x.w;
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < SB_CHUNK; q += 2) {
+                    scalar_b_fragment(fa1, sa + (kk + q + 1) * SB_TILE_M);
+#pragma unroll
+                    for (int j = 0; j < SB_WAVE_N; j += 2) scalar_b_pair<INNER_POW>(acc[j], acc[j + 1], fa0, sb[q][j], sb[q][j + 1]);
+                    scalar_b_fragment(fa0, sa + (kk + q + 2) * SB_TILE_M);       // past the slice on its last k: read, never used
+#pragma unroll
+                    for (int j = 0; j < SB_WAVE_N; j += 2) scalar_b_pair<INNER_POW>(acc[j], acc[j + 1], fa1, sb[q + 1][j], sb[q + 1][j + 1]);
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // this wave's copies of the next slice have landed
+        __syncthreads();
+    }
+}
+
+// Outer power, epsilon mask, kernel function, regularised diagonal -- finish_tile of build_kernel.hpp on this kernel's
+// 16 x 4 results per lane: columns n0 .. n0 + 15, rows m_first .. m_first + 3.
+__device__ __forceinline__ void scalar_b_finish(float (&acc)[SB_WAVE_N][4], const BuildKernelArgs &args, int batch, int m_first, int n0)
+{
+    const int outer_power = args.outer_power;
+    const int kernel_type = args.kernel_type;
+    float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
+    if (outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
+    if (kernel_type != KERNEL_NONE) {
+        const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
+        neg_gamma = kernel_neg_gamma(kernel_type, bw);
+        regularization = args.regularization ? args.regularization[batch * args.regularization_bs] : args.regularization_value;
+    }
+    const float epsilon = args.epsilon;
+    auto for_each = [&](auto &&f) {
+#pragma unroll
+        for (int j = 0; j < SB_WAVE_N; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[j][i] = f(acc[j][i]);
+    };
+    switch (outer_power) {
+    case POW_ABS: for_each([](float v) { return __builtin_fabsf(v); }); break;
+    case POW_SQUARE: for_each([](float v) { return v * v; }); break;
+    case POW_SQRT: for_each([](float v) { return __builtin_amdgcn_sqrtf(v); }); break;
+    case POW_POW: for_each([p_outer](float v) { return exp2f(p_outer * log2f(v)); }); break;
+    default: break;
+    }
+    if (kernel_type != KERNEL_NONE)
+        for_each([epsilon, neg_gamma](float v) { return expf((v < epsilon ? 0.0f : v) * neg_gamma); });
+    if (kernel_type != KERNEL_NONE && regularization != 0.0f) {
+        const float diagonal_value = 1.0f + regularization;
+#pragma unroll
+        for (int j = 0; j < SB_WAVE_N; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (args.reg_off_x + m_first + i == args.reg_off_y + n0 + j) acc[j][i] = diagonal_value;
+    }
+}
+
 // The operands come in twice: inside `args`, and as restrict-qualified parameters, which is what lets the compiler
 // prove that nothing the kernel writes (the copies into LDS, the result) can change b, and so load it with scalar
 // loads (through args.b it takes vector loads of one address for all lanes, and the kernel spills).
@@ -78,7 +184,6 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
     // sample taken in front of them left the call to the direct kernel (the matrix-core kernel has then only stamped
     // its tiles, and the repair launch behind finds none of the stamps), nothing otherwise.
     if (args.sample != nullptr && !sample_leaves_it_to_the_direct_kernel(args.sample)) return;
-    // two slices of 16 k-rows, and one row that the fragment read ahead of the last k of the second slice touches
     __shared__ __attribute__((aligned(16))) float lds_a[(2 * BK_TILE_K + 1) * SB_TILE_M];
     const int tid = threadIdx.x;
     const int batch = blockIdx.y;
@@ -129,122 +234,32 @@ __global__ __launch_bounds__(BK_THREADS, 4) void build_kernel_scalar_b(const Bui
     const int columns = args.n - n0 < SB_WAVE_N ? args.n - n0 : SB_WAVE_N;     // ... and these are stored
     const bool lane_copies = 4 * lane < m_valid;                 // the 16 bytes lie inside the row: its length is a multiple of 4 floats
 
-    typedef const __attribute__((address_space(1))) void *global_address;
-    typedef __attribute__((address_space(3))) void *lds_address;
-    // copy j of 4 per slice and wave: k-row 4 * wave + j, 256 floats = 64 lanes x 16 bytes
-    const float *src[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) src[j] = operand_a + batch * args.a_bs + (i64)(4 * wave + j) * args.a_ld + m0 + 4 * lane;
-    const i64 step_a = (i64)BK_TILE_K * args.a_ld;
-    auto copy_slice = [&](int buffer) {
-        if (lane_copies) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const unsigned to = (unsigned)(unsigned long)(lds_address)(lds_a + (buffer * BK_TILE_K + 4 * wave + j) * SB_TILE_M);
-                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"((global_address)src[j]), "s"(to) : "memory", "m0");
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++) src[j] += step_a;
-    };
-
     float acc[SB_WAVE_N][4];
 #pragma unroll
     for (int j = 0; j < SB_WAVE_N; j++)
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[j][i] = 0.0f;
-
-    const int k_slices = args.k / BK_TILE_K;
-    const float *b_columns = operand_b + batch * args.b_bs + n0;    // uniform: the loads below are scalar loads
-    copy_slice(0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
-    __syncthreads();
-    for (int slice = 0; slice < k_slices; slice++) {
-        const int cur = slice & 1;
-        if (slice + 1 < k_slices) copy_slice(cur ^ 1);
-        if (wave_has_columns) {
-            const float *sa = lds_a + cur * BK_TILE_K * SB_TILE_M + 4 * lane;
-            const float *bk = b_columns + (i64)slice * BK_TILE_K * args.b_ld;
-            float fa0[4], fa1[4];
-            scalar_b_fragment(fa0, sa);
-#pragma unroll 1
-            for (int kk = 0; kk < BK_TILE_K; kk += SB_CHUNK) {
-                float sb[SB_CHUNK][SB_WAVE_N];
-#pragma unroll
-                for (int q = 0; q < SB_CHUNK; q++) {
-                    const float4 *row = reinterpret_cast<const float4 *>(bk + (i64)(kk + q) * args.b_ld);
-#pragma unroll
-                    for (int v = 0; v < SB_WAVE_N / 4; v++) {
-                        const float4 x = row[v];
-                        sb[q][4 * v] = x.x; sb[q][4 * v + 1] = x.y; sb[q][4 * v + 2] = x.z; sb[q][4 * v + 3] = x.w;
-                    }
-                }
-#pragma unroll
-                for (int q = 0; q < SB_CHUNK; q += 2) {
-                    scalar_b_fragment(fa1, sa + (kk + q + 1) * SB_TILE_M);
-#pragma unroll
-                    for (int j = 0; j < SB_WAVE_N; j += 2) scalar_b_pair<INNER_POW>(acc[j], acc[j + 1], fa0, sb[q][j], sb[q][j + 1]);
-                    scalar_b_fragment(fa0, sa + (kk + q + 2) * SB_TILE_M);       // past the slice on its last k: read, never used
-#pragma unroll
-                    for (int j = 0; j < SB_WAVE_N; j += 2) scalar_b_pair<INNER_POW>(acc[j], acc[j + 1], fa1, sb[q + 1][j], sb[q + 1][j + 1]);
-                }
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);      // this wave's copies of the next slice have landed
-        __syncthreads();
-    }
+    scalar_b_walk<INNER_POW>(acc, operand_a + batch * args.a_bs + m0 + 4 * lane, args.a_ld,
+                             operand_b + batch * args.b_bs + n0, args.b_ld, args.k / BK_TILE_K, lane_copies, wave_has_columns, lds_a, lane, wave);
     if (!wave_has_columns && !args.symmetric) return;
 
-    // Epilogue: outer power, epsilon mask, kernel function, regularised diagonal -- finish_tile of build_kernel.hpp on
-    // this kernel's 16 x 4 results per lane.  What depends on the lane's position is derived from a copy of the lane
-    // id that the compiler cannot see through, so that it is not computed before the walk and kept through it.
+    // Epilogue and stores.  What depends on the lane's position is derived from a copy of the lane id that the compiler
+    // cannot see through, so that it is not computed before the walk and kept through it.
     if (wave_has_columns) {
         int lane_after = lane;
         asm volatile("" : "+v"(lane_after));
-        const int outer_power = args.outer_power;
-        const int kernel_type = args.kernel_type;
-        float p_outer = 0.0f, neg_gamma = 0.0f, regularization = 0.0f;
-        if (outer_power == POW_POW) p_outer = args.p_outer ? args.p_outer[batch * args.p_outer_bs] : args.p_outer_value;
-        if (kernel_type != KERNEL_NONE) {
-            const float bw = args.bandwidth ? args.bandwidth[batch * args.bandwidth_bs] : args.bandwidth_value;
-            neg_gamma = kernel_neg_gamma(kernel_type, bw);
-            regularization = args.regularization ? args.regularization[batch * args.regularization_bs] : args.regularization_value;
-        }
-        const float epsilon = args.epsilon;
-        auto for_each = [&](auto &&f) {
-    #pragma unroll
-            for (int j = 0; j < SB_WAVE_N; j++)
-    #pragma unroll
-                for (int i = 0; i < 4; i++) acc[j][i] = f(acc[j][i]);
-        };
-        switch (outer_power) {
-        case POW_ABS: for_each([](float v) { return __builtin_fabsf(v); }); break;
-        case POW_SQUARE: for_each([](float v) { return v * v; }); break;
-        case POW_SQRT: for_each([](float v) { return __builtin_amdgcn_sqrtf(v); }); break;
-        case POW_POW: for_each([p_outer](float v) { return exp2f(p_outer * log2f(v)); }); break;
-        default: break;
-        }
-        if (kernel_type != KERNEL_NONE)
-            for_each([epsilon, neg_gamma](float v) { return expf((v < epsilon ? 0.0f : v) * neg_gamma); });
         const int m_first = m0 + 4 * lane_after;
-        if (kernel_type != KERNEL_NONE && regularization != 0.0f) {
-            const float diagonal_value = 1.0f + regularization;
-    #pragma unroll
-            for (int j = 0; j < SB_WAVE_N; j++)
-    #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    if (args.reg_off_x + m_first + i == args.reg_off_y + n0 + j) acc[j][i] = diagonal_value;
-        }
-        // Stores: a wave writes 1 KB of consecutive m for each of its 16 columns.
+        scalar_b_finish(acc, args, batch, m_first, n0);
+        // a wave writes 1 KB of consecutive m for each of its 16 columns
         float *c_rows = result + batch * args.c_bs + (i64)n0 * args.c_ld + m_first;
         if (args.c_vec && m_first + 3 < args.m) {
-    #pragma unroll
+#pragma unroll
             for (int j = 0; j < SB_WAVE_N; j++)
                 if (j < columns) *reinterpret_cast<float4 *>(c_rows + (i64)j * args.c_ld) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
         } else {
-    #pragma unroll
+#pragma unroll
             for (int j = 0; j < SB_WAVE_N; j++)
-    #pragma unroll
+#pragma unroll
                 for (int i = 0; i < 4; i++)
                     if (j < columns && m_first + i < args.m) c_rows[(i64)j * args.c_ld + i] = acc[j][i];
         }
