@@ -152,7 +152,7 @@ enum kmc_flags {
      * (points stored cluster by cluster) leave the call on the matrix cores.  This flag leaves the
      * sample out: every part is multiplied, checked and, if need be, recomputed. */
     KMC_FLAG_NO_PROBE = 1024,
-    /* kmc_build_kernel, inner_operator DIFF with inner_power ABS or SQUARE on the direct kernel (none of the
+    /* kmc_build_kernel, inner_operator DIFF with inner_power ABS, SQUARE or a scalar exponent of 3 or 4 on the direct kernel (none of the
      * flags above), with gram_workspace: the fastest direct kernel for large problems (b in scalar registers)
      * takes its operands as k-major panels (rows contiguous, 16-byte aligned, k a multiple of 16, n a multiple
      * of 16).  With this flag the library copies operands stored any other way -- k contiguous as torch

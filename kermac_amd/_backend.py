@@ -35,6 +35,7 @@ OP_DOT = 1
 POW_NOOP = 0
 POW_ABS = 1
 POW_SQUARE = 2
+POW_POW = 4
 
 FLAG_FORCE_SCALAR_ACCESS = 1
 FLAG_NEGATE_DIFF = 2

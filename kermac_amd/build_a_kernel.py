@@ -641,8 +641,11 @@ def run_kernel(
         plan.keepalive.append(_attach_gram_centre(params, stream, a.device))
         plan.keepalive.append(_attach_gram_workspace(params, a.device))
     elif (cut is None and not params.flags & (_backend.FLAG_DOT_PIECES | _backend.FLAG_L1_FIXED)
-            and params.inner_operator == _backend.OP_DIFF and params.inner_power in (_backend.POW_ABS, _backend.POW_SQUARE)):
-        # absolute and squared differences on the direct kernel: large problems whose operands its fastest
+            and params.inner_operator == _backend.OP_DIFF
+            and (params.inner_power in (_backend.POW_ABS, _backend.POW_SQUARE)
+                 or (params.inner_power == _backend.POW_POW and not params.p_inner and params.p_inner_value in (3.0, 4.0)
+                     and not params.flags & _backend.FLAG_GENERIC_POWER))):
+        # absolute differences and their squares, cubes and fourth powers on the direct kernel: large problems whose operands its fastest
         # variant cannot take as they are (k contiguous, as torch allocates them; K or N not multiples of 16) run
         # on copies that it can, when the library wants room for them (include/kermac_amd.h, KMC_FLAG_DIRECT_PANELS)
         params.flags |= _backend.FLAG_DIRECT_PANELS

@@ -53,9 +53,11 @@ static bool scalar_b_applies(const kmc::BuildKernelArgs &args, int64_t *grid_wid
 template <int LOAD_A, int LOAD_B>
 static hipError_t launch_one(const kmc::BuildKernelArgs &args, dim3 grid, hipStream_t stream)
 {
-    // absolute and squared differences of large problems whose rows are contiguous on both sides: b in scalar registers
+    // absolute differences, their squares, cubes and fourth powers, of large problems whose rows are contiguous on both
+    // sides: b in scalar registers
     if constexpr (LOAD_A == kmc::LOAD_COL_VEC && LOAD_B == kmc::LOAD_COL_VEC && KMC_INNER_OP == kmc::OP_DIFF &&
-                  (KMC_INNER_POW == kmc::POW_ABS || KMC_INNER_POW == kmc::POW_SQUARE)) {
+                  (KMC_INNER_POW == kmc::POW_ABS || KMC_INNER_POW == kmc::POW_SQUARE || KMC_INNER_POW == kmc::POW_ABS_CUBE ||
+                   KMC_INNER_POW == kmc::POW_ABS_FOURTH)) {
         int64_t grid_width = 0;
         if (scalar_b_applies(args, &grid_width)) {
             kmc::BuildKernelArgs copy = args;

@@ -45,18 +45,40 @@ constexpr int SB_XCD_ROWS = 2;      // row blocks of a that one XCD works on at 
 template <int INNER_POW>
 __device__ __forceinline__ void scalar_b_pair(float (&acc0)[4], float (&acc1)[4], const float (&fa)[4], float b0, float b1)
 {
-    static_assert(INNER_POW == POW_ABS || INNER_POW == POW_SQUARE, "absolute and squared differences only");
+    static_assert(INNER_POW == POW_ABS || INNER_POW == POW_SQUARE || INNER_POW == POW_ABS_CUBE || INNER_POW == POW_ABS_FOURTH,
+                  "absolute differences, their squares, cubes and fourth powers");
     float t0, t1, t2, t3, t4, t5, t6, t7;
     if (INNER_POW == POW_ABS) {
         asm volatile(KMC_SB_SUB8
                      "v_add_f32 %0, |%8|, %0\n\tv_add_f32 %1, |%9|, %1\n\tv_add_f32 %2, |%10|, %2\n\tv_add_f32 %3, |%11|, %3\n\t"
                      "v_add_f32 %4, |%12|, %4\n\tv_add_f32 %5, |%13|, %5\n\tv_add_f32 %6, |%14|, %6\n\tv_add_f32 %7, |%15|, %7"
                      KMC_SB_OPERANDS);
-    } else {
+    } else if (INNER_POW == POW_SQUARE) {
         asm volatile(KMC_SB_SUB8
                      "v_fmac_f32 %0, %8, %8\n\tv_fmac_f32 %1, %9, %9\n\tv_fmac_f32 %2, %10, %10\n\tv_fmac_f32 %3, %11, %11\n\t"
                      "v_fmac_f32 %4, %12, %12\n\tv_fmac_f32 %5, %13, %13\n\tv_fmac_f32 %6, %14, %14\n\tv_fmac_f32 %7, %15, %15"
                      KMC_SB_OPERANDS);
+    } else if (INNER_POW == POW_ABS_FOURTH) {
+        // (t t) (t t), as inner_term of device_common.hpp compiles: the square in place of t, then one multiply-add
+        asm volatile(KMC_SB_SUB8
+                     "v_mul_f32 %8, %8, %8\n\tv_mul_f32 %9, %9, %9\n\tv_mul_f32 %10, %10, %10\n\tv_mul_f32 %11, %11, %11\n\t"
+                     "v_mul_f32 %12, %12, %12\n\tv_mul_f32 %13, %13, %13\n\tv_mul_f32 %14, %14, %14\n\tv_mul_f32 %15, %15, %15\n\t"
+                     "v_fmac_f32 %0, %8, %8\n\tv_fmac_f32 %1, %9, %9\n\tv_fmac_f32 %2, %10, %10\n\tv_fmac_f32 %3, %11, %11\n\t"
+                     "v_fmac_f32 %4, %12, %12\n\tv_fmac_f32 %5, %13, %13\n\tv_fmac_f32 %6, %14, %14\n\tv_fmac_f32 %7, %15, %15"
+                     KMC_SB_OPERANDS);
+    } else {
+        // |t| (t t): the squares into a second set of registers, then |t| times them added to the sums in one instruction each
+        float u0, u1, u2, u3, u4, u5, u6, u7;
+        asm volatile("v_sub_f32 %8, %28, %24\n\tv_sub_f32 %9, %28, %25\n\tv_sub_f32 %10, %28, %26\n\tv_sub_f32 %11, %28, %27\n\t"
+                     "v_sub_f32 %12, %29, %24\n\tv_sub_f32 %13, %29, %25\n\tv_sub_f32 %14, %29, %26\n\tv_sub_f32 %15, %29, %27\n\t"
+                     "v_mul_f32 %16, %8, %8\n\tv_mul_f32 %17, %9, %9\n\tv_mul_f32 %18, %10, %10\n\tv_mul_f32 %19, %11, %11\n\t"
+                     "v_mul_f32 %20, %12, %12\n\tv_mul_f32 %21, %13, %13\n\tv_mul_f32 %22, %14, %14\n\tv_mul_f32 %23, %15, %15\n\t"
+                     "v_fma_f32 %0, |%8|, %16, %0\n\tv_fma_f32 %1, |%9|, %17, %1\n\tv_fma_f32 %2, |%10|, %18, %2\n\tv_fma_f32 %3, |%11|, %19, %3\n\t"
+                     "v_fma_f32 %4, |%12|, %20, %4\n\tv_fma_f32 %5, |%13|, %21, %5\n\tv_fma_f32 %6, |%14|, %22, %6\n\tv_fma_f32 %7, |%15|, %23, %7"
+                     : "+v"(acc0[0]), "+v"(acc0[1]), "+v"(acc0[2]), "+v"(acc0[3]), "+v"(acc1[0]), "+v"(acc1[1]), "+v"(acc1[2]), "+v"(acc1[3]),
+                       "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7),
+                       "=&v"(u0), "=&v"(u1), "=&v"(u2), "=&v"(u3), "=&v"(u4), "=&v"(u5), "=&v"(u6), "=&v"(u7)
+                     : "v"(fa[0]), "v"(fa[1]), "v"(fa[2]), "v"(fa[3]), "s"(b0), "s"(b1));
     }
 }
 

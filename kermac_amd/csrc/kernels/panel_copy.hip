@@ -84,7 +84,10 @@ bool plan_panels(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
 {
     if (!(p->flags & KMC_FLAG_DIRECT_PANELS)) return false;
     if (p->flags & (KMC_FLAG_L2_GRAM | KMC_FLAG_L2_GRAM_BF16 | KMC_FLAG_DOT_PIECES | KMC_FLAG_L1_FIXED | KMC_FLAG_FORCE_SCALAR_ACCESS)) return false;
-    if (p->inner_operator != KMC_OP_DIFF || (p->inner_power != KMC_POW_ABS && p->inner_power != KMC_POW_SQUARE)) return false;
+    // the inner powers build_kernel_scalar_b exists for: |x|, x^2, and the scalar exponents 3 and 4 that kmc_build_kernel evaluates as products
+    const bool cube_or_fourth = p->inner_power == KMC_POW_POW && !p->p_inner && !(p->flags & KMC_FLAG_GENERIC_POWER) &&
+                                (p->p_inner_value == 3.0f || p->p_inner_value == 4.0f);
+    if (p->inner_operator != KMC_OP_DIFF || (p->inner_power != KMC_POW_ABS && p->inner_power != KMC_POW_SQUARE && !cube_or_fourth)) return false;
     if (args.symmetric || args.k_total != 0 || args.repair_only || args.m < 1 || args.n < 1 || args.k < 1 || args.l < 1) return false;
     if (!args.c_vec) return false;
     const int64_t tiles = ceil_div(args.m, kmc::SB_TILE_M) * ceil_div(args.n, kmc::SB_TILE_N);

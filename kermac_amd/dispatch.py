@@ -82,12 +82,12 @@ _ROWS = (
      "direct `build_kernel` (ahead of time for DIFF + NOOP/ABS/SQUARE/POW and DOT + NOOP, else compiled on first use); scalar p of 0.5, 1.5, 3, 4 on "
      "the exact-form variants"),
     ("every direct launch",
-     "absolute or squared differences, both operands with m / n contiguous and 16-byte aligned, K and N multiples of 16, K ≥ {DIRECT_SCALAR_B_MIN_K}, "
+     "absolute differences, their squares, and the scalar exponents 3 and 4; both operands with m / n contiguous and 16-byte aligned, K and N multiples of 16, K ≥ {DIRECT_SCALAR_B_MIN_K}, "
      "≥ {DIRECT_SCALAR_B_MIN_TILES} tiles of 256 × 64 in every batch entry ({DIRECT_SCALAR_B_MIN_TILES_SYMMETRIC} tiles of one triangle for a set against itself), "
      "not ranges of one contraction, not a repair launch",
      "`build_kernel_scalar_b` (b in scalar registers, only a through LDS; 92 registers, four waves per SIMD)"),
     ("",
-     "absolute or squared differences of operands that kernel cannot take as they are (k contiguous, misaligned, K or N not multiples of 16), "
+     "the same inner terms on operands that kernel cannot take as they are (k contiguous, misaligned, K or N not multiples of 16), "
      "K ≥ {DIRECT_PANELS_MIN_K}, ≥ {DIRECT_PANELS_MIN_TILES} tiles of 256 × 64 in every batch entry, result 16-byte aligned, not ranges of one "
      "contraction, not a set against itself, and scratch memory allowed",
      "`panel_copy` of each such operand into padded k-major panels, then `build_kernel_scalar_b` on the copies"),

@@ -67,6 +67,15 @@ def test_matches_truth_and_the_ordinary_kernel(device, panels, M, N, K, layout, 
     assert torch.equal(got, plain), "not the ordinary kernel's bits"
 
 
+@pytest.mark.parametrize("p", [3.0, 4.0])
+def test_cubes_and_fourth_powers_take_the_copies_too(device, panels, p):
+    g = torch.Generator().manual_seed(17)
+    a, b = operand(700, 70, device, g, True), operand(333, 70, device, g, True)
+    got = kermac.cdist(a, b, p=p)
+    assert_close_to_truth(got[0], torch.cdist(a.double(), b.double(), p=p), rtol=1e-5, atol=1e-30, what=f"p={p}")
+    assert torch.equal(got, without_copies(panels, lambda: kermac.cdist(a, b, p=p))), "not the ordinary kernel's bits"
+
+
 def test_the_route_is_taken_where_the_library_says_so(device, panels):
     """The workspace the library asks for is what the call allocates: with the cap on scratch memory at zero nothing is
     copied and the result is the same; a call whose operands the kernel takes as they are asks for nothing."""

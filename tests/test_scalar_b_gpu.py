@@ -52,6 +52,20 @@ def test_matches_truth_and_the_ordinary_kernel(device, scalar_b, M, N, K, p):
     assert torch.equal(got, plain.reshape(got.shape)), "not the ordinary kernel's bits"
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 80, 32), (1000, 912, 64), (515, 1040, 208)])
+@pytest.mark.parametrize("p", [3.0, 4.0])
+def test_cubes_and_fourth_powers(device, scalar_b, M, N, K, p):
+    """The scalar exponents 3 and 4, which the library evaluates as |t| (t t) and (t t)(t t): against float64, and the
+    ordinary kernel's bits."""
+    a, b = panels(M, N, K, device, M + N + K)
+    got = kermac.cdist(a, b, p=p)
+    truth = torch.cdist(a.double(), b.double(), p=p)
+    assert_close_to_truth(got[0], truth, rtol=1e-5, atol=1e-30, what=f"p={p} {M}x{N}x{K}")
+    assert torch.equal(got, ordinary(scalar_b, lambda: kermac.cdist(a, b, p=p))), "not the ordinary kernel's bits"
+    raw = kermac.cdist(a, b, p=p, skip_epilogue=True)
+    assert torch.equal(raw, ordinary(scalar_b, lambda: kermac.cdist(a, b, p=p, skip_epilogue=True)))
+
+
 @pytest.mark.parametrize("M,N,K,L", [(256 * 15 + 9, 320, 16, None), (256 * 16, 336, 32, None), (256 * 17 + 100, 64 * 7 + 16, 16, None),
                                      (256 * 35 + 1, 208, 16, None), (256 * 33, 64 * 3, 32, 3), (256 * 18 + 77, 64 * 5 + 48, 16, 5)])
 def test_every_tile_of_the_band_order_is_walked_once(device, scalar_b, M, N, K, L):
