@@ -471,6 +471,10 @@ def main():
                         help="cdist (default, the headline metric, with the other two configurations as extra keys); "
                              "cdist_grad = only the Laplace-kernel RFM gradient configuration; kernel_coef = only the "
                              "fused Laplace kernel matrix x coefficients configuration")
+    parser.add_argument("--operand-layout", choices=["k_major", "torch"], default="k_major",
+                        help="with --only-p1 / --only-p: 'torch' hands over a[M, K], b[N, K], out[M, N] as torch allocates them "
+                             "(k and n contiguous) instead of BASELINE's K-major panels; the library then copies the operands "
+                             "into K-major panels inside the timed call")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also run one plain elementwise copy kernel over 1 GiB (read 1 GiB, write 1 GiB), so that "
                              "hardware byte counters collected by a profiler can be scaled against a known transfer")
@@ -498,6 +502,13 @@ def main():
     b_store = torch.randn(K, N, device=device)
     out_store = torch.empty(N, M, device=device)
     a, b, out = a_store.t(), b_store.t(), out_store.t()      # the operator's [M,K] / [N,K] / [M,N] views
+
+    if args.operand_layout == "torch":
+        if not (args.only_p1 or args.only_p is not None):
+            sys.exit("bench.py: --operand-layout torch goes with --only-p1 or --only-p (the default run measures BASELINE's layout "
+                     "and carries this one as per_p['1.0_torch_layout'])")
+        a, b = a.contiguous(), b.contiguous()
+        out = out_store.view(-1)[:M * N].view(M, N)
 
     if args.calibration_copy:
         calibration_copy(device)
@@ -698,7 +709,8 @@ def main():
             other_configs[name]["steps"], other_configs[name]["warmup"] = side_steps, 1
 
     achieved = OPS_PER_CALL / kernel_ms / 1e9
-    traffic, traffic_source = measured_traffic() if headline_p == 1.0 and kermac.get_l1_mode() == "direct" else (None, None)
+    traffic, traffic_source = (measured_traffic() if headline_p == 1.0 and kermac.get_l1_mode() == "direct" and args.operand_layout == "k_major"
+                               else (None, None))
     inner = {1.0: "POW_ABS", 2.0: "POW_SQUARE"}.get(headline_p, "POW_POW")
     headline_kernel = (f"kmc::build_kernel_scalar_b<OP_DIFF,{inner}>" if inner != "POW_POW"
                        else f"kmc::build_kernel<OP_DIFF,{inner},LOAD_COL_VEC,LOAD_COL_VEC>")
@@ -719,8 +731,10 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"cdist p={headline_p} fp32, a[K=1024,M=30000] b[K=1024,N=30000] K-major N(0,1) seed 1, "
-                               "out[N=30000,M=30000] with epilogue, no batch (BASELINE configs[1])",
+        "config": {"workload": (f"cdist p={headline_p} fp32, a[K=1024,M=30000] b[K=1024,N=30000] K-major N(0,1) seed 1, "
+                                "out[N=30000,M=30000] with epilogue, no batch (BASELINE configs[1])" if args.operand_layout == "k_major" else
+                                f"cdist p={headline_p} fp32, a[M=30000,K=1024] b[N=30000,K=1024] out[M=30000,N=30000] as torch allocates "
+                                "them, N(0,1) seed 1, with epilogue, no batch (BASELINE configs[1] in the other storage order)"),
                    "M": M, "N": N, "K": K, "p": headline_p},
         "per_p": per_p,
         "roofline": {
