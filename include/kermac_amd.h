@@ -160,8 +160,8 @@ enum kmc_flags {
      * a zero in both operands adds nothing to a sum, padded columns are not stored) and runs that kernel on
      * the copies: one read and one write of each copied operand against 5 to 7 % of the kernel's time.  The
      * sums are the direct kernel's bit for bit.  kmc_gram_workspace_bytes says which calls take the route
-     * (5400 tiles of 256 x 64 per batch entry, k >= 64, an operand that needs a copy, not a panel against
-     * itself, 16-byte aligned c; KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE: any size) and how much memory it wants
+     * (5400 tiles of 256 x 64 per batch entry -- 16000 tiles of one triangle for a panel against itself, which
+     * is copied once --, k >= 64, an operand that needs a copy, 16-byte aligned c; KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE: any size) and how much memory it wants
      * (4 bytes per element of the padded copies).  Without a workspace, or for a call the query reports 0
      * for, the direct kernels run on the operands as they are.  The reference has one kernel for all
      * storage orders (include/build_a_kernel.cuh:484-539). */

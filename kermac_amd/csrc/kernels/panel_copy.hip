@@ -6,8 +6,8 @@
 // (k contiguous), misaligned views, and shapes with other K or N run the three-wave kernel, 5 to 7 % slower.  With
 // KMC_FLAG_DIRECT_PANELS and a workspace, kmc_build_kernel copies the operands that do not fit into panels that
 // do -- [entry][k rounded up to 16][rows rounded up to 64], zeros in the padding (a zero in both operands adds
-// |0 - 0| = 0 to a sum, and padded columns of b are computed but not stored) -- and launches that kernel on the
-// copies.  A copy reads and writes its operand once: 0.1 ms for 30000 x 1024 against the 1.5 ms the kernel gains
+// |0 - 0| = 0 to a sum, and padded columns of b are computed but not stored; a panel against itself is copied once)
+// -- and launches that kernel on the copies.  A copy reads and writes its operand once: 0.1 ms for 30000 x 1024 against the 1.5 ms the kernel gains
 // at M = N = 30000.  The sums are those of the direct kernels bit for bit (same terms, same order).
 // The reference has one kernel for all storage orders (include/build_a_kernel.cuh:484-539) and no copies.
 #include <hip/hip_runtime.h>
@@ -88,11 +88,14 @@ bool plan_panels(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
     const bool cube_or_fourth = p->inner_power == KMC_POW_POW && !p->p_inner && !(p->flags & KMC_FLAG_GENERIC_POWER) &&
                                 (p->p_inner_value == 3.0f || p->p_inner_value == 4.0f);
     if (p->inner_operator != KMC_OP_DIFF || (p->inner_power != KMC_POW_ABS && p->inner_power != KMC_POW_SQUARE && !cube_or_fourth)) return false;
-    if (args.symmetric || args.k_total != 0 || args.repair_only || args.m < 1 || args.n < 1 || args.k < 1 || args.l < 1) return false;
+    if (args.k_total != 0 || args.repair_only || args.m < 1 || args.n < 1 || args.k < 1 || args.l < 1) return false;
     if (!args.c_vec) return false;
-    const int64_t tiles = ceil_div(args.m, kmc::SB_TILE_M) * ceil_div(args.n, kmc::SB_TILE_N);
+    const int64_t tiles_m = ceil_div(args.m, kmc::SB_TILE_M), tiles_n = ceil_div(args.n, kmc::SB_TILE_N);
+    // a panel against itself: the kernel runs the tiles that reach the diagonal or lie below it, and has a size rule of its own for them
+    const int64_t tiles = args.symmetric ? 2 * (tiles_m - 1) * tiles_m + (4 * tiles_m < tiles_n ? 4 * tiles_m : tiles_n) : tiles_m * tiles_n;
+    const int64_t enough = args.symmetric ? kmc_rules::DIRECT_SCALAR_B_MIN_TILES_SYMMETRIC : kmc_rules::DIRECT_PANELS_MIN_TILES;
     const bool any_size = p->flags & KMC_FLAG_GRAM_WORKSPACE_ANY_SIZE;
-    if (!any_size && (tiles < kmc_rules::DIRECT_PANELS_MIN_TILES || args.k < kmc_rules::DIRECT_PANELS_MIN_K)) return false;
+    if (!any_size && (tiles < enough || args.k < kmc_rules::DIRECT_PANELS_MIN_K)) return false;
     if (tiles > 0x7fffffff) return false;
     auto fits = [&](const float *x, int64_t ld, int64_t bs, int majorness) {
         return majorness == KMC_COL_MAJOR && aligned16(x) && ld % 4 == 0 && bs % 4 == 0;
@@ -108,6 +111,12 @@ bool plan_panels(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &a
     plan->entries_b = p->b_bs == 0 ? 1 : args.l;
     plan->bytes_a = plan->copy_a ? round_up(4ll * plan->entries_a * plan->k_padded * plan->m_padded, 256) : 0;
     plan->bytes_b = plan->copy_b ? round_up(4ll * plan->entries_b * plan->k_padded * plan->n_padded, 256) : 0;
+    if (args.symmetric) {
+        // one panel on both sides: one copy
+        plan->copy_a = plan->copy_b = true;
+        plan->bytes_a = round_up(4ll * plan->entries_a * plan->k_padded * plan->m_padded, 256);
+        plan->bytes_b = 0;
+    }
     return true;
 }
 
@@ -155,7 +164,10 @@ hipError_t launch_direct_panels(const kmc_build_kernel_params *p, kmc::BuildKern
         args->a_ld = plan.m_padded;
         args->a_bs = plan.entries_a == 1 ? 0 : static_cast<int64_t>(plan.k_padded) * plan.m_padded;
     }
-    if (plan.copy_b) {
+    if (args->symmetric) {
+        args->b = args->a; args->b_ld = args->a_ld; args->b_bs = args->a_bs;
+        args->panels |= kmc::BK_PANELS_B_PADDED;
+    } else if (plan.copy_b) {
         float *panel = reinterpret_cast<float *>(workspace + plan.bytes_a);
         hipError_t e = copy_panel(p->b, p->b_ld, p->b_bs, p->b_majorness, args->n, args->k, plan.entries_b, panel, plan.n_padded,
                                   plan.k_padded, stream);

@@ -88,8 +88,8 @@ _ROWS = (
      "`build_kernel_scalar_b` (b in scalar registers, only a through LDS; 92 registers, four waves per SIMD)"),
     ("",
      "the same inner terms on operands that kernel cannot take as they are (k contiguous, misaligned, K or N not multiples of 16), "
-     "K ≥ {DIRECT_PANELS_MIN_K}, ≥ {DIRECT_PANELS_MIN_TILES} tiles of 256 × 64 in every batch entry, result 16-byte aligned, not ranges of one "
-     "contraction, not a set against itself, and scratch memory allowed",
+     "K ≥ {DIRECT_PANELS_MIN_K}, ≥ {DIRECT_PANELS_MIN_TILES} tiles of 256 × 64 in every batch entry ({DIRECT_SCALAR_B_MIN_TILES_SYMMETRIC} of one triangle for a "
+     "set against itself, which is copied once), result 16-byte aligned, not ranges of one contraction, and scratch memory allowed",
      "`panel_copy` of each such operand into padded k-major panels, then `build_kernel_scalar_b` on the copies"),
     ("",
      "both operands with m / n contiguous and 16-byte aligned, K ≥ {DIRECT_FOUR_WAVES_MIN_K}, inner power not fractional, not a repair launch",

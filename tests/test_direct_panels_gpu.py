@@ -76,6 +76,22 @@ def test_cubes_and_fourth_powers_take_the_copies_too(device, panels, p):
     assert torch.equal(got, without_copies(panels, lambda: kermac.cdist(a, b, p=p))), "not the ordinary kernel's bits"
 
 
+@pytest.mark.parametrize("M,K,k_contiguous", [(700, 70, True), (1030, 48, True), (523, 20, False), (2051, 16, True)])
+@pytest.mark.parametrize("p", [1.0, 2.0])
+def test_a_panel_against_itself_is_copied_once(device, panels, M, K, k_contiguous, p):
+    """One copy serves both sides; the kernel runs the tiles that reach the diagonal or lie below it and stores each twice:
+    symmetric bit for bit, zero diagonal, the ordinary kernels' result."""
+    g = torch.Generator().manual_seed(M + K)
+    a = operand(M, K, device, g, k_contiguous)
+    out = torch.full((M, M), float("nan"), device=device).t()
+    got = kermac.cdist(a, a, out=out, p=p)
+    assert not torch.isnan(got).any(), "elements left out"
+    assert torch.equal(got, got.t()) and (torch.diagonal(got) == 0).all()
+    assert torch.equal(got, without_copies(panels, lambda: kermac.cdist(a, a, p=p))[0]), "not the ordinary kernel's bits"
+    rows = slice(0, M, 5)
+    assert_close_to_truth(got[rows], truth_of(a[rows], a, p), rtol=1e-5, atol=1e-5, what=f"a against a {M}x{K}")
+
+
 def test_the_route_is_taken_where_the_library_says_so(device, panels):
     """The workspace the library asks for is what the call allocates: with the cap on scratch memory at zero nothing is
     copied and the result is the same; a call whose operands the kernel takes as they are asks for nothing."""

@@ -635,7 +635,8 @@ def test_workspace_queries_need_no_gpu(monkeypatch):
     assert panels(10000, 10000, 1024) > 0 and panels(9000, 9000, 1024) == 0         # 6280 and 5076 tiles
     assert panels(9000, 9000, 1024, l=4) == 0                                       # per batch entry
     assert panels(30000, 30000, 48) == 0
-    assert panels(30000, 30000, 1024, same=True) == 0                               # a set against itself: half the tiles instead
+    assert panels(30000, 30000, 1024, same=True) == 1024 * 30016 * 4               # a set against itself: one copy, from 16000 tiles of the triangle on
+    assert panels(16384, 16384, 1024, same=True) == 0                              # 8320 tiles
     assert panels(30000, 30000, 1024, flags=0) == 0
     assert panels(30000, 30000, 1024, flags=_backend.FLAG_DIRECT_PANELS | _backend.FLAG_L1_FIXED) == absolute_differences(30000, 30000, 1024)   # that route's own
     assert panels(300, 200, 5, flags=_backend.FLAG_DIRECT_PANELS | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE) == 16 * (320 + 256) * 4
