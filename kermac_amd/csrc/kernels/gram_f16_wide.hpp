@@ -140,12 +140,11 @@ __device__ __forceinline__ const float *gram_rows_centre(const GramRowsArgs &arg
     return centre[padded] != 0.0f ? centre : nullptr;      // the flag behind the vector: see centre_to_subtract
 }
 
-// One thread per row, one workgroup per 256 rows and range of slices.  (The two row kernels are
+// One thread per row, one workgroup per 256 rows and range of slices.  (The row kernels are
 // templates only so that every translation unit that includes this header may hold them.)
-template <int UNUSED = 0>
-__global__ __launch_bounds__(GW_ROW_THREADS) void gram_row_stats(const GramRowsArgs args)
+__device__ __forceinline__ void gram_row_stats_of(const GramRowsArgs &args, int block)
 {
-    const int row = blockIdx.x * GW_ROW_THREADS + threadIdx.x;
+    const int row = block * GW_ROW_THREADS + threadIdx.x;
     const int range = blockIdx.y, batch = blockIdx.z;
     const float *x = args.x + batch * args.bs;
     const float *centre = gram_rows_centre(args, batch);
@@ -169,9 +168,14 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_row_stats(const GramRowsA
 }
 
 template <int UNUSED = 0>
-__global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsArgs args)
+__global__ __launch_bounds__(GW_ROW_THREADS) void gram_row_stats(const GramRowsArgs args)
 {
-    const int row = blockIdx.x * GW_ROW_THREADS + threadIdx.x;
+    gram_row_stats_of(args, blockIdx.x);
+}
+
+__device__ __forceinline__ void gram_f16_split_of(const GramRowsArgs &args, int block)
+{
+    const int row = block * GW_ROW_THREADS + threadIdx.x;
     const int range = blockIdx.y, batch = blockIdx.z;
     const float *x = args.x + batch * args.bs;
     const float *centre = gram_rows_centre(args, batch);
@@ -222,6 +226,40 @@ __global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsA
 #pragma unroll
             for (int segment = 0; segment < GW_SEGMENTS; segment++) dst[(i64)segment * args.rows_pad] = gram_chunk{0u, 0u, 0u, 0u};
         }
+    }
+}
+
+template <int UNUSED = 0>
+__global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split(const GramRowsArgs args)
+{
+    gram_f16_split_of(args, blockIdx.x);
+}
+
+// Both operands of a call in one launch each (at a few thousand rows a launch of these kernels is its own latency, and
+// two of them one after the other cost twice that): the first `first_blocks` workgroups along x take the first operand.
+// Both have the same ranges of slices; an operand with fewer batch entries than the grid leaves the surplus idle.
+struct GramRowsPair {
+    GramRowsArgs first, second;
+    int first_blocks, first_batches, second_batches;
+};
+
+template <int UNUSED = 0>
+__global__ __launch_bounds__(GW_ROW_THREADS) void gram_row_stats_pair(const GramRowsPair pair)
+{
+    if ((int)blockIdx.x < pair.first_blocks) {
+        if ((int)blockIdx.z < pair.first_batches) gram_row_stats_of(pair.first, blockIdx.x);
+    } else if ((int)blockIdx.z < pair.second_batches) {
+        gram_row_stats_of(pair.second, blockIdx.x - pair.first_blocks);
+    }
+}
+
+template <int UNUSED = 0>
+__global__ __launch_bounds__(GW_ROW_THREADS) void gram_f16_split_pair(const GramRowsPair pair)
+{
+    if ((int)blockIdx.x < pair.first_blocks) {
+        if ((int)blockIdx.z < pair.first_batches) gram_f16_split_of(pair.first, blockIdx.x);
+    } else if ((int)blockIdx.z < pair.second_batches) {
+        gram_f16_split_of(pair.second, blockIdx.x - pair.first_blocks);
     }
 }
 

@@ -222,6 +222,24 @@ hipError_t launch_gram_rows(const kmc::GramRowsArgs &rows_of, int batches, hipSt
     return launch(kmc::gram_f16_split<0>, grid, dim3(kmc::GW_ROW_THREADS), stream, rows_of);
 }
 
+// The same for both operands of a call, in two launches instead of four.
+hipError_t launch_gram_rows_pair(const kmc::GramRowsArgs &first, int first_batches, const kmc::GramRowsArgs &second, int second_batches,
+                                 hipStream_t stream)
+{
+    if (first.ranges != second.ranges) {
+        hipError_t status = launch_gram_rows(first, first_batches, stream);
+        return status != hipSuccess ? status : launch_gram_rows(second, second_batches, stream);
+    }
+    kmc::GramRowsPair pair;
+    pair.first = first; pair.second = second;
+    pair.first_blocks = first.rows_pad / kmc::GW_ROW_THREADS;
+    pair.first_batches = first_batches; pair.second_batches = second_batches;
+    const dim3 grid(pair.first_blocks + second.rows_pad / kmc::GW_ROW_THREADS, first.ranges, first_batches > second_batches ? first_batches : second_batches);
+    hipError_t status = launch(kmc::gram_row_stats_pair<0>, grid, dim3(kmc::GW_ROW_THREADS), stream, pair);
+    if (status != hipSuccess) return status;
+    return launch(kmc::gram_f16_split_pair<0>, grid, dim3(kmc::GW_ROW_THREADS), stream, pair);
+}
+
 // Bytes of workspace the path needs for this problem; 0 when it does not apply.
 int64_t gram_f16_wide_bytes(const kmc_build_kernel_params *p, const kmc::BuildKernelArgs &args)
 {
@@ -245,12 +263,15 @@ hipError_t launch_gram_f16_wide(const kmc_build_kernel_params *p, const kmc::Bui
     const kmc::GramRowsArgs rows_a = rows_args(args.a, args.a_ld, args.a_bs, args.m, p->a_majorness, scalar_only, args, layout, layout.a, workspace);
     const kmc::GramRowsArgs rows_b = rows_args(args.b, args.b_ld, args.b_bs, args.n, p->b_majorness, scalar_only, args, layout, layout.b, workspace);
     // the region of a lies first in the workspace and its size does not depend on b
-    hipError_t status = split_of_a_is_kept(p, args, layout) ? hipSuccess : launch_gram_rows(rows_a, layout.a.batches, stream);
-    if (status != hipSuccess) return status;
-    if (!args.symmetric) {
-        status = launch_gram_rows(rows_b, layout.b.batches, stream);
-        if (status != hipSuccess) return status;
+    const bool a_is_kept = split_of_a_is_kept(p, args, layout);
+    hipError_t status = hipSuccess;
+    if (!a_is_kept && !args.symmetric) {
+        status = launch_gram_rows_pair(rows_a, layout.a.batches, rows_b, layout.b.batches, stream);
+    } else {
+        if (!a_is_kept) status = launch_gram_rows(rows_a, layout.a.batches, stream);
+        if (status == hipSuccess && !args.symmetric) status = launch_gram_rows(rows_b, layout.b.batches, stream);
     }
+    if (status != hipSuccess) return status;
 
     kmc::GramWideArgs wide = {};
     wide.kernel = args;
