@@ -451,8 +451,7 @@ int launch_norm_gradient_l2_wide(const kmc_norm_gradient_params *p, hipStream_t 
     const kmc::GramRowsArgs rows_a = rows_args(p->a, p->a_ld, p->a_bs, p->m, KMC_COL_MAJOR, scalar_only, walk, wide, wide.a, workspace);
     const kmc::GramRowsArgs rows_b = rows_args(prepare.products, prepare.products_ld, prepare.products_bs, rows, KMC_ROW_MAJOR, scalar_only,
                                                walk, wide, wide.b, workspace);
-    status = launch_gram_rows(rows_a, wide.a.batches, stream);
-    if (status == hipSuccess) status = launch_gram_rows(rows_b, wide.b.batches, stream);
+    status = launch_gram_rows_pair(rows_a, wide.a.batches, rows_b, wide.b.batches, stream);
     if (status != hipSuccess) return fail_hip(status, "gram_row_stats / gram_f16_split launch");
 
     kmc::GramWideArgs product = {};

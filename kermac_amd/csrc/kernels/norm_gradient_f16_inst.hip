@@ -121,7 +121,8 @@ kmc::GramRowsArgs rows_args(const float *x, int64_t ld, int64_t bs, int rows, bo
 
 }  // namespace
 
-hipError_t launch_gram_rows(const kmc::GramRowsArgs &rows_of, int batches, hipStream_t stream);     // gram_f16_wide_inst.hip
+hipError_t launch_gram_rows_pair(const kmc::GramRowsArgs &first, int first_batches, const kmc::GramRowsArgs &second, int second_batches,
+                                 hipStream_t stream);     // gram_f16_wide_inst.hip
 
 int64_t norm_gradient_f16_bytes(const kmc_norm_gradient_params *p)
 {
@@ -142,9 +143,7 @@ hipError_t launch_norm_gradient_f16(const kmc_norm_gradient_params *p, bool a_ve
     (void)a_vec;
     const kmc::GramRowsArgs rows_a = rows_args(p->a, p->a_ld, p->a_bs, p->m, false, false, p->k, layout, layout.a, workspace);
     const kmc::GramRowsArgs rows_c = rows_args(p->c, p->c_ld, p->c_bs, p->o, true, c_vec, p->k, layout, layout.c, workspace);
-    hipError_t status = launch_gram_rows(rows_a, layout.a.batches, stream);
-    if (status != hipSuccess) return status;
-    status = launch_gram_rows(rows_c, layout.c.batches, stream);
+    hipError_t status = launch_gram_rows_pair(rows_a, layout.a.batches, rows_c, layout.c.batches, stream);
     if (status != hipSuccess) return status;
 
     kmc::GradientPadArgs pad = {};
