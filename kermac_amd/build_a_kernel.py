@@ -648,18 +648,27 @@ def run_kernel(
         # absolute differences and their squares, cubes and fourth powers on the direct kernel: large problems whose operands its fastest
         # variant cannot take as they are (k contiguous, as torch allocates them; K or N not multiples of 16) run
         # on copies that it can, when the library wants room for them (include/kermac_amd.h, KMC_FLAG_DIRECT_PANELS)
-        params.flags |= _backend.FLAG_DIRECT_PANELS
-        if os.environ.get("KERMAC_AMD_DIRECT_PANELS_ANY_SIZE", "0") not in ("", "0"):
-            params.flags |= _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE      # tests send small shapes down the route
-        workspace = _attach_gram_workspace(params, a.device, switch="KERMAC_AMD_DIRECT_PANELS")
-        if workspace is None:
-            params.flags &= ~(_backend.FLAG_DIRECT_PANELS | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE)
-        plan.keepalive.append(workspace)
+        any_size = os.environ.get("KERMAC_AMD_DIRECT_PANELS_ANY_SIZE", "0") not in ("", "0")     # tests send small shapes down the route
+        # (the library decides; a call far below its size rule is not worth the question: small calls are bound by the host)
+        if any_size or -(-params.m // 256) * -(-params.n // 64) >= _direct_panels_min_tiles():
+            params.flags |= _backend.FLAG_DIRECT_PANELS
+            if any_size:
+                params.flags |= _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE
+            workspace = _attach_gram_workspace(params, a.device, switch="KERMAC_AMD_DIRECT_PANELS")
+            if workspace is None:
+                params.flags &= ~(_backend.FLAG_DIRECT_PANELS | _backend.FLAG_GRAM_WORKSPACE_ANY_SIZE)
+            plan.keepalive.append(workspace)
     if cut is None:
         launch(params)
     else:
         _run_cut_over_contraction(cut, params, launch, stream, a.device)
     return plan.out
+
+
+@functools.lru_cache(maxsize=1)
+def _direct_panels_min_tiles() -> int:
+    """The smallest count of 256 x 64 tiles per batch entry for which the library copies operands for its direct kernel."""
+    return int(_backend.dispatch_rules()["DIRECT_PANELS_MIN_TILES"])
 
 
 def _attach_gram_centre(params, stream, device):
