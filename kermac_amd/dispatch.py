@@ -53,7 +53,7 @@ _ROWS = (
      "{WIDE_MIN_TILES_PER_SIDE_X2} · (tiles_m + tiles_n), ≤ {WIDE_MAX_PADDING_PERCENT} % of the tiles' area padding; with k contiguous in both "
      "operands instead: K ≥ {WIDE_K_CONTIGUOUS_MIN_K}, ≥ {WIDE_K_CONTIGUOUS_MIN_TILES} tiles, tiles · K ≥ {WIDE_K_CONTIGUOUS_MIN_TILES_TIMES_K}, M and N ≥ "
      "{WIDE_K_CONTIGUOUS_MIN_ROWS}",
-     "`gram_probe_operands`, `gram_row_stats` + `gram_f16_split` per operand, `gram_f16_wide` (fp16 pieces, 256 × 256 tiles), repair launch "
+     "`gram_row_stats_pair` + `gram_f16_split_pair` (both operands per launch), `gram_probe_operands`, `gram_f16_wide` (fp16 pieces, 256 × 256 tiles), repair launch "
      "of the direct kernel"),
     ("",
      "K ≥ {build_a_kernel.AUTO_ONE_STEP_MIN_K}, trust < 1, "
