@@ -154,3 +154,51 @@ def test_large_problem_by_the_librarys_own_rule(device):
     assert torch.cuda.memory_stats(device)["allocation.all.allocated"] - before == 2       # the result and the copies
     sample = slice(0, 10000, 131)
     assert_close_to_truth(got[0, sample], l1_distances_float64(a[sample], b), rtol=1e-5, atol=1e-30, what="10000 x 10008 x 200")
+
+
+def test_random_calls_with_both_variants_forced(device, monkeypatch):
+    """300 seeded random calls -- shapes around the tile edges, both storage orders, misaligned views, batches with shared
+    operands, a set against itself, row-major results, Laplace kernels with an offset diagonal -- once with the copies and the
+    kernel with b in scalar registers forced wherever they can run, once with both switched off: the same bits, no NaN."""
+    import random
+    rng = random.Random(20240521)
+    g = torch.Generator().manual_seed(99)
+    kermac.set_l2_mode("direct")
+    try:
+        for case in range(300):
+            M = rng.choice([1, 3, 64, 255, 256, 257, 300, 512, 777, 1024, 1500, 2049])
+            N = rng.choice([1, 16, 17, 48, 64, 65, 100, 256, 300, 640, 1000])
+            K = rng.choice([1, 5, 16, 17, 32, 48, 100, 128, 130])
+            L = rng.choice([None, None, 2, 3])
+            p = rng.choice([1.0, 2.0])
+            same = rng.random() < 0.15
+            shared_a = L is not None and rng.random() < 0.2
+            shared_b = L is not None and not shared_a and rng.random() < 0.2
+            a = operand(M, K, device, g, rng.random() < 0.5, L=None if shared_a else L, misaligned=rng.random() < 0.2)
+            b = a if same else operand(N, K, device, g, rng.random() < 0.5, L=None if shared_b else L, misaligned=rng.random() < 0.2)
+            columns = M if same else N
+            row_major_out = L is None and rng.random() < 0.3
+            laplace = rng.random() < 0.5
+            offsets = (0, 0) if same else (rng.choice([0, 0, 2]), rng.choice([0, 0, 1]))
+
+            def call():
+                if laplace:
+                    descriptor = kermac.kernel_descriptor_laplace_l1 if p == 1.0 else kermac.kernel_descriptor_laplace_l2
+                    return kermac.run_kernel(descriptor, a, b, bandwidth=3.0, regularization=0.5, regularization_offset_x=offsets[0],
+                                             regularization_offset_y=offsets[1])
+                out = torch.full((M, columns), float("nan"), device=device) if row_major_out else None
+                return kermac.cdist(a, b, p=p, out=out)
+
+            monkeypatch.setenv("KERMAC_AMD_DIRECT_PANELS_ANY_SIZE", "1")
+            monkeypatch.setenv("KERMAC_AMD_SCALAR_B_MIN_TILES", "1")
+            forced = call()
+            monkeypatch.delenv("KERMAC_AMD_DIRECT_PANELS_ANY_SIZE")
+            monkeypatch.setenv("KERMAC_AMD_SCALAR_B_MIN_TILES", "2000000000")
+            monkeypatch.setenv("KERMAC_AMD_DIRECT_PANELS", "0")
+            plain = call()
+            monkeypatch.delenv("KERMAC_AMD_DIRECT_PANELS")
+            what = f"case {case}: {M} x {columns} x {K}, L = {L}, p = {p}, a against itself {same}, laplace {laplace}"
+            assert not torch.isnan(forced).any(), what
+            assert torch.equal(forced, plain), what
+    finally:
+        kermac.set_l2_mode(kermac.DEFAULT_L2_MODE)
